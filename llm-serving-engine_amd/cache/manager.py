@@ -1,0 +1,371 @@
+"""The cache manager: pages of keys and values with a block table per request,
+one pool per group of layers with the same need, and slots of fixed-size state.
+
+The reference keeps one tensor [L, 2, NB, P, Hkv, D] for all layers, one block
+table per sequence and a metadata row per sequence (`kv_cache.py:91-179`).  Here
+the layers that run are first sorted into groups by what their mixer needs
+(all keys, a window of keys, a fixed state, nothing); every paged group has its
+own pool, storage [cells, 2, NB, Hkv, P, D] and block tables, and a windowed
+group gives a page back as soon as no later query can read it.  A request's
+slot (the reference's metadata row) is its block-table row in every group and
+its index into every fixed-state tensor.
+"""
+
+from __future__ import annotations
+
+import math
+from collections import deque
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..config.serving import CacheConfig
+from ..engine.batch import CacheCell
+from ..parts.base import FixedState, PagedKeyValue
+from ..parts.model import ModelSpec
+from .pool import CacheFullError, PagePool
+
+
+@dataclass
+class PageGroup:
+    need: PagedKeyValue
+    cells: list[int]  # runs of the run order that own a cell in this group
+    pool: PagePool
+    storage: torch.Tensor | None  # [len(cells), 2, NB, Hkv, P, D]
+    tables: np.ndarray  # int32 [max_sequences, max_blocks]; -1 where no page is held
+    peak_pages: int = 0
+
+    @property
+    def bytes_per_page(self) -> int:
+        if self.storage is None:
+            return 0
+        return self.storage[:, :, 0].numel() * self.storage.element_size()
+
+
+@dataclass
+class SequenceRecord:
+    request_id: str
+    slot: int
+    length: int = 0
+    # per group: number of leading logical blocks already given back (window passed)
+    released: list[int] = field(default_factory=list)
+    last_access_tick: int = 0
+
+
+@dataclass(frozen=True)
+class Reservation:
+    """Where the next `count` tokens of a request go."""
+
+    request_id: str
+    slot: int
+    start: int
+    count: int
+    slots: tuple[np.ndarray, ...]  # per group: int32 [count], page * page_size + offset
+
+
+class CacheManager:
+    def __init__(
+        self,
+        spec: ModelSpec,
+        config: CacheConfig,
+        *,
+        max_sequence_length: int,
+        dtype: torch.dtype = torch.float32,
+        device: str | torch.device = "cpu",
+    ) -> None:
+        self.spec = spec
+        self.config = config
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.page_size = config.block_size
+        self.max_sequence_length = max_sequence_length
+        self.max_blocks_per_sequence = math.ceil(max_sequence_length / config.block_size)
+        self.sequences: dict[str, SequenceRecord] = {}
+        self._free_slots: deque[int] = deque(range(config.max_sequences))
+        self._tick = 0
+        self._high_water = {"pages": 0, "used_tokens": 0, "sequences": 0}
+
+        self.groups: list[PageGroup] = []
+        self._cell_of_run: list[tuple[str, int, int] | None] = []  # (kind, group or state index, index inside)
+        self.states: list[torch.Tensor] = []
+        self._state_needs: list[FixedState] = []
+        by_need: dict[PagedKeyValue, int] = {}
+        owners: dict[int, tuple[str, int, int]] = {}
+        for index, run in enumerate(spec.run_order):
+            if run.reads is not None:
+                self._cell_of_run.append(owners[run.reads])
+                continue
+            need = spec.cell_need(index)
+            if need is None:
+                entry = None
+            elif isinstance(need, PagedKeyValue):
+                if need not in by_need:
+                    by_need[need] = len(self.groups)
+                    self.groups.append(
+                        PageGroup(
+                            need,
+                            [],
+                            PagePool(config.num_blocks),
+                            None,
+                            np.full((config.max_sequences, self.max_blocks_per_sequence), -1, np.int32),
+                        )
+                    )
+                group = by_need[need]
+                self.groups[group].cells.append(index)
+                entry = ("pages", group, len(self.groups[group].cells) - 1)
+            elif isinstance(need, FixedState):
+                self._state_needs.append(need)
+                self.states.append(
+                    torch.zeros((config.max_sequences, *need.shape), dtype=torch.float32, device=self.device)
+                )
+                entry = ("state", len(self.states) - 1, 0)
+            else:
+                raise TypeError(f"run {index}: unknown cache need {need!r}")
+            owners[index] = entry
+            self._cell_of_run.append(entry)
+        for group in self.groups:
+            need = group.need
+            shape = (len(group.cells), 2, config.num_blocks, need.num_kv_heads, self.page_size, need.head_dim)
+            group.storage = torch.zeros(shape, dtype=dtype, device=self.device)
+
+    # ------------------------------------------------------------------ views
+
+    def cells(self) -> list[CacheCell | None]:
+        """One cell per entry of the run order, in order."""
+        views: list[CacheCell | None] = []
+        for index, entry in enumerate(self._cell_of_run):
+            writable = self.spec.run_order[index].reads is None
+            if entry is None:
+                views.append(None)
+            elif entry[0] == "pages":
+                group = self.groups[entry[1]]
+                views.append(
+                    CacheCell(
+                        need=group.need,
+                        writable=writable,
+                        group=entry[1],
+                        keys=group.storage[entry[2], 0],
+                        values=group.storage[entry[2], 1],
+                    )
+                )
+            else:
+                views.append(
+                    CacheCell(need=self._state_needs[entry[1]], writable=writable, state=self.states[entry[1]])
+                )
+        return views
+
+    # ------------------------------------------------------------------ requests
+
+    def create(self, request_id: str) -> int:
+        """Gives the request a slot: an empty block-table row in every group and
+        zeroed fixed state (reference `kv_cache.py:135-143`)."""
+        if request_id in self.sequences:
+            raise ValueError(f"sequence {request_id!r} already exists")
+        if not self._free_slots:
+            raise CacheFullError("paged cache has no free request slots")
+        slot = self._free_slots.popleft()
+        for group in self.groups:
+            group.tables[slot].fill(-1)
+        for state in self.states:
+            state[slot].zero_()
+        self.sequences[request_id] = SequenceRecord(request_id, slot, released=[0] * len(self.groups))
+        return slot
+
+    def _first_needed_block(self, group: PageGroup, start: int) -> int:
+        """Blocks below this index hold no key that a query at position >= start reads."""
+        if group.need.window is None:
+            return 0
+        return max(0, start - group.need.window + 1) // self.page_size
+
+    def pages_needed(self, request_id: str, count: int) -> list[tuple[int, int]]:
+        """Per group: (pages to allocate, pages given back first) for the next `count` tokens."""
+        record = self.sequences[request_id]
+        need = []
+        for index, group in enumerate(self.groups):
+            held_until = math.ceil(record.length / self.page_size)
+            wanted_until = math.ceil((record.length + count) / self.page_size)
+            first = self._first_needed_block(group, record.length)
+            giving_back = max(0, min(first, held_until) - record.released[index])
+            need.append((wanted_until - held_until, giving_back))
+        return need
+
+    def fits(self, plan: list[tuple[str, int]]) -> bool:
+        """Whether every (request, count) of `plan` can be reserved, in order."""
+        free = [group.pool.free_pages for group in self.groups]
+        for request_id, count in plan:
+            record = self.sequences[request_id]
+            if record.length + count > self.max_sequence_length:
+                return False
+            for index, (allocate, give_back) in enumerate(self.pages_needed(request_id, count)):
+                free[index] += give_back - allocate
+                if free[index] < 0:
+                    return False
+        return True
+
+    def pages_short(self, plan: list[tuple[str, int]]) -> int:
+        """How many pages are missing, summed over groups, to reserve all of `plan`."""
+        short = 0
+        for index, group in enumerate(self.groups):
+            balance = group.pool.free_pages
+            for request_id, count in plan:
+                allocate, give_back = self.pages_needed(request_id, count)[index]
+                balance += give_back - allocate
+            short += max(0, -balance)
+        return short
+
+    def reserve(self, request_id: str, count: int) -> Reservation:
+        """Takes the cache entries of the request's next `count` tokens
+        (reference `kv_cache.py:145-179`).  Pages that a window has passed are
+        given back first.  Raises `CacheFullError`, holding nothing new, if a
+        pool runs dry or the request would outgrow the longest sequence."""
+        if count <= 0:
+            raise ValueError("count must be positive")
+        record = self.sequences[request_id]
+        start = record.length
+        if start + count > self.max_sequence_length:
+            raise CacheFullError("sequence exceeds the longest sequence the cache was built for")
+        if not self.fits([(request_id, count)]):
+            raise CacheFullError("paged cache has no free pages")
+        page_size = self.page_size
+        positions = np.arange(start, start + count)
+        slots = []
+        for index, group in enumerate(self.groups):
+            table = group.tables[record.slot]
+            first = min(self._first_needed_block(group, start), math.ceil(start / page_size))
+            for block in range(record.released[index], first):
+                group.pool.free(int(table[block]), request_id)
+                table[block] = -1
+            record.released[index] = max(record.released[index], first)
+            for block in range(math.ceil(start / page_size), math.ceil((start + count) / page_size)):
+                table[block] = group.pool.allocate(request_id)
+            group.peak_pages = max(group.peak_pages, group.pool.used_pages)
+            pages = table[positions // page_size].astype(np.int64)
+            slots.append((pages * page_size + positions % page_size).astype(np.int32))
+        record.length = start + count
+        self._touch(record)
+        used = sum(group.pool.used_pages for group in self.groups)
+        if used >= self._high_water["pages"]:
+            self._high_water = {
+                "pages": used,
+                "used_tokens": sum(item.length for item in self.sequences.values()),
+                "sequences": len(self.sequences),
+            }
+        return Reservation(request_id, record.slot, start, count, tuple(slots))
+
+    def block_table(self, request_id: str, group: int = 0) -> list[int]:
+        record = self.sequences[request_id]
+        blocks = math.ceil(record.length / self.page_size)
+        return self.groups[group].tables[record.slot, :blocks].tolist()
+
+    def free(self, request_id: str) -> None:
+        """Gives back everything the request holds (reference `kv_cache.py:344-350`)."""
+        record = self.sequences.pop(request_id)
+        for group in self.groups:
+            table = group.tables[record.slot]
+            for page in table[table >= 0].tolist():
+                group.pool.free(page, request_id)
+            table.fill(-1)
+        self._free_slots.append(record.slot)
+
+    def evict(self, policy: str = "largest", exclude: set[str] | None = None) -> tuple[str, int]:
+        """Frees one request chosen by `policy` and returns (its id, tokens to
+        recompute) (reference `kv_cache.py:352-369`)."""
+        candidates = [
+            record for record in self.sequences.values() if not exclude or record.request_id not in exclude
+        ]
+        if not candidates:
+            raise CacheFullError("no evictable sequences")
+        if policy == "largest":
+            victim = max(candidates, key=lambda item: (item.length, -item.last_access_tick))
+        elif policy == "lru":
+            victim = min(candidates, key=lambda item: item.last_access_tick)
+        else:
+            raise ValueError(f"unknown eviction policy: {policy}")
+        recompute = victim.length
+        self.free(victim.request_id)
+        return victim.request_id, recompute
+
+    def _touch(self, record: SequenceRecord) -> None:
+        self._tick += 1
+        record.last_access_tick = self._tick
+
+    # ------------------------------------------------------------------ accounting
+
+    @property
+    def free_pages(self) -> int:
+        """Free pages of the fullest group."""
+        return min((group.pool.free_pages for group in self.groups), default=0)
+
+    @property
+    def used_pages(self) -> int:
+        return sum(group.pool.used_pages for group in self.groups)
+
+    @property
+    def capacity_tokens(self) -> int:
+        return self.config.num_blocks * self.page_size
+
+    def check_invariants(self) -> None:
+        """No page lost, held twice, or held by a request that is gone."""
+        for index, group in enumerate(self.groups):
+            held: dict[int, str] = {}
+            for record in self.sequences.values():
+                table = group.tables[record.slot]
+                blocks = math.ceil(record.length / self.page_size)
+                for block in range(self.max_blocks_per_sequence):
+                    page = int(table[block])
+                    live = record.released[index] <= block < blocks
+                    if live != (page >= 0):
+                        raise AssertionError(f"group {index}: {record.request_id} block {block} holds {page}")
+                    if page >= 0:
+                        if page in held:
+                            raise AssertionError(f"group {index}: page {page} held twice")
+                        held[page] = record.request_id
+            for page, owner in held.items():
+                if group.pool.owner_of(page) != owner:
+                    raise AssertionError(f"group {index}: page {page} owner mismatch")
+            if group.pool.used_pages != len(held):
+                raise AssertionError(f"group {index}: {group.pool.used_pages} pages out, {len(held)} in tables")
+            if group.pool.used_pages + group.pool.free_pages != group.pool.num_pages:
+                raise AssertionError(f"group {index}: pages lost")
+            live_slots = {record.slot for record in self.sequences.values()}
+            for slot in range(self.config.max_sequences):
+                if slot not in live_slots and (group.tables[slot] >= 0).any():
+                    raise AssertionError(f"group {index}: free slot {slot} still holds pages")
+        if len(self._free_slots) + len(self.sequences) != self.config.max_sequences:
+            raise AssertionError("request slots lost")
+
+    def stats(self, contiguous_max_length: int | None = None) -> dict[str, float]:
+        """The reference's accounting (`kv_cache.py:386-413`), summed over groups."""
+        used_tokens = sum(record.length for record in self.sequences.values())
+        used = self.used_pages
+        total = sum(group.pool.num_pages for group in self.groups)
+        held_tokens = 0
+        for index, group in enumerate(self.groups):
+            for record in self.sequences.values():
+                held_tokens += record.length - record.released[index] * self.page_size
+        allocated_slots = used * self.page_size
+        waste = allocated_slots - held_tokens
+        allocated_bytes = sum(group.pool.used_pages * group.bytes_per_page for group in self.groups)
+        peak_bytes = sum(group.peak_pages * group.bytes_per_page for group in self.groups)
+        result = {
+            "blocks_used": float(used),
+            "blocks_free": float(total - used),
+            "used_tokens": float(used_tokens),
+            "paged_waste_tokens": float(waste),
+            "paged_fragmentation_pct": 100.0 * waste / max(allocated_slots, 1),
+            "paged_allocated_gb": allocated_bytes / 1024**3,
+            "peak_blocks_used": float(self._high_water["pages"]),
+            "peak_paged_allocated_gb": peak_bytes / 1024**3,
+        }
+        if contiguous_max_length is not None:
+            bytes_per_token = sum(group.bytes_per_page for group in self.groups) / self.page_size
+            contiguous_slots = self._high_water["sequences"] * contiguous_max_length
+            contiguous_waste = max(contiguous_slots - self._high_water["used_tokens"], 0)
+            paged_slots = self._high_water["pages"] * self.page_size / max(len(self.groups), 1)
+            result.update(
+                contiguous_waste_tokens=float(contiguous_waste),
+                contiguous_waste_gb=contiguous_waste * bytes_per_token / 1024**3,
+                memory_reduction_pct=100.0 * (contiguous_slots - paged_slots) / max(contiguous_slots, 1),
+            )
+        return result

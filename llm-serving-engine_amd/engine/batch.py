@@ -1,0 +1,82 @@
+"""The facts about one step that every part may read: which tokens run, at
+which positions, for which request, and where their cache entries lie.
+
+One step is a flat list of T tokens.  Request b contributes the consecutive
+tokens [query_start[b], query_start[b+1]) at positions
+[context_length[b] - count, context_length[b]): a portion of a prompt, a single
+decoded token, anything between.  The reference passes the same facts per row
+(`engine.py:303-315`, `kv_cache.py:208-247`); here they are per request, so a
+kernel can treat a portion as a tile of queries rather than as unrelated rows.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any
+
+import torch
+
+
+@dataclass(frozen=True)
+class SequenceChunk:
+    """Host-side record of one request's share of the step."""
+
+    request_id: str
+    slot: int  # the request's state slot and block-table row
+    start: int  # position of its first token in this step
+    count: int  # tokens in this step
+
+    @property
+    def context_length(self) -> int:
+        return self.start + self.count
+
+
+@dataclass
+class GroupBatch:
+    """Per cache group: where this step's tokens are written, and each request's pages."""
+
+    page_size: int
+    block_tables: torch.Tensor  # int32 [B, width]; -1 where no page is held
+    slot_mapping: torch.Tensor  # int32 [T]: page * page_size + offset
+    width: int
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    chunks: list[SequenceChunk]
+    token_ids: torch.Tensor  # int32 [T]
+    positions: torch.Tensor  # int32 [T]
+    token_sequence: torch.Tensor  # int32 [T]: index b of the token's request in this step
+    query_start: torch.Tensor  # int32 [B + 1]
+    context_lengths: torch.Tensor  # int32 [B]: tokens cached after this step
+    state_slots: torch.Tensor  # int32 [B]
+    groups: list[GroupBatch]
+    logit_rows: torch.Tensor  # int32 [R]: token rows whose logits are wanted
+    num_logit_rows: int
+    max_query_length: int
+    max_context_length: int
+    # Kernel libraries may keep per-step work lists here (built once, used by every layer).
+    scratch: dict[str, Any] = field(default_factory=dict)
+
+    @property
+    def num_sequences(self) -> int:
+        return len(self.chunks)
+
+
+@dataclass
+class CacheCell:
+    """What one run of a layer sees of the cache.
+
+    For a paged need: `keys` and `values` are [pages, kv_heads, page_size,
+    head_dim] and `group` indexes `StepBatch.groups`.  For a fixed state:
+    `state` is [slots, *shape] float32, indexed by `StepBatch.state_slots`.
+    `writable` is False when the run reads a cell that another run owns.
+    """
+
+    need: Any
+    writable: bool = True
+    group: int = -1
+    keys: torch.Tensor | None = None
+    values: torch.Tensor | None = None
+    state: torch.Tensor | None = None

@@ -1,0 +1,60 @@
+"""The operations the parts call.  The product has one implementation, the HIP
+library in `hip.py`; the interface is spelled out so that tests can check parts,
+cache and step function with a stand-in of their own on a machine without a GPU.
+
+Conventions: the residual stream and every value added to it are float32 in
+every run dtype; activations between kernels are in the run dtype (bfloat16 or
+float32); products accumulate in float32; logits are float32.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Protocol
+
+import torch
+
+
+class Kernels(Protocol):
+    device: torch.device
+    dtype: torch.dtype
+
+    def to_device(self, tensor: torch.Tensor) -> torch.Tensor: ...
+
+    def embedding(self, table: torch.Tensor, token_ids: torch.Tensor) -> torch.Tensor:
+        """float32 rows [T, hidden] of `table` at `token_ids`."""
+
+    def add_rms_norm(
+        self, hidden: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float
+    ) -> torch.Tensor:
+        """`hidden += delta` in place (float32), then rows * rsqrt(mean(rows^2) + eps) * weight in the run dtype."""
+
+    def prepare_linear(self, weights: list[torch.Tensor], biases: list[torch.Tensor] | None) -> Any:
+        """Concatenates [N_i, K] weights (and biases) along N into whatever layout `linear` wants."""
+
+    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor) -> Any: ...
+
+    def linear(self, x: torch.Tensor, weights: Any, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """x [T, K] @ W^T + bias -> [T, N] in `out_dtype` (the run dtype if None)."""
+
+    def gated_linear(self, x: torch.Tensor, weights: Any) -> torch.Tensor:
+        """silu(x Wg^T) * (x Wu^T) -> [T, I] in the run dtype."""
+
+    def rotate_and_store(
+        self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any,
+        inverse_frequencies: torch.Tensor | None, pairing: str,
+    ) -> None:
+        """Rotary on the q and k heads of `qkv` in place; k and v into the cell's pages if it is writable."""
+
+    def paged_attention(
+        self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any, scale: float, window: int | None
+    ) -> torch.Tensor:
+        """Attention of the q heads of `qkv` over the cell's pages -> [T, heads * head_dim]."""
+
+    def gather_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
+        """float32 (hidden + delta)[rows]."""
+
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor: ...
+
+    def sample(
+        self, logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor, uniforms: torch.Tensor
+    ) -> torch.Tensor: ...

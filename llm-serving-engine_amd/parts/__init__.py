@@ -1,0 +1,20 @@
+from .base import (
+    BLOCKS,
+    FEED_FORWARDS,
+    MIXERS,
+    NORMS,
+    POSITIONS,
+    FixedState,
+    PagedKeyValue,
+    Part,
+    Registry,
+    TensorSpec,
+)
+from .norm import RMSNorm, RMSNormSpec
+from .position import HeadLayout, NoPositionSpec, PositionEncoding, Rotary, RotarySpec
+from .attention import Attention, AttentionSpec, Mixer
+from .feed_forward import FeedForward, GatedMLP, GatedMLPSpec
+from .block import Block, PreNormBlock, PreNormBlockSpec
+from .model import DecoderModel, LayerDefinition, LayerRun, ModelSpec
+
+__all__ = [name for name in dir() if not name.startswith("_")]

@@ -1,0 +1,90 @@
+"""The tests' own small configurations.  They differ in every size and option:
+head counts and group size, head size, widths that are no power of two, number
+of layers, vocabulary, eps, theta, rotary pairing, tied or untied head, window,
+page size, how norm weights are drawn and stored."""
+
+from __future__ import annotations
+
+from pathlib import Path
+
+import torch
+
+from llmserve_amd import Qwen2Config
+from llmserve_amd.weights import write_model_folder
+
+# A: 2 layers, G = 2, head size 16, tied, no window, reference pairing, page 16.
+TINY_A = Qwen2Config(
+    vocab_size=256,
+    hidden_size=64,
+    intermediate_size=128,
+    num_layers=2,
+    num_attention_heads=4,
+    num_key_value_heads=2,
+    head_dim=16,
+    max_position_embeddings=512,
+    rope_theta=10000.0,
+    rms_norm_eps=1e-6,
+    attention_bias=True,
+    tie_word_embeddings=True,
+    rope_pairing="adjacent",
+)
+PAGE_A = 16
+
+# B: 3 layers, one kv head (G = 6), head size 32, untied, widths 192/320/384,
+# layers 1 and 2 see a window of 24 keys, checkpoint pairing, page 8.
+TINY_B = Qwen2Config(
+    vocab_size=384,
+    hidden_size=192,
+    intermediate_size=320,
+    num_layers=3,
+    num_attention_heads=6,
+    num_key_value_heads=1,
+    head_dim=32,
+    max_position_embeddings=1024,
+    rope_theta=1e6,
+    rms_norm_eps=1e-5,
+    attention_bias=True,
+    tie_word_embeddings=False,
+    rope_pairing="half",
+    use_sliding_window=True,
+    sliding_window=24,
+    max_window_layers=1,
+)
+PAGE_B = 8
+
+# C: hidden size differs from heads * head_dim, 5 heads over 5 kv heads (G = 1),
+# head size 48, no bias; used where a third shape helps.
+TINY_C = Qwen2Config(
+    vocab_size=131,
+    hidden_size=80,
+    intermediate_size=112,
+    num_layers=2,
+    num_attention_heads=5,
+    num_key_value_heads=5,
+    head_dim=48,
+    max_position_embeddings=256,
+    rope_theta=500.0,
+    rms_norm_eps=1e-4,
+    attention_bias=False,
+    tie_word_embeddings=False,
+    rope_pairing="half",
+)
+PAGE_C = 32
+
+
+def write_tiny_folders(root: Path) -> dict[str, Path]:
+    return {
+        # norm weights 1.0 as the reference initialises them, biases drawn
+        "A": write_model_folder(root / "A", TINY_A, seed=11, norm_std=0.0),
+        # norm weights N(1, 0.1), stored in 32-bit so that they stay so in a bfloat16 run
+        "B": write_model_folder(root / "B", TINY_B, seed=23, norm_std=0.1, wide_roles=("norm",)),
+        "C": write_model_folder(root / "C", TINY_C, seed=5, norm_std=0.1, std=0.05),
+    }
+
+
+CONFIGS = {"A": (TINY_A, PAGE_A), "B": (TINY_B, PAGE_B), "C": (TINY_C, PAGE_C)}
+
+
+def random_tokens(count: int, vocab: int, seed: int) -> list[int]:
+    generator = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (count,), generator=generator).tolist()
