@@ -1,0 +1,72 @@
+// Shared by every kernel file: element types, wave and block reductions, launch checks.
+// Everything here is for gfx950 (CDNA4): 64-wide waves, MFMA, 160 KB LDS per CU.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16_t;
+
+#define WAVE 64
+
+// Every entry point returns 0 or a HIP error code; the Python side raises on non-zero.
+#define LAUNCH_STATUS() ((int)hipGetLastError())
+
+// Argument errors that the host can detect before a launch.
+#define ERR_BAD_ARGUMENT 1001
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return (float)v; }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return (bf16_t)v; }
+
+// Loads element i of a tensor whose element type is chosen at run time (0: bf16, 1: float).
+__device__ __forceinline__ float load_as_float(const void* base, int is_float, size_t i) {
+  return is_float ? ((const float*)base)[i] : (float)((const bf16_t*)base)[i];
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int offset = WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int offset = WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.  The order of the
+// additions depends only on the block size, so equal inputs give equal bits in every launch.
+__device__ __forceinline__ float block_sum(float v, float* shared /* >= 17 floats */) {
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, waves = (blockDim.x + WAVE - 1) / WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) shared[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float total = 0.f;
+    for (int i = 0; i < waves; ++i) total += shared[i];
+    shared[16] = total;
+  }
+  __syncthreads();
+  return shared[16];
+}
+
+__device__ __forceinline__ float block_max(float v, float* shared /* >= 17 floats */) {
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, waves = (blockDim.x + WAVE - 1) / WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) shared[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float best = shared[0];
+    for (int i = 1; i < waves; ++i) best = fmaxf(best, shared[i]);
+    shared[16] = best;
+  }
+  __syncthreads();
+  return shared[16];
+}

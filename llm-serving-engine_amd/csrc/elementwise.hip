@@ -1,0 +1,166 @@
+// Embedding gather, residual add + RMSNorm, rotary position encoding with the cache
+// write, SiLU * up, and row gather.  All arithmetic is float32; inputs and outputs are
+// bfloat16 or float32 as the template says.
+#include "common.h"
+
+// ---------------------------------------------------------------------------- embedding
+// out[t, :] = float(table[ids[t], :])        (reference model.py:293)
+template <typename T>
+__global__ void embedding_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                 float* __restrict__ out, int hidden) {
+  const size_t row = (size_t)ids[blockIdx.x];
+  const T* src = table + row * hidden;
+  float* dst = out + (size_t)blockIdx.x * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+}
+
+extern "C" int llmserve_embedding(const void* table, int table_is_float, const int* ids, float* out,
+                                  int tokens, int hidden, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (table_is_float)
+    hipLaunchKernelGGL(embedding_kernel<float>, dim3(tokens), dim3(256), 0, stream, (const float*)table, ids, out, hidden);
+  else
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)table, ids, out, hidden);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- add + RMSNorm
+// hidden[t] += delta[t] (if delta); out[t] = hidden[t] * rsqrt(mean(hidden[t]^2) + eps) * weight
+// (reference model.py:20-23, :200-201).  One block per row; the sum of squares is added in
+// an order that depends only on the row length, so a row's result is the same in any batch.
+template <typename TO>
+__global__ void add_rms_norm_kernel(float* __restrict__ hidden, const float* __restrict__ delta,
+                                    const void* __restrict__ weight, int weight_is_float,
+                                    TO* __restrict__ out, int width, float eps) {
+  __shared__ float shared[17];
+  float* row = hidden + (size_t)blockIdx.x * width;
+  const float* add = delta ? delta + (size_t)blockIdx.x * width : nullptr;
+  float squares = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = row[i];
+    if (add) {
+      v += add[i];
+      row[i] = v;
+    }
+    squares += v * v;
+  }
+  const float total = block_sum(squares, shared);
+  const float scale = rsqrtf(total / (float)width + eps);
+  TO* dst = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    dst[i] = from_float<TO>(row[i] * scale * load_as_float(weight, weight_is_float, i));
+}
+
+extern "C" int llmserve_add_rms_norm(float* hidden, const float* delta, const void* weight, int weight_is_float,
+                                     void* out, int out_is_float, int rows, int width, float eps,
+                                     hipStream_t stream) {
+  if (rows <= 0) return 0;
+  const int threads = width >= 2048 ? 512 : 256;
+  if (out_is_float)
+    hipLaunchKernelGGL(add_rms_norm_kernel<float>, dim3(rows), dim3(threads), 0, stream, hidden, delta, weight,
+                       weight_is_float, (float*)out, width, eps);
+  else
+    hipLaunchKernelGGL(add_rms_norm_kernel<bf16_t>, dim3(rows), dim3(threads), 0, stream, hidden, delta, weight,
+                       weight_is_float, (bf16_t*)out, width, eps);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- rotary + cache write
+// A token's row of qkv is [q heads | k heads | v heads], each head `dim` wide.  q and k heads
+// are rotated in place by the token's position (reference model.py:35-43): the pair (a, b)
+// becomes (a cos - b sin, b cos + a sin) with angle = position * inverse[j], all in float32.
+// pairing 0: none, 1: adjacent pairs (2j, 2j+1), 2: half pairs (j, j + dim/2).
+// k (after rotation) and v are then written to the pages: slot = page * page_size + offset,
+// pages laid out [page, kv_head, offset, dim] (reference kv_cache.py:249-266 writes
+// [page, offset, kv_head, dim]).  slots may be null (nothing is stored); a negative slot
+// skips the token.
+template <typename T>
+__global__ void rotate_and_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                        const float* __restrict__ inverse, int pairing, int heads, int kv_heads,
+                                        int dim, T* __restrict__ keys, T* __restrict__ values,
+                                        const int* __restrict__ slots, int page_size) {
+  const int token = blockIdx.x;
+  const int half = dim / 2;
+  T* row = qkv + (size_t)token * (heads + 2 * kv_heads) * dim;
+  const float position = (float)positions[token];
+  if (pairing != 0) {
+    const int pairs = (heads + kv_heads) * half;
+    for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+      const int head = i / half, j = i % half;
+      float sine, cosine;
+      sincosf(position * inverse[j], &sine, &cosine);
+      T* h = row + head * dim;
+      const int ia = pairing == 1 ? 2 * j : j;
+      const int ib = pairing == 1 ? 2 * j + 1 : j + half;
+      const float a = to_float(h[ia]), b = to_float(h[ib]);
+      h[ia] = from_float<T>(a * cosine - b * sine);
+      h[ib] = from_float<T>(b * cosine + a * sine);
+    }
+  }
+  if (slots == nullptr) return;
+  const int slot = slots[token];
+  if (slot < 0) return;
+  __syncthreads();  // the rotated k is read back below by other threads
+  const int page = slot / page_size, offset = slot % page_size;
+  const T* k_row = row + heads * dim;
+  const T* v_row = k_row + kv_heads * dim;
+  for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
+    const int head = i / dim, d = i % dim;
+    const size_t at = (((size_t)page * kv_heads + head) * page_size + offset) * dim + d;
+    keys[at] = k_row[i];
+    values[at] = v_row[i];
+  }
+}
+
+extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const int* positions, const float* inverse,
+                                         int pairing, int tokens, int heads, int kv_heads, int dim, void* keys,
+                                         void* values, const int* slots, int page_size, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (dim % 2 || (pairing != 0 && inverse == nullptr) || pairing < 0 || pairing > 2) return ERR_BAD_ARGUMENT;
+  if (is_float)
+    hipLaunchKernelGGL(rotate_and_store_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float*)qkv, positions,
+                       inverse, pairing, heads, kv_heads, dim, (float*)keys, (float*)values, slots, page_size);
+  else
+    hipLaunchKernelGGL(rotate_and_store_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t*)qkv, positions,
+                       inverse, pairing, heads, kv_heads, dim, (bf16_t*)keys, (bf16_t*)values, slots, page_size);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- SiLU(gate) * up
+// in: [rows, 2 * width] float32, gate in the first half of each row; out: [rows, width].
+// silu(z) = z * sigmoid(z)  (reference model.py:188).
+template <typename TO>
+__global__ void silu_mul_kernel(const float* __restrict__ in, TO* __restrict__ out, int width) {
+  const float* row = in + (size_t)blockIdx.x * 2 * width;
+  TO* dst = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float g = row[i], u = row[width + i];
+    dst[i] = from_float<TO>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int llmserve_silu_mul(const float* in, void* out, int out_is_float, int rows, int width,
+                                 hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (out_is_float)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, dim3(rows), dim3(256), 0, stream, in, (float*)out, width);
+  else
+    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, in, (bf16_t*)out, width);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- gather rows
+// out[r] = hidden[rows[r]] (+ delta[rows[r]])
+__global__ void gather_rows_kernel(const float* __restrict__ hidden, const float* __restrict__ delta,
+                                   const int* __restrict__ rows, float* __restrict__ out, int width) {
+  const size_t src = (size_t)rows[blockIdx.x] * width;
+  float* dst = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = hidden[src + i] + (delta ? delta[src + i] : 0.f);
+}
+
+extern "C" int llmserve_gather_rows(const float* hidden, const float* delta, const int* rows, float* out, int count,
+                                    int width, hipStream_t stream) {
+  if (count <= 0) return 0;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(count), dim3(256), 0, stream, hidden, delta, rows, out, width);
+  return LAUNCH_STATUS();
+}

@@ -1,0 +1,229 @@
+"""The HIP kernel library: every operation of the model on gfx950.
+
+There is no other implementation in the product: without a GPU, or without a
+compiler to build a missing library, construction fails with an error.
+Kernels are called through their C entry points with raw device pointers on
+torch's current stream, so a step can be captured into a HIP graph.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+
+from .build import load_module
+
+_PAIRINGS = {"none": 0, "adjacent": 1, "half": 2}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _is_float(tensor: torch.Tensor) -> int:
+    if tensor.dtype == torch.float32:
+        return 1
+    if tensor.dtype == torch.bfloat16:
+        return 0
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, not {tensor.dtype}")
+
+
+def _pointer(tensor: torch.Tensor | None) -> ctypes.c_void_p:
+    if tensor is None:
+        return ctypes.c_void_p(0)
+    if not tensor.is_contiguous():
+        raise KernelError("kernels take contiguous tensors")
+    return ctypes.c_void_p(tensor.data_ptr())
+
+
+def _check(status: int, what: str) -> None:
+    if status == 1001:
+        raise KernelError(f"{what}: the kernel refuses these sizes or arguments")
+    if status != 0:
+        raise KernelError(f"{what}: HIP error {status}")
+
+
+@dataclass
+class LinearWeights:
+    """A product's right-hand side: weight [N, K] and bias [N] or None, as loaded."""
+
+    weight: torch.Tensor
+    bias: torch.Tensor | None
+
+    @property
+    def out_features(self) -> int:
+        return self.weight.shape[0]
+
+    @property
+    def in_features(self) -> int:
+        return self.weight.shape[1]
+
+
+@dataclass
+class GatedLinearWeights:
+    """Gate and up weights as one [2 I, K] right-hand side: gate rows first."""
+
+    both: LinearWeights
+    width: int
+
+
+class HipKernels:
+    def __init__(self, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0") -> None:
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise KernelError(f"run dtype must be bfloat16 or float32, not {dtype}")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the engine runs on an MI355X only and has no CPU path")
+        self.dtype = dtype
+        self.device = torch.device(device)
+        name = torch.cuda.get_device_properties(self.device).gcnArchName
+        if not name.startswith("gfx950"):
+            raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
+        self._elementwise = load_module("elementwise")
+        self._gemm_generic = load_module("gemm_generic")
+        self._attention_generic = load_module("attention_generic")
+        self._sampling = None
+
+    # ------------------------------------------------------------------ helpers
+
+    @property
+    def _stream(self) -> ctypes.c_void_p:
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def to_device(self, tensor: torch.Tensor) -> torch.Tensor:
+        return tensor.to(self.device).contiguous()
+
+    def _empty(self, shape, dtype) -> torch.Tensor:
+        return torch.empty(shape, dtype=dtype, device=self.device)
+
+    # ------------------------------------------------------------------ elementwise
+
+    def embedding(self, table: torch.Tensor, token_ids: torch.Tensor) -> torch.Tensor:
+        tokens, hidden = token_ids.shape[0], table.shape[1]
+        out = self._empty((tokens, hidden), torch.float32)
+        status = self._elementwise.llmserve_embedding(
+            _pointer(table), _is_float(table), _pointer(token_ids), _pointer(out), tokens, hidden, self._stream
+        )
+        _check(status, "embedding")
+        return out
+
+    def add_rms_norm(self, hidden, delta, weight, eps: float) -> torch.Tensor:
+        rows, width = hidden.shape
+        if hidden.dtype != torch.float32 or (delta is not None and delta.dtype != torch.float32):
+            raise KernelError("add_rms_norm: the residual stream and what is added to it are float32")
+        out = self._empty((rows, width), self.dtype)
+        status = self._elementwise.llmserve_add_rms_norm(
+            _pointer(hidden), _pointer(delta), _pointer(weight), _is_float(weight), _pointer(out), _is_float(out),
+            rows, width, ctypes.c_float(eps), self._stream,
+        )
+        _check(status, "add_rms_norm")
+        return out
+
+    def rotate_and_store(self, qkv, layout, batch, cell, inverse_frequencies, pairing: str) -> None:
+        tokens = qkv.shape[0]
+        if qkv.shape[1] != layout.width:
+            raise KernelError("rotate_and_store: qkv does not have the layout's width")
+        store = cell is not None and cell.writable
+        group = batch.groups[cell.group] if store else None
+        if store and (cell.keys.dtype != qkv.dtype or cell.keys.shape[1:] != (layout.num_kv_heads, group.page_size, layout.head_dim)):
+            raise KernelError("rotate_and_store: the cell's pages do not fit the layout")
+        status = self._elementwise.llmserve_rotate_and_store(
+            _pointer(qkv), _is_float(qkv), _pointer(batch.positions), _pointer(inverse_frequencies),
+            _PAIRINGS[pairing], tokens, layout.num_heads, layout.num_kv_heads, layout.head_dim,
+            _pointer(cell.keys if store else None), _pointer(cell.values if store else None),
+            _pointer(group.slot_mapping if store else None), group.page_size if store else 1, self._stream,
+        )
+        _check(status, "rotate_and_store")
+
+    def gather_rows(self, hidden, delta, rows) -> torch.Tensor:
+        count, width = rows.shape[0], hidden.shape[1]
+        out = self._empty((count, width), torch.float32)
+        status = self._elementwise.llmserve_gather_rows(
+            _pointer(hidden), _pointer(delta), _pointer(rows), _pointer(out), count, width, self._stream
+        )
+        _check(status, "gather_rows")
+        return out
+
+    # ------------------------------------------------------------------ products
+
+    def prepare_linear(self, weights: list[torch.Tensor], biases: list[torch.Tensor] | None) -> LinearWeights:
+        kinds = {w.dtype for w in weights}
+        if len(kinds) > 1:
+            weights = [w.float() for w in weights]
+        weight = torch.cat(list(weights), dim=0).contiguous() if len(weights) > 1 else weights[0].contiguous()
+        bias = None
+        if biases:
+            if len({b.dtype for b in biases}) > 1:
+                biases = [b.float() for b in biases]
+            bias = torch.cat(list(biases), dim=0).contiguous() if len(biases) > 1 else biases[0].contiguous()
+        return LinearWeights(weight, bias)
+
+    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor) -> GatedLinearWeights:
+        return GatedLinearWeights(self.prepare_linear([gate, up], None), gate.shape[0])
+
+    def linear(self, x: torch.Tensor, weights: LinearWeights, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        rows, inner = x.shape
+        if inner != weights.in_features:
+            raise KernelError(f"linear: x has {inner} columns, the weight {weights.in_features}")
+        out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
+        bias = weights.bias
+        status = self._gemm_generic.llmserve_gemm_generic(
+            _pointer(x), _is_float(x), _pointer(weights.weight), _is_float(weights.weight), _pointer(bias),
+            _is_float(bias) if bias is not None else 0, _pointer(out), _is_float(out), rows,
+            weights.out_features, inner, self._stream,
+        )
+        _check(status, "linear")
+        return out
+
+    def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
+        both = self.linear(x, weights.both, out_dtype=torch.float32)
+        out = self._empty((x.shape[0], weights.width), self.dtype)
+        status = self._elementwise.llmserve_silu_mul(
+            _pointer(both), _pointer(out), _is_float(out), x.shape[0], weights.width, self._stream
+        )
+        _check(status, "silu_mul")
+        return out
+
+    # ------------------------------------------------------------------ attention
+
+    def paged_attention(self, qkv, layout, batch, cell, scale: float, window: int | None) -> torch.Tensor:
+        tokens = qkv.shape[0]
+        group = batch.groups[cell.group]
+        if cell.keys.dtype != qkv.dtype:
+            raise KernelError("paged_attention: queries and pages differ in type")
+        out = self._empty((tokens, layout.num_heads * layout.head_dim), qkv.dtype)
+        status = self._attention_generic.llmserve_attention_generic(
+            _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
+            _pointer(group.block_tables), group.width, _pointer(batch.token_sequence), _pointer(batch.positions),
+            tokens, layout.num_heads, layout.num_kv_heads, layout.head_dim, group.page_size,
+            ctypes.c_float(scale), int(window or 0), self._stream,
+        )
+        _check(status, "paged_attention")
+        return out
+
+    # ------------------------------------------------------------------ sampling
+
+    def _sampling_library(self):
+        if self._sampling is None:
+            self._sampling = load_module("sampling")
+        return self._sampling
+
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor:
+        rows, vocab = logits.shape
+        out = self._empty((rows,), torch.int32)
+        status = self._sampling_library().llmserve_argmax(_pointer(logits), _pointer(out), rows, vocab, self._stream)
+        _check(status, "argmax")
+        return out
+
+    def sample(self, logits, temperatures, top_ps, uniforms) -> torch.Tensor:
+        rows, vocab = logits.shape
+        out = self._empty((rows,), torch.int32)
+        scratch = self._empty((rows, vocab), torch.float32)
+        status = self._sampling_library().llmserve_sample(
+            _pointer(logits), _pointer(temperatures), _pointer(top_ps), _pointer(uniforms), _pointer(scratch),
+            _pointer(out), rows, vocab, self._stream,
+        )
+        _check(status, "sample")
+        return out
