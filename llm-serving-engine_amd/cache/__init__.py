@@ -1,4 +1,5 @@
+from .cell import CacheCell
 from .manager import CacheManager, PageGroup, Reservation, SequenceRecord
 from .pool import CacheFullError, PagePool
 
-__all__ = ["CacheFullError", "CacheManager", "PageGroup", "PagePool", "Reservation", "SequenceRecord"]
+__all__ = ["CacheCell", "CacheFullError", "CacheManager", "PageGroup", "PagePool", "Reservation", "SequenceRecord"]

@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from ..config.serving import CacheConfig
-from ..engine.batch import CacheCell
+from .cell import CacheCell
 from ..parts.base import FixedState, PagedKeyValue
 from ..parts.model import ModelSpec
 from .pool import CacheFullError, PagePool

@@ -175,7 +175,7 @@ class Qwen2Config(ArchitectureConfig):
         if activation not in (None, "silu"):
             raise ConfigError(f"Qwen2 config: hidden_act {activation!r} is not supported")
         use_window = reader.boolean("use_sliding_window", default=False)
-        layers = reader.integer("num_layers", "num_hidden_layers")
+        layers = reader.integer("num_hidden_layers", "num_layers")
         return cls(
             vocab_size=reader.integer("vocab_size"),
             hidden_size=hidden,

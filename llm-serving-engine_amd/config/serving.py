@@ -22,4 +22,4 @@ class SchedulerConfig:
     max_batch_size: int = 16
     max_tokens_per_step: int = 2_048
     policy: str = "fcfs"  # fcfs | sjf | priority
-    preemption: str = "largest"  # the request holding most tokens goes first
+    preemption: str = "largest"  # who gives way when pages run out: largest | latest (never the oldest)
