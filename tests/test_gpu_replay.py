@@ -1,0 +1,101 @@
+"""Replays the same requests through bin/trace_run whole, with the last 32 tokens one by
+one, in portions of changing size, and mixed with other requests in a pool so small that
+pages are used again; in 32-bit and in bfloat16; against the plain implementation."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from tests.gpu_helpers import TraceBuilder, replay
+from tests.plain import qwen2_plain as plain
+from tests.tiny import CONFIGS, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+# float32: rounding only.  bfloat16: activations are rounded to 8 bits of mantissa between
+# kernels; logits of these models are of order 1, and the same bound holds for every way of cutting.
+TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
+LENGTHS = {"A": [1, 5, 17, 33, 70, 100], "B": [2, 9, 23, 40, 64, 100], "C": [3, 48, 65]}
+
+
+def build_trace(prompts: dict[str, list[int]], page: int):
+    trace = TraceBuilder()
+    # 1. each request alone and whole
+    for name, tokens in prompts.items():
+        trace.step([(f"whole-{name}", tokens)], end=[f"whole-{name}"])
+    # 2. most of it in one step, the last 32 tokens one by one
+    for name, tokens in prompts.items():
+        if len(tokens) <= 33:
+            continue
+        head = len(tokens) - 32
+        trace.step([(f"tail-{name}", tokens[:head])], want="last")
+        for index in range(head, len(tokens)):
+            trace.step([(f"tail-{name}", tokens[index : index + 1])], end=[f"tail-{name}"] if index == len(tokens) - 1 else [])
+    # 3. portions of changing size, down to two tokens (and one at the end where it remains)
+    sizes = [7, 2, 16, 3, 2, 31, 5, 2, 64]
+    for name, tokens in prompts.items():
+        at, turn = 0, 0
+        while at < len(tokens):
+            count = min(sizes[turn % len(sizes)], len(tokens) - at)
+            last = at + count == len(tokens)
+            trace.step([(f"cut-{name}", tokens[at : at + count])], end=[f"cut-{name}"] if last else [])
+            at, turn = at + count, turn + 1
+    # 4. mixed: up to four live requests, portions of some beside decoded tokens of others
+    names = list(prompts)
+    rng = torch.Generator().manual_seed(9)
+    done = {name: 0 for name in names}
+    waiting, live = list(names) + [], []
+    budget = 4 * 64  # tokens the pool holds; each live request counts rounded up to 64
+    while waiting or live:
+        while waiting and len(live) < 4 and sum(-(-len(prompts[n]) // 64) * 64 for n in live + [waiting[0]]) <= budget:
+            live.append(waiting.pop(0))
+        entries, ended = [], []
+        for name in live:
+            left = len(prompts[name]) - done[name]
+            count = 1 if done[name] >= len(prompts[name]) // 2 else min(left, int(torch.randint(2, 14, (1,), generator=rng)))
+            entries.append((f"mix-{name}", prompts[name][done[name] : done[name] + count]))
+            done[name] += count
+            if done[name] == len(prompts[name]):
+                ended.append(name)
+        trace.step(entries, end=[f"mix-{name}" for name in ended])
+        for name in ended:
+            live.remove(name)
+    return trace
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_replay_matches_plain_under_every_cut(model_folders, tmp_path, name, dtype):
+    config, page = CONFIGS[name]
+    folder = model_folders[name]
+    plain_config, weights = plain.PlainConfig.from_folder(folder), plain.read_weights(folder)
+    prompts = {f"p{n}": random_tokens(n, config.vocab_size, seed=100 + n) for n in LENGTHS[name]}
+    expected = {key: plain.forward(weights, plain_config, tokens) for key, tokens in prompts.items()}
+    trace = build_trace(prompts, page)
+    results = replay(folder, dtype, trace.steps, tmp_path / "out", max_tokens=4 * 64, block_size=page,
+                     vocab=config.vocab_size)
+    rows = trace.collect(results)
+    checked = 0
+    for (request, position), logits in rows.items():
+        mode, key = request.split("-", 1)
+        torch.testing.assert_close(
+            logits.double(), expected[key][position], **TOLERANCE[dtype],
+            msg=lambda m: f"{mode} {key} position {position}: {m}",
+        )
+        checked += 1
+    whole = sum(len(t) for t in prompts.values())
+    assert checked >= 3 * whole  # whole, cut and mixed give every position; tails add theirs
+
+
+def test_float32_cuts_agree_with_each_other_to_rounding(model_folders, tmp_path):
+    """How the tokens are cut must not matter beyond rounding: compare the cuts with each other,
+    tighter than with the plain implementation."""
+    config, page = CONFIGS["B"]
+    prompts = {"p90": random_tokens(90, config.vocab_size, seed=77)}
+    trace = build_trace(prompts, page)
+    rows = trace.collect(replay(model_folders["B"], "float32", trace.steps, tmp_path / "out", 256, page, config.vocab_size))
+    for position in range(90):
+        whole = rows[("whole-p90", position)]
+        for mode in ("cut", "mix"):
+            torch.testing.assert_close(rows[(f"{mode}-p90", position)], whole, atol=3e-6, rtol=1e-5)
