@@ -1,0 +1,299 @@
+"""Each kernel alone against a plain float32 reference of the same operation, at sizes
+other than the tiny models': widths and vocabularies that are no power of two, head sizes
+in steps of 16, odd numbers of heads and groups, pages of several sizes, shuffled pages."""
+
+from __future__ import annotations
+
+import math
+import types
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+TOLERANCE = {torch.float32: dict(atol=2e-5, rtol=2e-5), torch.bfloat16: dict(atol=2e-2, rtol=2e-2)}
+
+
+@pytest.fixture(scope="module")
+def kernels():
+    from llmserve_amd.kernels import HipKernels
+
+    return {dtype: HipKernels(dtype) for dtype in DTYPES}
+
+
+def on_gpu(tensor, dtype=None):
+    return tensor.to("cuda", dtype) if dtype else tensor.to("cuda")
+
+
+def rounded(tensor, dtype):
+    """What the kernel sees: the reference's inputs rounded to the run dtype."""
+    return tensor.to(dtype).double()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(kernels, dtype):
+    table = torch.randn(301, 72)
+    ids = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32)
+    out = kernels[dtype].embedding(on_gpu(table, dtype), on_gpu(ids))
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out.cpu().double(), rounded(table, dtype)[ids.long()], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width,eps", [(72, 1e-6), (1000, 1e-2), (4099, 1e-5)])
+def test_add_rms_norm(kernels, dtype, width, eps):
+    hidden, delta = torch.randn(7, width), 0.3 * torch.randn(7, width)
+    weight = 1 + 0.2 * torch.randn(width)
+    for weight_dtype in (dtype, torch.float32):
+        device_hidden = on_gpu(hidden.clone())
+        out = kernels[dtype].add_rms_norm(device_hidden, on_gpu(delta), on_gpu(weight, weight_dtype), eps)
+        summed = hidden.double() + delta.double()
+        torch.testing.assert_close(device_hidden.cpu().double(), summed, atol=1e-6, rtol=1e-6)
+        expected = plain.rms_norm(summed, rounded(weight, weight_dtype), eps)
+        assert out.dtype == dtype
+        torch.testing.assert_close(out.cpu().double(), expected, **TOLERANCE[dtype])
+    alone = kernels[dtype].add_rms_norm(on_gpu(hidden.clone()), None, on_gpu(weight, dtype), eps)
+    torch.testing.assert_close(alone.cpu().double(), plain.rms_norm(hidden.double(), rounded(weight, dtype), eps), **TOLERANCE[dtype])
+    small = 1e-4 * hidden  # eps decides here
+    tiny = kernels[dtype].add_rms_norm(on_gpu(small.clone()), None, on_gpu(torch.ones(width), dtype), eps)
+    torch.testing.assert_close(tiny.cpu().double(), plain.rms_norm(small.double(), torch.ones(width).double(), eps), **TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,inner,outer", [(1, 72, 50), (5, 200, 333), (70, 129, 65), (130, 64, 1000)])
+def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
+    k = kernels[dtype]
+    x, w, b = torch.randn(rows, inner), 0.1 * torch.randn(outer, inner), torch.randn(outer)
+    expected = rounded(x, dtype) @ rounded(w, dtype).T + rounded(b, dtype)
+    parts = [w[: outer // 3], w[outer // 3 :]], [b[: outer // 3], b[outer // 3 :]]
+    handle = k.prepare_linear([on_gpu(p, dtype) for p in parts[0]], [on_gpu(p, dtype) for p in parts[1]])
+    for out_dtype in (None, torch.float32):
+        out = k.linear(on_gpu(x, dtype), handle, out_dtype=out_dtype)
+        assert out.dtype == (out_dtype or dtype)
+        tolerance = TOLERANCE[dtype] if out_dtype is None else dict(atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(out.cpu().double(), expected, **tolerance)
+    no_bias = k.linear(on_gpu(x, dtype), k.prepare_linear([on_gpu(w, dtype)], None), out_dtype=torch.float32)
+    torch.testing.assert_close(no_bias.cpu().double(), expected - rounded(b, dtype), atol=1e-4, rtol=1e-4)
+    # a weight kept in 32-bit under a bfloat16 run
+    wide = k.linear(on_gpu(x, dtype), k.prepare_linear([on_gpu(w)], None), out_dtype=torch.float32)
+    torch.testing.assert_close(wide.cpu().double(), rounded(x, dtype) @ w.double().T, atol=1e-4, rtol=1e-4)
+    up = 0.1 * torch.randn(outer, inner)
+    gated = k.gated_linear(on_gpu(x, dtype), k.prepare_gated_linear(on_gpu(w, dtype), on_gpu(up, dtype)))
+    want = F.silu(rounded(x, dtype) @ rounded(w, dtype).T) * (rounded(x, dtype) @ rounded(up, dtype).T)
+    torch.testing.assert_close(gated.cpu().double(), want, **TOLERANCE[dtype])
+
+
+def paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=0, spare_pages=3):
+    """Requests with `lengths[i]` cached tokens of which the last `counts[i]` are this step's.
+    Returns the step's batch, the cell with garbage in every unused slot, and per-request q, k, v."""
+    from llmserve_amd.cache import CacheCell
+    from llmserve_amd.engine.batch import GroupBatch, SequenceChunk, StepBatch
+    from llmserve_amd.parts import HeadLayout, PagedKeyValue
+
+    generator = torch.Generator().manual_seed(shuffle_seed)
+    blocks = [math.ceil(n / page) for n in lengths]
+    pages = sum(blocks) + spare_pages
+    order = torch.randperm(pages, generator=generator).tolist()
+    width = max(blocks)
+    tables = torch.full((len(lengths), width), -1, dtype=torch.int32)
+    keys = torch.full((pages, kv_heads, page, dim), float("nan"))
+    values = torch.full((pages, kv_heads, page, dim), float("nan"))
+    per_request, slot_mapping, positions, token_sequence, chunks = [], [], [], [], []
+    for index, (length, count) in enumerate(zip(lengths, counts)):
+        mine = [order.pop() for _ in range(blocks[index])]
+        tables[index, : len(mine)] = torch.tensor(mine, dtype=torch.int32)
+        q = torch.randn(length, heads, dim, generator=generator)
+        k = torch.randn(length, kv_heads, dim, generator=generator)
+        v = torch.randn(length, kv_heads, dim, generator=generator)
+        per_request.append((q, k, v))
+        for position in range(length):
+            keys[mine[position // page], :, position % page] = k[position]
+            values[mine[position // page], :, position % page] = v[position]
+        for position in range(length - count, length):
+            slot_mapping.append(mine[position // page] * page + position % page)
+            positions.append(position)
+            token_sequence.append(index)
+        chunks.append(SequenceChunk(f"r{index}", index, length - count, count))
+    starts = [0]
+    for count in counts:
+        starts.append(starts[-1] + count)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+    group = GroupBatch(page, tables.cuda(), ints(slot_mapping), width)
+    batch = StepBatch(
+        num_tokens=sum(counts), chunks=chunks, token_ids=ints([0] * sum(counts)), positions=ints(positions),
+        token_sequence=ints(token_sequence), query_start=ints(starts), context_lengths=ints(lengths),
+        state_slots=ints(list(range(len(lengths)))), groups=[group], logit_rows=ints([]), num_logit_rows=0,
+        max_query_length=max(counts), max_context_length=max(lengths),
+    )
+    cell = CacheCell(PagedKeyValue(kv_heads, dim), True, 0, keys.to("cuda", dtype), values.to("cuda", dtype))
+    return batch, cell, per_request, HeadLayout(heads, kv_heads, dim)
+
+
+def step_rows(per_request, counts, heads, kv_heads, dim):
+    """The step's qkv rows [T, (heads + 2 kv) * dim] from the per-request tensors."""
+    rows = []
+    for (q, k, v), count in zip(per_request, counts):
+        rows.append(torch.cat([q[-count:].flatten(1), k[-count:].flatten(1), v[-count:].flatten(1)], dim=1))
+    return torch.cat(rows)
+
+
+ATTENTION_SHAPES = [  # heads, kv_heads, dim, page
+    (12, 2, 32, 16),  # the reference's own test shape (tests/test_triton_paged_attention.py:24)
+    (6, 1, 48, 8),
+    (5, 5, 80, 4),
+    (8, 2, 128, 16),
+    (3, 1, 112, 64),
+    (4, 4, 16, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,page", ATTENTION_SHAPES)
+def test_paged_attention_at_page_edges(kernels, dtype, heads, kv_heads, dim, page):
+    """Lengths around page edges (the reference's 1, 15, 16, 17, 31, 32, 33, scaled to the page),
+    single decoded tokens beside portions, shuffled pages, garbage in unused slots."""
+    lengths = [1, page - 1 or 1, page, page + 1, 2 * page - 1, 2 * page, 2 * page + 1, 5 * page + 3, 150]
+    counts = [1, 1, page, 1, 3, 2 * page, 1, 2 * page + 2, 1]
+    counts = [min(count, length) for count, length in zip(counts, lengths)]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=dim)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    scale = 0.37
+    out = kernels[dtype].paged_attention(qkv, layout, batch, cell, scale, None).cpu().double()
+    expected = []
+    for (q, k, v), count in zip(per_request, counts):
+        full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), scale)
+        expected.append(full[-count:].flatten(1))
+    torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 40])
+def test_paged_attention_window_edge(kernels, dtype, window):
+    """One key far back is made to stand out: it must count exactly while it is inside the window."""
+    heads, kv_heads, dim, page = 4, 2, 32, 8
+    lengths, counts = [70, 41], [30, 1]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=window)
+    for q, k, v in per_request:  # the key at the window's far edge of the last query dominates its scores
+        edge = q.shape[0] - window
+        if edge >= 0:
+            k[edge] = 4.0 * q[-1, ::2]
+    batch, cell, _, _ = _rewrite_cell(batch, cell, per_request, page, dtype)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    out = kernels[dtype].paged_attention(qkv, layout, batch, cell, 0.25, window).cpu().double()
+    expected = []
+    for (q, k, v), count in zip(per_request, counts):
+        full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), 0.25, window)
+        expected.append(full[-count:].flatten(1))
+    torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
+    wider = kernels[dtype].paged_attention(qkv, layout, batch, cell, 0.25, window + 1).cpu().double()
+    assert not torch.allclose(wider, out, atol=1e-2)
+
+
+def _rewrite_cell(batch, cell, per_request, page, dtype):
+    keys, values = cell.keys.cpu().float(), cell.values.cpu().float()
+    tables = batch.groups[0].block_tables.cpu()
+    for index, (q, k, v) in enumerate(per_request):
+        for position in range(k.shape[0]):
+            keys[tables[index, position // page], :, position % page] = k[position]
+            values[tables[index, position // page], :, position % page] = v[position]
+    cell.keys, cell.values = keys.to("cuda", dtype), values.to("cuda", dtype)
+    return batch, cell, per_request, None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_a_far_key_among_hundreds(kernels, dtype):
+    heads, kv_heads, dim, page = 6, 2, 64, 16
+    lengths, counts = [700], [1]
+    for far in (0, 15, 16, 337, 698):
+        batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=far)
+        q, k, v = per_request[0]
+        k[far] = 3.0 * q[-1, ::3]  # for heads 0 and 3 this key dominates; v[far] must come out
+        _rewrite_cell(batch, cell, per_request, page, dtype)
+        qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+        out = kernels[dtype].paged_attention(qkv, layout, batch, cell, 1.0, None).cpu().double().view(heads, dim)
+        full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), 1.0)[-1]
+        torch.testing.assert_close(out, full, **TOLERANCE[dtype])
+        torch.testing.assert_close(out[0], rounded(v, dtype)[far, 0], atol=5e-2, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("pairing", ["adjacent", "half", "none"])
+@pytest.mark.parametrize("heads,kv_heads,dim,page", [(6, 2, 32, 8), (5, 1, 48, 16), (2, 2, 128, 4)])
+def test_rotate_and_store(kernels, dtype, pairing, heads, kv_heads, dim, page):
+    lengths, counts = [9, 40, 1], [9, 3, 1]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype)
+    before_keys, before_values = cell.keys.clone(), cell.values.clone()
+    rows = step_rows(per_request, counts, heads, kv_heads, dim)
+    qkv = on_gpu(rows, dtype)
+    theta = 5000.0
+    inverse = 1.0 / (theta ** (torch.arange(0, dim, 2).float() / dim))
+    kernels[dtype].rotate_and_store(qkv, layout, batch, cell, None if pairing == "none" else on_gpu(inverse), pairing)
+    positions = batch.positions.cpu().long()
+    view = rounded(rows, dtype).view(-1, heads + 2 * kv_heads, dim)
+    angles = plain.rope_angles(dim, theta, positions)
+    rotate = {"adjacent": plain.rope_adjacent, "half": plain.rope_half, "none": lambda x, a: x}[pairing]
+    expected = torch.cat([rotate(view[:, : heads + kv_heads], angles), view[:, heads + kv_heads :]], dim=1)
+    torch.testing.assert_close(qkv.cpu().double().view_as(expected), expected, **TOLERANCE[dtype])
+    slots = batch.groups[0].slot_mapping.cpu().long()
+    stored_k = cell.keys.cpu().double()[slots // page, :, slots % page]
+    stored_v = cell.values.cpu().double()[slots // page, :, slots % page]
+    torch.testing.assert_close(stored_k, expected[:, heads : heads + kv_heads], **TOLERANCE[dtype])
+    torch.testing.assert_close(stored_v, expected[:, heads + kv_heads :], atol=0, rtol=0)
+    untouched = torch.ones(cell.keys.shape[0], page, dtype=torch.bool)
+    untouched[slots // page, slots % page] = False
+    same = lambda a, b: torch.equal(torch.nan_to_num(a.float().cpu(), nan=7.0), torch.nan_to_num(b.float().cpu(), nan=7.0))
+    assert same(cell.keys.transpose(1, 2)[untouched], before_keys.transpose(1, 2)[untouched])
+    assert same(cell.values.transpose(1, 2)[untouched], before_values.transpose(1, 2)[untouched])
+    # a cell that is only read stores nothing
+    readonly = types.SimpleNamespace(writable=False)
+    again = on_gpu(rows, dtype)
+    kernels[dtype].rotate_and_store(again, layout, batch, readonly, None if pairing == "none" else on_gpu(inverse), pairing)
+    torch.testing.assert_close(again, qkv)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gather_rows(kernels, dtype):
+    hidden, delta = torch.randn(9, 100), torch.randn(9, 100)
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    out = kernels[dtype].gather_rows(on_gpu(hidden), on_gpu(delta), on_gpu(rows))
+    torch.testing.assert_close(out.cpu(), (hidden + delta)[rows.long()])
+    torch.testing.assert_close(kernels[dtype].gather_rows(on_gpu(hidden), None, on_gpu(rows)).cpu(), hidden[rows.long()])
+
+
+@pytest.mark.parametrize("vocab", [5, 1000, 1025, 151936])
+def test_argmax_and_sampling(kernels, vocab):
+    k = kernels[torch.float32]
+    torch.manual_seed(vocab)
+    rows = 6
+    logits = 3.0 * torch.randn(rows, vocab)
+    logits[1, vocab // 2] = logits[1].max() + 1
+    logits[2, [3, vocab - 1]] = 50.0  # a tie: the first wins
+    assert k.argmax(on_gpu(logits)).cpu().tolist() == logits.argmax(-1).tolist()
+    assert k.argmax(on_gpu(logits)).cpu().tolist()[2] == 3
+    cases = [(0.0, 1.0), (0.8, 1.0), (0.7, 0.8), (1.5, 0.3), (0.2, 0.95), (1.0, 1.0)]
+    for draw in range(12):
+        uniforms = [plain.uniform_for(draw, row) for row in range(rows)]
+        got = k.sample(
+            on_gpu(logits), on_gpu(torch.tensor([c[0] for c in cases])), on_gpu(torch.tensor([c[1] for c in cases])),
+            on_gpu(torch.tensor(uniforms)),
+        ).cpu().tolist()
+        want = [plain.sample(logits[row], cases[row][0], cases[row][1], uniforms[row]) for row in range(rows)]
+        assert got == want, (draw, got, want)
+
+
+def test_sampling_edges(kernels):
+    k = kernels[torch.float32]
+    logits = torch.tensor([[0.0, 0.0, 0.0, 0.0], [5.0, 1.0, 5.0, 5.0], [1.0, 2.0, 3.0, 4.0]])
+    for u, want in ((0.0, [0, 0, 0]), (0.26, [1, 0, 0]), (0.9999, [3, 3, 3])):
+        got = k.sample(on_gpu(logits), on_gpu(torch.full((3,), 1.0)), on_gpu(torch.ones(3)), on_gpu(torch.full((3,), u))).cpu().tolist()
+        assert got[0] == want[0] and got[2] == plain.sample(logits[2], 1.0, 1.0, u)
+    # top-p with ties: equal entries are kept in index order until the mass is reached
+    for u in (0.0, 0.3, 0.4, 0.7, 0.99):
+        got = k.sample(on_gpu(logits), on_gpu(torch.full((3,), 1.0)), on_gpu(torch.full((3,), 0.6)), on_gpu(torch.full((3,), u))).cpu().tolist()
+        want = [plain.sample(logits[row], 1.0, 0.6, u) for row in range(3)]
+        assert got == want, (u, got, want)
