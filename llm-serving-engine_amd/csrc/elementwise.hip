@@ -127,15 +127,16 @@ extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const int* pos
 }
 
 // ---------------------------------------------------------------------------- SiLU(gate) * up
-// in: [rows, 2 * width] float32, gate in the first half of each row; out: [rows, width].
+// in: [rows, 2 * width] float32 with gate_j at column 2j and up_j at column 2j + 1 (the
+// product that made it had its weight rows interleaved); out: [rows, width].
 // silu(z) = z * sigmoid(z)  (reference model.py:188).
 template <typename TO>
 __global__ void silu_mul_kernel(const float* __restrict__ in, TO* __restrict__ out, int width) {
-  const float* row = in + (size_t)blockIdx.x * 2 * width;
+  const float2* row = (const float2*)(in + (size_t)blockIdx.x * 2 * width);
   TO* dst = out + (size_t)blockIdx.x * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float g = row[i], u = row[width + i];
-    dst[i] = from_float<TO>(g / (1.f + expf(-g)) * u);
+    const float2 pair = row[i];
+    dst[i] = from_float<TO>(pair.x / (1.f + expf(-pair.x)) * pair.y);
   }
 }
 

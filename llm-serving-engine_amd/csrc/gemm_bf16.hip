@@ -1,0 +1,156 @@
+// bfloat16 products on the matrix cores (MFMA), float32 accumulation.
+//
+// gemm_skinny: out[M, N] = x[M, K] . w[N, K]^T (+ bias) for M <= 64, the shape of decoding.
+// Such a product is a stream of the weight matrix from HBM, so the kernel is built around
+// that stream: a workgroup owns 16 weight rows and its waves split K between them; every
+// lane keeps two groups of four 16-byte loads of its weight row in flight; the weights go
+// straight from global memory into the A operand of v_mfma_f32_16x16x32_bf16 (lane l holds
+// row l % 16, k = (l / 16) * 8 .. + 8 of a 32-wide step), the few activation rows into the B
+// operand, so the result tile D[n][m] leaves four consecutive n of one token in each lane.
+// The waves' partial tiles are added through LDS in wave order, so a row's bits depend on
+// the shape of the weight only, not on what else is in the batch.
+//
+// With `gated`, weight rows alternate gate_j, up_j and the epilogue writes
+// silu(gate) * up (reference model.py:188) to out[M, N / 2].
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define STEP 32   // k per MFMA
+#define GROUP 4   // MFMA steps a wave loads at once: 128 k, 256 bytes of each weight row
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *(const bf16x8*)p; }
+
+template <int WAVES, int MT, typename TO, bool GATED>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
+                                                                 const bf16_t* __restrict__ w,
+                                                                 const void* __restrict__ bias, int bias_is_float,
+                                                                 TO* __restrict__ out, int M, int N, int K) {
+  extern __shared__ float partial[];  // [WAVES][MT][64 lanes][4]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int n = min((int)blockIdx.x * 16 + r, N - 1);
+  const bf16_t* w_row = w + (size_t)n * K + g * 8;
+  const bf16_t* x_row[MT];
+  bool x_live[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + r;
+    x_live[t] = m < M;
+    x_row[t] = x + (size_t)min(m, M - 1) * K + g * 8;
+  }
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  const int groups = K / (STEP * GROUP);
+  bf16x8 a[GROUP], a_next[GROUP];
+  int group = wave;
+  if (group < groups) {
+#pragma unroll
+    for (int u = 0; u < GROUP; ++u) a[u] = load8(w_row + (group * GROUP + u) * STEP);
+  }
+  while (group < groups) {
+    const int next = group + WAVES;
+    if (next < groups) {
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) a_next[u] = load8(w_row + (next * GROUP + u) * STEP);
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      bf16x8 b[GROUP];
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) b[u] = x_live[t] ? load8(x_row[t] + (group * GROUP + u) * STEP) : zero;
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u], acc[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < GROUP; ++u) a[u] = a_next[u];
+    group = next;
+  }
+  // the steps left over when K is not a multiple of 128
+  for (int step = groups * GROUP + wave; step < K / STEP; step += WAVES) {
+    const bf16x8 a_tail = load8(w_row + step * STEP);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const bf16x8 b_tail = x_live[t] ? load8(x_row[t] + step * STEP) : zero;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_tail, b_tail, acc[t], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < MT; ++t) *(f32x4*)(partial + ((wave * MT + t) * 64 + lane) * 4) = acc[t];
+  __syncthreads();
+  if (wave >= MT) return;
+  // wave t finishes token tile t: lane holds token m = t * 16 + r, rows n0 + g * 4 .. + 4
+  const int t = wave;
+  f32x4 total = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int v = 0; v < WAVES; ++v) total += *(const f32x4*)(partial + ((v * MT + t) * 64 + lane) * 4);
+  const int m = t * 16 + r;
+  const int n_first = blockIdx.x * 16 + g * 4;
+  if (m >= M) return;
+  if (bias) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n_first + i < N) total[i] += load_as_float(bias, bias_is_float, n_first + i);
+  }
+  if (GATED) {
+    TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (n_first + 2 * i + 1 < N) {
+        const float gate = total[2 * i], up = total[2 * i + 1];
+        dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+      }
+    }
+  } else {
+    TO* dst = out + (size_t)m * N + n_first;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n_first + i < N) dst[i] = from_float<TO>(total[i]);
+  }
+}
+
+template <int WAVES, int MT, typename TO, bool GATED>
+static int launch_skinny(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
+                         int K, hipStream_t stream) {
+  const size_t lds = (size_t)WAVES * MT * 64 * 4 * sizeof(float);
+  hipLaunchKernelGGL((gemm_skinny_kernel<WAVES, MT, TO, GATED>), dim3((N + 15) / 16), dim3(WAVES * 64), lds, stream,
+                     (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K);
+  return LAUNCH_STATUS();
+}
+
+template <int WAVES, typename TO, bool GATED>
+static int pick_tiles(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
+                      hipStream_t stream) {
+  if (M <= 16) return launch_skinny<WAVES, 1, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+  if (M <= 32) return launch_skinny<WAVES, 2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+  return launch_skinny<WAVES, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+}
+
+template <typename TO, bool GATED>
+static int pick_waves(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
+                      hipStream_t stream) {
+  // enough waves to cover the chip (about 2,048), but no more than there are 128-wide groups of K
+  const int tiles = (N + 15) / 16, groups = max(1, K / (STEP * GROUP));
+  int waves = 4;
+  while (waves < 16 && waves * tiles < 2048 && waves * 2 <= groups) waves *= 2;
+  if (waves == 4) return pick_tiles<4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+  if (waves == 8) return pick_tiles<8, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+  return pick_tiles<16, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+}
+
+// x, w bfloat16; out bfloat16 or float32.  Needs 1 <= M <= 64, K a multiple of 32, and with
+// `gated` an even N.  Any N.
+extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
+                                    int out_is_float, int gated, int M, int N, int K, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % STEP || (gated && N % 2)) return ERR_BAD_ARGUMENT;
+  if (gated)
+    return out_is_float ? pick_waves<float, true>(x, w, bias, bias_is_float, out, M, N, K, stream)
+                        : pick_waves<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, stream);
+  return out_is_float ? pick_waves<float, false>(x, w, bias, bias_is_float, out, M, N, K, stream)
+                      : pick_waves<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, stream);
+}

@@ -64,7 +64,9 @@ class LinearWeights:
 
 @dataclass
 class GatedLinearWeights:
-    """Gate and up weights as one [2 I, K] right-hand side: gate rows first."""
+    """Gate and up weights as one [2 I, K] right-hand side with rows interleaved:
+    gate_0, up_0, gate_1, up_1, ...  A kernel's output tile then holds a gate and
+    its up side by side, and act(gate) * up is applied before anything is stored."""
 
     both: LinearWeights
     width: int
@@ -84,6 +86,7 @@ class HipKernels:
         self._elementwise = load_module("elementwise")
         self._gemm_generic = load_module("gemm_generic")
         self._attention_generic = load_module("attention_generic")
+        self._gemm_bf16 = load_module("gemm_bf16") if dtype == torch.bfloat16 else None
         self._sampling = None
 
     # ------------------------------------------------------------------ helpers
@@ -161,7 +164,21 @@ class HipKernels:
         return LinearWeights(weight, bias)
 
     def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor) -> GatedLinearWeights:
-        return GatedLinearWeights(self.prepare_linear([gate, up], None), gate.shape[0])
+        if gate.shape != up.shape:
+            raise KernelError("gated_linear: gate and up differ in shape")
+        if gate.dtype != up.dtype:
+            gate, up = gate.float(), up.float()
+        both = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
+        return GatedLinearWeights(LinearWeights(both, None), gate.shape[0])
+
+    def _skinny(self, x: torch.Tensor, weights: LinearWeights) -> bool:
+        """Whether the weight-streaming MFMA kernel takes this product."""
+        return (
+            x.dtype == torch.bfloat16
+            and weights.weight.dtype == torch.bfloat16
+            and 0 < x.shape[0] <= 64
+            and weights.in_features % 32 == 0
+        )
 
     def linear(self, x: torch.Tensor, weights: LinearWeights, out_dtype: torch.dtype | None = None) -> torch.Tensor:
         rows, inner = x.shape
@@ -169,17 +186,30 @@ class HipKernels:
             raise KernelError(f"linear: x has {inner} columns, the weight {weights.in_features}")
         out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
         bias = weights.bias
-        status = self._gemm_generic.llmserve_gemm_generic(
-            _pointer(x), _is_float(x), _pointer(weights.weight), _is_float(weights.weight), _pointer(bias),
-            _is_float(bias) if bias is not None else 0, _pointer(out), _is_float(out), rows,
-            weights.out_features, inner, self._stream,
-        )
+        bias_is_float = _is_float(bias) if bias is not None else 0
+        if self._skinny(x, weights):
+            status = self._gemm_bf16.llmserve_gemm_skinny(
+                _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out), _is_float(out),
+                0, rows, weights.out_features, inner, self._stream,
+            )
+        else:
+            status = self._gemm_generic.llmserve_gemm_generic(
+                _pointer(x), _is_float(x), _pointer(weights.weight), _is_float(weights.weight), _pointer(bias),
+                bias_is_float, _pointer(out), _is_float(out), rows, weights.out_features, inner, self._stream,
+            )
         _check(status, "linear")
         return out
 
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
-        both = self.linear(x, weights.both, out_dtype=torch.float32)
         out = self._empty((x.shape[0], weights.width), self.dtype)
+        if self._skinny(x, weights.both):
+            status = self._gemm_bf16.llmserve_gemm_skinny(
+                _pointer(x), _pointer(weights.both.weight), _pointer(None), 0, _pointer(out), _is_float(out), 1,
+                x.shape[0], 2 * weights.width, x.shape[1], self._stream,
+            )
+            _check(status, "gated_linear")
+            return out
+        both = self.linear(x, weights.both, out_dtype=torch.float32)
         status = self._elementwise.llmserve_silu_mul(
             _pointer(both), _pointer(out), _is_float(out), x.shape[0], weights.width, self._stream
         )

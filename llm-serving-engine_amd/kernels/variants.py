@@ -7,6 +7,7 @@ from __future__ import annotations
 DEFAULT_VARIANTS: dict[str, list[dict[str, object]]] = {
     "elementwise": [{}],
     "gemm_generic": [{}],
+    "gemm_bf16": [{}],
     "attention_generic": [{}],
     "sampling": [{}],
 }

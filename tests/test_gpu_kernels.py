@@ -65,10 +65,13 @@ def test_add_rms_norm(kernels, dtype, width, eps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows,inner,outer", [(1, 72, 50), (5, 200, 333), (70, 129, 65), (130, 64, 1000)])
+@pytest.mark.parametrize("rows,inner,outer", [(1, 72, 50), (5, 200, 333), (70, 129, 65), (130, 64, 1000),
+                                              (1, 256, 48), (8, 1536, 272), (16, 96, 1000), (17, 1184, 50), (33, 512, 24),
+                                              (64, 4480, 130), (64, 160, 2048)])
 def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
     k = kernels[dtype]
-    x, w, b = torch.randn(rows, inner), 0.1 * torch.randn(outer, inner), torch.randn(outer)
+    # weights scaled so that every output is of order one, whatever `inner` is
+    x, w, b = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer)
     expected = rounded(x, dtype) @ rounded(w, dtype).T + rounded(b, dtype)
     parts = [w[: outer // 3], w[outer // 3 :]], [b[: outer // 3], b[outer // 3 :]]
     handle = k.prepare_linear([on_gpu(p, dtype) for p in parts[0]], [on_gpu(p, dtype) for p in parts[1]])
@@ -82,7 +85,7 @@ def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
     # a weight kept in 32-bit under a bfloat16 run
     wide = k.linear(on_gpu(x, dtype), k.prepare_linear([on_gpu(w)], None), out_dtype=torch.float32)
     torch.testing.assert_close(wide.cpu().double(), rounded(x, dtype) @ w.double().T, atol=1e-4, rtol=1e-4)
-    up = 0.1 * torch.randn(outer, inner)
+    up = torch.randn(outer, inner) / math.sqrt(inner)
     gated = k.gated_linear(on_gpu(x, dtype), k.prepare_gated_linear(on_gpu(w, dtype), on_gpu(up, dtype)))
     want = F.silu(rounded(x, dtype) @ rounded(w, dtype).T) * (rounded(x, dtype) @ rounded(up, dtype).T)
     torch.testing.assert_close(gated.cpu().double(), want, **TOLERANCE[dtype])
