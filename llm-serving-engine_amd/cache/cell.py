@@ -12,8 +12,10 @@ import torch
 class CacheCell:
     """What one run of a layer sees of the cache.
 
-    For a paged need: `keys` and `values` are [pages, kv_heads, page_size,
-    head_dim] and `group` indexes `StepBatch.groups`.  For a fixed state:
+    For a paged need: `keys` is [pages, kv_heads, page_size, head_dim], `values`
+    is stored transposed, [pages, kv_heads, head_dim, page_size] (attention
+    sums over keys, and the matrix cores want the summed index contiguous), and
+    `group` indexes `StepBatch.groups`.  For a fixed state:
     `state` is [slots, *shape] float32, indexed by `StepBatch.state_slots`.
     `writable` is False when the run reads a cell that another run owns.
     """

@@ -146,7 +146,9 @@ class CacheManager:
                         writable=writable,
                         group=entry[1],
                         keys=group.storage[entry[2], 0],
-                        values=group.storage[entry[2], 1],
+                        values=group.storage[entry[2], 1].view(
+                            self.config.num_blocks, group.need.num_kv_heads, group.need.head_dim, self.page_size
+                        ),
                     )
                 )
             else:

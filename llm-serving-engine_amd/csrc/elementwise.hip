@@ -71,8 +71,8 @@ extern "C" int llmserve_add_rms_norm(float* hidden, const float* delta, const vo
 // becomes (a cos - b sin, b cos + a sin) with angle = position * inverse[j], all in float32.
 // pairing 0: none, 1: adjacent pairs (2j, 2j+1), 2: half pairs (j, j + dim/2).
 // k (after rotation) and v are then written to the pages: slot = page * page_size + offset,
-// pages laid out [page, kv_head, offset, dim] (reference kv_cache.py:249-266 writes
-// [page, offset, kv_head, dim]).  slots may be null (nothing is stored); a negative slot
+// key pages laid out [page, kv_head, offset, dim], value pages transposed [page, kv_head,
+// dim, offset] (reference kv_cache.py:249-266 writes both as [page, offset, kv_head, dim]).  slots may be null (nothing is stored); a negative slot
 // skips the token.
 template <typename T>
 __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
@@ -106,9 +106,9 @@ __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const int* __restri
   const T* v_row = k_row + kv_heads * dim;
   for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
     const int head = i / dim, d = i % dim;
-    const size_t at = (((size_t)page * kv_heads + head) * page_size + offset) * dim + d;
-    keys[at] = k_row[i];
-    values[at] = v_row[i];
+    const size_t block = ((size_t)page * kv_heads + head) * page_size * dim;
+    keys[block + (size_t)offset * dim + d] = k_row[i];
+    values[block + (size_t)d * page_size + offset] = v_row[i];
   }
 }
 

@@ -87,6 +87,7 @@ class HipKernels:
         self._gemm_generic = load_module("gemm_generic")
         self._attention_generic = load_module("attention_generic")
         self._gemm_bf16 = load_module("gemm_bf16") if dtype == torch.bfloat16 else None
+        self._attention_bf16: dict[int, ctypes.CDLL] = {}  # by head size, compiled when a model needs it
         self._sampling = None
 
     # ------------------------------------------------------------------ helpers
@@ -218,20 +219,82 @@ class HipKernels:
 
     # ------------------------------------------------------------------ attention
 
+    def _attention_library(self, head_dim: int):
+        if head_dim not in self._attention_bf16:
+            self._attention_bf16[head_dim] = load_module("attention_bf16", {"HEAD_DIM": head_dim})
+        return self._attention_bf16[head_dim]
+
+    def _attention_work(self, batch, tokens_per_item: int, longer_than: int, up_to: int | None):
+        """Work items (request, first row, tokens, 0) for the requests of the step whose token
+        count lies in (longer_than, up_to], cut into items of `tokens_per_item` tokens.  Built
+        once per step and kept on the batch."""
+        key = ("attention_work", tokens_per_item, longer_than, up_to)
+        if key not in batch.scratch:
+            import numpy as np
+
+            counts = np.array([chunk.count for chunk in batch.chunks], dtype=np.int64)
+            starts = np.concatenate([[0], np.cumsum(counts)[:-1]])
+            chosen = counts > longer_than
+            if up_to is not None:
+                chosen &= counts <= up_to
+            which = np.nonzero(chosen)[0]
+            items = -(-counts[which] // tokens_per_item)
+            request = np.repeat(which, items)
+            inside = np.arange(int(items.sum())) - np.repeat(np.cumsum(items) - items, items)
+            first = inside * tokens_per_item
+            tokens = np.minimum(tokens_per_item, counts[request] - first)
+            work = np.stack([request, starts[request] + first, tokens, np.zeros_like(first)], axis=1).astype(np.int32)
+            batch.scratch[key] = (self.to_device(torch.from_numpy(work)) if len(work) else None, len(work))
+        return batch.scratch[key]
+
     def paged_attention(self, qkv, layout, batch, cell, scale: float, window: int | None) -> torch.Tensor:
         tokens = qkv.shape[0]
         group = batch.groups[cell.group]
         if cell.keys.dtype != qkv.dtype:
             raise KernelError("paged_attention: queries and pages differ in type")
         out = self._empty((tokens, layout.num_heads * layout.head_dim), qkv.dtype)
+        dim = layout.head_dim
+        if qkv.dtype == torch.bfloat16 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
+            self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0))
+            return out
         status = self._attention_generic.llmserve_attention_generic(
             _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
             _pointer(group.block_tables), group.width, _pointer(batch.token_sequence), _pointer(batch.positions),
-            tokens, layout.num_heads, layout.num_kv_heads, layout.head_dim, group.page_size,
+            tokens, layout.num_heads, layout.num_kv_heads, dim, group.page_size,
             ctypes.c_float(scale), int(window or 0), self._stream,
         )
         _check(status, "paged_attention")
         return out
+
+    def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int) -> None:
+        """The MFMA kernel: requests that bring a few tokens (decoding) one column tile per
+        wave, split over the keys when there are few of them; longer portions four tiles per wave."""
+        library = self._attention_library(layout.head_dim)
+        heads, kv_heads = layout.num_heads, layout.num_kv_heads
+        per_tile = max(1, 16 // (heads // kv_heads))
+        head_tiles = -(-(heads // kv_heads) // 16)
+        tokens = qkv.shape[0]
+        launches = [(1, *self._attention_work(batch, per_tile, 0, per_tile))]
+        if batch.max_query_length > per_tile:
+            launches.append((4, *self._attention_work(batch, 4 * per_tile, per_tile, None)))
+        for column_tiles, work, items in launches:
+            if items == 0:
+                continue
+            splits, partial_acc, partial_ml = 1, None, None
+            if batch.max_query_length <= per_tile:  # only then does one launch cover every row
+                blocks = items * kv_heads * head_tiles
+                steps = -(-batch.max_context_length // 32)
+                splits = max(1, min(-(-1024 // blocks), -(-steps // 4), 64))
+                if splits > 1:
+                    partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), torch.float32)
+                    partial_ml = self._empty((tokens * heads * splits * 2,), torch.float32)
+            status = library.llmserve_attention_tiles(
+                _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
+                _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width,
+                _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
+                group.page_size, ctypes.c_float(scale), window, splits, self._stream,
+            )
+            _check(status, "paged_attention")
 
     # ------------------------------------------------------------------ sampling
 

@@ -105,7 +105,7 @@ def paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=
     width = max(blocks)
     tables = torch.full((len(lengths), width), -1, dtype=torch.int32)
     keys = torch.full((pages, kv_heads, page, dim), float("nan"))
-    values = torch.full((pages, kv_heads, page, dim), float("nan"))
+    values = torch.full((pages, kv_heads, dim, page), float("nan"))  # value pages are stored transposed
     per_request, slot_mapping, positions, token_sequence, chunks = [], [], [], [], []
     for index, (length, count) in enumerate(zip(lengths, counts)):
         mine = [order.pop() for _ in range(blocks[index])]
@@ -116,7 +116,7 @@ def paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=
         per_request.append((q, k, v))
         for position in range(length):
             keys[mine[position // page], :, position % page] = k[position]
-            values[mine[position // page], :, position % page] = v[position]
+            values[mine[position // page], :, :, position % page] = v[position]
         for position in range(length - count, length):
             slot_mapping.append(mine[position // page] * page + position % page)
             positions.append(position)
@@ -203,7 +203,7 @@ def _rewrite_cell(batch, cell, per_request, page, dtype):
     for index, (q, k, v) in enumerate(per_request):
         for position in range(k.shape[0]):
             keys[tables[index, position // page], :, position % page] = k[position]
-            values[tables[index, position // page], :, position % page] = v[position]
+            values[tables[index, position // page], :, :, position % page] = v[position]
     cell.keys, cell.values = keys.to("cuda", dtype), values.to("cuda", dtype)
     return batch, cell, per_request, None
 
@@ -244,14 +244,14 @@ def test_rotate_and_store(kernels, dtype, pairing, heads, kv_heads, dim, page):
     torch.testing.assert_close(qkv.cpu().double().view_as(expected), expected, **TOLERANCE[dtype])
     slots = batch.groups[0].slot_mapping.cpu().long()
     stored_k = cell.keys.cpu().double()[slots // page, :, slots % page]
-    stored_v = cell.values.cpu().double()[slots // page, :, slots % page]
+    stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
     torch.testing.assert_close(stored_k, expected[:, heads : heads + kv_heads], **TOLERANCE[dtype])
     torch.testing.assert_close(stored_v, expected[:, heads + kv_heads :], atol=0, rtol=0)
     untouched = torch.ones(cell.keys.shape[0], page, dtype=torch.bool)
     untouched[slots // page, slots % page] = False
     same = lambda a, b: torch.equal(torch.nan_to_num(a.float().cpu(), nan=7.0), torch.nan_to_num(b.float().cpu(), nan=7.0))
     assert same(cell.keys.transpose(1, 2)[untouched], before_keys.transpose(1, 2)[untouched])
-    assert same(cell.values.transpose(1, 2)[untouched], before_values.transpose(1, 2)[untouched])
+    assert same(cell.values.permute(0, 3, 1, 2)[untouched], before_values.permute(0, 3, 1, 2)[untouched])
     # a cell that is only read stores nothing
     readonly = types.SimpleNamespace(writable=False)
     again = on_gpu(rows, dtype)

@@ -79,7 +79,7 @@ class TorchKernels:
             slots = group.slot_mapping.long()
             pages, offsets = slots // group.page_size, slots % group.page_size
             cell.keys[pages, :, offsets] = view[:, heads : heads + kv_heads]
-            cell.values[pages, :, offsets] = view[:, heads + kv_heads :]
+            cell.values[pages, :, :, offsets] = view[:, heads + kv_heads :]  # pages are [kv, dim, offset]
 
     def paged_attention(self, qkv, layout, batch, cell, scale, window):
         tokens = qkv.shape[0]
@@ -96,7 +96,7 @@ class TorchKernels:
                 pages = table[where // group.page_size]
                 assert (pages >= 0).all(), "attention reads a page that was given back"
                 keys = cell.keys[pages, :, where % group.page_size].float()  # [n, kv, D]
-                values = cell.values[pages, :, where % group.page_size].float()
+                values = cell.values[pages, :, :, where % group.page_size].float()
                 keys = keys.repeat_interleave(heads // kv_heads, dim=1)
                 values = values.repeat_interleave(heads // kv_heads, dim=1)
                 scores = torch.einsum("hd,nhd->hn", queries[row], keys) * scale
