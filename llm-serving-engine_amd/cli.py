@@ -1,0 +1,213 @@
+"""The `llmserve` command line, in the reference's manner (`src/llmserve/cli.py:244-328`):
+argparse subcommands, with the reference's option names and meanings where it has them.
+
+    llmserve benchmark   run the synthetic open-loop workload through the engine
+    llmserve generate    generate tokens for one prompt
+    llmserve replay      feed token ids step by step and write logits (bin/trace_run)
+    llmserve random-model  write a model folder with seeded random weights
+
+The reference's `serve`, `quantize-eval` and `speculative-eval` have no counterpart here:
+servers, quantized weights and speculative decoding are outside this engine.
+"""
+
+from __future__ import annotations
+
+import argparse
+import asyncio
+import json
+import sys
+import tempfile
+from dataclasses import replace
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def _load_runtime(args):
+    """A model folder, or without --model the bundled tiny configuration with weights drawn
+    from --seed and the byte tokenizer (`cli.py:22-45`)."""
+    from .config import Qwen2Config
+    from .engine.tokenizer import ByteTokenizer, FileTokenizer
+    from .weights import load_model_folder, write_model_folder
+
+    if args.model:
+        loaded = load_model_folder(args.model, args.dtype)
+        try:
+            tokenizer = FileTokenizer(args.model)
+        except FileNotFoundError:
+            tokenizer = ByteTokenizer()
+        return loaded, tokenizer
+    config = Qwen2Config.from_json_file(ROOT / "configs" / "tiny.json")
+    folder = write_model_folder(Path(tempfile.mkdtemp(prefix="llmserve-tiny-")), config, seed=args.seed)
+    return load_model_folder(folder, args.dtype), ByteTokenizer()
+
+
+def _engine(args, loaded, tokenizer, *, batch_size: int, mode: str):
+    from .config import CacheConfig, SchedulerConfig
+    from .engine import LLMEngine
+
+    return LLMEngine(
+        loaded,
+        tokenizer,
+        cache_config=CacheConfig(args.block_size, args.num_blocks, max(batch_size, 1)),
+        scheduler_config=SchedulerConfig(batch_size, max(args.max_tokens_per_step, batch_size), args.policy),
+        scheduler_mode=mode,
+        prefill_chunk_size=args.prefill_chunk_size,
+        collect_iteration_metrics=True,
+        device=args.device if args.device != "auto" else "cuda:0",
+        dtype=args.dtype,
+    )
+
+
+async def _benchmark(args) -> None:
+    """`cli.py:48-125`: naive = one request at a time, the whole prefix again for every token;
+    paged = the engine with batch size 1; static and continuous = the two admission modes."""
+    from .benchmark import BenchmarkHarness, LoadProfile
+    from .sampling import GenerationConfig
+
+    loaded, tokenizer = _load_runtime(args)
+    profile = LoadProfile.from_yaml(args.profile)
+    longest = loaded.config.max_position_embeddings
+    profile = replace(
+        profile,
+        requests=args.requests or profile.requests,
+        arrival_rate=args.arrival_rate or profile.arrival_rate,
+        vocabulary_size=loaded.config.vocab_size,
+        prompt=replace(profile.prompt, maximum=min(profile.prompt.maximum, longest - profile.output.maximum)),
+    )
+    harness = BenchmarkHarness(profile)
+    batch_size = 1 if args.config in ("naive", "paged") else args.batch_size
+    engine = _engine(args, loaded, tokenizer, batch_size=batch_size, mode="static" if args.config == "static" else "continuous")
+
+    def settings(count: int) -> GenerationConfig:
+        return GenerationConfig(max_new_tokens=count, temperature=0.0, seed=args.seed, stop_token_ids=())
+
+    if args.config == "naive":
+        lock = asyncio.Lock()
+
+        async def generate(spec, callback):
+            async with lock:  # reference engine.py:83-105: no cache is kept between tokens
+                prompt, output = list(spec.prompt_token_ids), []
+                for _ in range(spec.max_new_tokens):
+                    token = (await engine.generate(prompt + output, settings(1)))[0]
+                    output.append(token)
+                    callback(token)
+                return output
+    else:
+
+        async def generate(spec, callback):
+            return await engine.generate(
+                list(spec.prompt_token_ids), settings(spec.max_new_tokens), callback, request_id=spec.request_id
+            )
+
+    report = await harness.run(f"{args.config}-{args.policy}", generate)
+    report.cache = engine.cache_stats
+    report.metadata["engine"] = engine.iteration_stats
+    await engine.close()
+    engine.runner.close()
+    output = Path(args.output)
+    output.parent.mkdir(parents=True, exist_ok=True)
+    report.write_json(output)
+    report.write_csv(output.with_suffix(".csv"))
+    print(json.dumps(report.summary, indent=2))
+
+
+async def _generate(args) -> None:
+    from .sampling import GenerationConfig
+
+    loaded, tokenizer = _load_runtime(args)
+    engine = _engine(args, loaded, tokenizer, batch_size=1, mode="continuous")
+    prompt = [int(t) for t in args.prompt_tokens.split(",")] if args.prompt_tokens else args.prompt
+    settings = GenerationConfig(args.max_tokens, args.temperature, args.top_p, args.seed, tuple(args.stop_token_id or ()))
+    tokens = await engine.generate(prompt, settings)
+    await engine.close()
+    engine.runner.close()
+    print(json.dumps({"token_ids": tokens, "text": tokenizer.decode(tokens)}))
+
+
+def _replay(args) -> int:
+    import subprocess
+
+    command = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", args.model, "--dtype", args.dtype, "--out",
+               args.out, "--max-tokens", str(args.max_tokens), "--block-size", str(args.block_size)]
+    return subprocess.call(command)
+
+
+def _random_model(args) -> None:
+    import torch
+
+    from .config import Qwen2Config
+    from .weights import write_model_folder
+
+    config = Qwen2Config.from_json_file(args.config)
+    folder = write_model_folder(args.output, config, args.seed, dtype=torch.bfloat16, norm_std=args.norm_std,
+                                bias_std=args.bias_std, std=args.std)
+    print(folder)
+
+
+def _engine_options(parser: argparse.ArgumentParser) -> None:
+    parser.add_argument("--model", help="model folder with config.json and safetensors files")
+    parser.add_argument("--device", default="auto")
+    parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    parser.add_argument("--block-size", type=int, default=16)
+    parser.add_argument("--num-blocks", type=int, default=1024)
+    parser.add_argument("--prefill-chunk-size", type=int, default=16)
+    parser.add_argument("--max-tokens-per-step", type=int, default=2048)
+    parser.add_argument("--policy", choices=("fcfs", "sjf", "priority"), default="fcfs")
+    parser.add_argument("--seed", type=int, default=7)
+
+
+def build_parser() -> argparse.ArgumentParser:
+    parser = argparse.ArgumentParser(prog="llmserve")
+    commands = parser.add_subparsers(dest="command", required=True)
+
+    benchmark = commands.add_parser("benchmark", help="run the synthetic workload")
+    benchmark.add_argument("--config", choices=("naive", "paged", "static", "continuous"), default="continuous")
+    benchmark.add_argument("--profile", default=str(ROOT / "configs" / "benchmark-sharegpt.yaml"))
+    benchmark.add_argument("--requests", type=int)
+    benchmark.add_argument("--arrival-rate", type=float)
+    benchmark.add_argument("--batch-size", type=int, default=16)
+    benchmark.add_argument("--output", default="artifacts/benchmark.json")
+    _engine_options(benchmark)
+
+    generate = commands.add_parser("generate", help="generate tokens for one prompt")
+    generate.add_argument("--prompt", default="Explain paged attention in one paragraph.")
+    generate.add_argument("--prompt-tokens", help="comma-separated token ids instead of --prompt")
+    generate.add_argument("--max-tokens", type=int, default=32)
+    generate.add_argument("--temperature", type=float, default=0.0)
+    generate.add_argument("--top-p", type=float, default=1.0)
+    generate.add_argument("--stop-token-id", type=int, action="append")
+    _engine_options(generate)
+
+    replay = commands.add_parser("replay", help="feed token ids step by step (stdin) and write logits")
+    replay.add_argument("--model", required=True)
+    replay.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    replay.add_argument("--out", required=True)
+    replay.add_argument("--max-tokens", type=int, required=True)
+    replay.add_argument("--block-size", type=int, default=16)
+
+    random_model = commands.add_parser("random-model", help="write a model folder with seeded random weights")
+    random_model.add_argument("--config", required=True, help="a config.json")
+    random_model.add_argument("--output", required=True)
+    random_model.add_argument("--seed", type=int, default=7)
+    random_model.add_argument("--std", type=float, default=0.02)
+    random_model.add_argument("--bias-std", type=float, default=0.02)
+    random_model.add_argument("--norm-std", type=float, default=0.0)
+    return parser
+
+
+def main(argv: list[str] | None = None) -> int:
+    args = build_parser().parse_args(argv)
+    if args.command == "benchmark":
+        asyncio.run(_benchmark(args))
+    elif args.command == "generate":
+        asyncio.run(_generate(args))
+    elif args.command == "replay":
+        return _replay(args)
+    else:
+        _random_model(args)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -127,26 +127,31 @@ extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const int* pos
 }
 
 // ---------------------------------------------------------------------------- SiLU(gate) * up
-// in: [rows, 2 * width] float32 with gate_j at column 2j and up_j at column 2j + 1 (the
+// in: [rows, 2 * width] float32 or bfloat16 with gate_j at column 2j and up_j at column 2j + 1 (the
 // product that made it had its weight rows interleaved); out: [rows, width].
 // silu(z) = z * sigmoid(z)  (reference model.py:188).
-template <typename TO>
-__global__ void silu_mul_kernel(const float* __restrict__ in, TO* __restrict__ out, int width) {
-  const float2* row = (const float2*)(in + (size_t)blockIdx.x * 2 * width);
+template <typename TI, typename TO>
+__global__ void silu_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out, int width) {
+  const TI* row = in + (size_t)blockIdx.x * 2 * width;
   TO* dst = out + (size_t)blockIdx.x * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float2 pair = row[i];
-    dst[i] = from_float<TO>(pair.x / (1.f + expf(-pair.x)) * pair.y);
+    const float gate = to_float(row[2 * i]), up = to_float(row[2 * i + 1]);
+    dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
   }
 }
 
-extern "C" int llmserve_silu_mul(const float* in, void* out, int out_is_float, int rows, int width,
+extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
                                  hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (out_is_float)
-    hipLaunchKernelGGL(silu_mul_kernel<float>, dim3(rows), dim3(256), 0, stream, in, (float*)out, width);
+  const dim3 grid(rows), block(256);
+  if (in_is_float && out_is_float)
+    hipLaunchKernelGGL((silu_mul_kernel<float, float>), grid, block, 0, stream, (const float*)in, (float*)out, width);
+  else if (in_is_float)
+    hipLaunchKernelGGL((silu_mul_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)in, (bf16_t*)out, width);
+  else if (out_is_float)
+    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)in, (float*)out, width);
   else
-    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, in, (bf16_t*)out, width);
+    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, width);
   return LAUNCH_STATUS();
 }
 

@@ -11,6 +11,7 @@ counterpart is the second half of `LLMEngine._step` plus
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from typing import Any
 
 import numpy as np
 import torch
@@ -33,45 +34,69 @@ class StepEntry:
     want: tuple[int, ...] | list[int] = field(default_factory=tuple)
 
 
-def build_step_batch(
+def _pack_step(
     reservations: list[Reservation],
     entries: list[StepEntry],
     cache: CacheManager,
-    device: torch.device,
-) -> StepBatch:
-    """All index arrays of a step, packed on the host and sent in one copy."""
+    *,
+    pad_to: int | None = None,
+    width: int | None = None,
+) -> tuple[np.ndarray, list[int], list[int], dict]:
+    """The step's index arrays as one int32 array: token ids, positions, request index per
+    token, query starts, context lengths, state slots, wanted rows, then per cache group the
+    slot of every token and the requests' block-table rows.  With `pad_to`, requests are
+    padded to that many (one token each, stored nowhere, reading page 0), for a captured graph."""
     counts = np.array([r.count for r in reservations], dtype=np.int64)
-    total = int(counts.sum())
-    query_start = np.zeros(len(reservations) + 1, dtype=np.int32)
-    query_start[1:] = np.cumsum(counts)
-    token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
-    positions = np.concatenate([np.arange(r.start, r.start + r.count, dtype=np.int32) for r in reservations])
-    token_sequence = np.repeat(np.arange(len(reservations), dtype=np.int32), counts)
-    context = np.array([r.start + r.count for r in reservations], dtype=np.int32)
-    slots = np.array([r.slot for r in reservations], dtype=np.int32)
+    requests = len(reservations)
+    padded = pad_to if pad_to is not None else requests
+    extra = padded - requests
+    total = int(counts.sum()) + extra
+    query_start = np.zeros(padded + 1, dtype=np.int32)
+    query_start[1:] = np.cumsum(np.concatenate([counts, np.ones(extra, np.int64)]))
+    token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries] + [np.zeros(extra, np.int32)])
+    positions = np.concatenate(
+        [np.arange(r.start, r.start + r.count, dtype=np.int32) for r in reservations] + [np.zeros(extra, np.int32)]
+    )
+    token_sequence = np.repeat(np.arange(padded, dtype=np.int32), np.concatenate([counts, np.ones(extra, np.int64)]))
+    context = np.array([r.start + r.count for r in reservations] + [1] * extra, dtype=np.int32)
+    slots = np.array([r.slot for r in reservations] + [0] * extra, dtype=np.int32)
     rows = [query_start[b] + np.asarray(e.want, dtype=np.int32) for b, e in enumerate(entries)]
     logit_rows = np.concatenate(rows).astype(np.int32) if rows else np.zeros(0, np.int32)
-
+    if pad_to is not None:
+        logit_rows = np.arange(padded, dtype=np.int32)
     pieces = [token_ids, positions, token_sequence, query_start, context, slots, logit_rows]
     widths = []
+    real_slots = slots[:requests]
     for index, group in enumerate(cache.groups):
-        width = max(1, int(-(-int(context.max()) // cache.page_size)))
-        widths.append(width)
-        pieces.append(np.concatenate([r.slots[index] for r in reservations]))
-        pieces.append(group.tables[slots, :width].reshape(-1))
-    sizes = [piece.size for piece in pieces]
-    packed = torch.from_numpy(np.concatenate(pieces).astype(np.int32, copy=False))
-    on_device = packed.to(device)
+        needed = max(1, int(-(-int(context.max()) // cache.page_size)))
+        group_width = width if width is not None else needed
+        widths.append(group_width)
+        mapping = np.concatenate([r.slots[index] for r in reservations] + [np.full(extra, -1, np.int32)])
+        tables = np.zeros((padded, group_width), dtype=np.int32)
+        tables[:requests, : min(needed, group_width)] = group.tables[real_slots, : min(needed, group_width)]
+        pieces.append(mapping)
+        pieces.append(tables.reshape(-1))
+    sizes = [int(piece.size) for piece in pieces]
+    facts = {
+        "num_tokens": total,
+        "num_logit_rows": int(logit_rows.size),
+        "max_query_length": int(counts.max()),
+        "max_context_length": int(context.max()),
+        "requests": padded,
+    }
+    return np.concatenate(pieces).astype(np.int32, copy=False), sizes, widths, facts
+
+
+def _view_step(
+    on_device: torch.Tensor, sizes: list[int], widths: list[int], facts: dict, chunks: list[SequenceChunk], page_size: int
+) -> StepBatch:
     views = list(torch.split(on_device, sizes))
     groups = []
-    for index in range(len(cache.groups)):
+    for index, width in enumerate(widths):
         mapping, tables = views[7 + 2 * index], views[8 + 2 * index]
-        groups.append(
-            GroupBatch(cache.page_size, tables.view(len(reservations), widths[index]), mapping, widths[index])
-        )
-    chunks = [SequenceChunk(r.request_id, r.slot, r.start, r.count) for r in reservations]
+        groups.append(GroupBatch(page_size, tables.view(facts["requests"], width), mapping, width))
     return StepBatch(
-        num_tokens=total,
+        num_tokens=facts["num_tokens"],
         chunks=chunks,
         token_ids=views[0],
         positions=views[1],
@@ -81,10 +106,40 @@ def build_step_batch(
         state_slots=views[5],
         groups=groups,
         logit_rows=views[6],
-        num_logit_rows=int(logit_rows.size),
-        max_query_length=int(counts.max()),
-        max_context_length=int(context.max()),
+        num_logit_rows=facts["num_logit_rows"],
+        max_query_length=facts["max_query_length"],
+        max_context_length=facts["max_context_length"],
     )
+
+
+def build_step_batch(
+    reservations: list[Reservation],
+    entries: list[StepEntry],
+    cache: CacheManager,
+    device: torch.device,
+) -> StepBatch:
+    """All index arrays of a step, packed on the host and sent in one copy."""
+    packed, sizes, widths, facts = _pack_step(reservations, entries, cache)
+    on_device = torch.from_numpy(packed).to(device)
+    chunks = [SequenceChunk(r.request_id, r.slot, r.start, r.count) for r in reservations]
+    return _view_step(on_device, sizes, widths, facts, chunks, cache.page_size)
+
+
+@dataclass
+class _DecodeGraph:
+    """One captured decode step: `requests` single tokens against block tables `width` wide."""
+
+    requests: int
+    width: int
+    graph: Any
+    static: torch.Tensor  # the packed index arrays the captured kernels read
+    host: list[torch.Tensor]  # two pinned staging buffers, used in turn
+    copied: list[Any]  # per staging buffer: the event after its last copy
+    logits: torch.Tensor
+    # The captured kernels read the batch's tensors by address, also the work lists that the
+    # kernel library keeps on it: the batch lives as long as the graph.
+    batch: StepBatch | None = None
+    turn: int = 0
 
 
 class ModelRunner:
@@ -97,6 +152,7 @@ class ModelRunner:
         cache_config: CacheConfig | None = None,
         *,
         max_sequence_length: int | None = None,
+        use_graphs: bool | None = None,
     ) -> None:
         self.loaded = loaded
         self.kernels = kernels
@@ -119,6 +175,14 @@ class ModelRunner:
         )
         self.cells = self.cache.cells()
         self.vocab_size = loaded.spec.vocab_size
+        self.use_graphs = self.device.type == "cuda" if use_graphs is None else use_graphs
+        self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
+
+    def close(self) -> None:
+        """Drops the captured graphs (while the device runtime is still up)."""
+        if self._graphs:
+            torch.cuda.synchronize(self.device)
+        self._graphs.clear()
 
     def add_request(self, request_id: str) -> int:
         return self.cache.create(request_id)
@@ -131,7 +195,8 @@ class ModelRunner:
 
     def step(self, entries: list[StepEntry], *, create_missing: bool = False) -> torch.Tensor:
         """Runs the entries as one batch; returns float32 logits [wanted, vocab]
-        in the order of the entries and of each entry's `want`.
+        in the order of the entries and of each entry's `want`.  The tensor may be a
+        view of a buffer that the next step overwrites: use it, or copy it, before then.
 
         Nothing is reserved if the batch does not fit (`CacheFullError`)."""
         if not entries:
@@ -165,6 +230,8 @@ class ModelRunner:
                 self.end_request(request_id)
             raise
         reservations = [self.cache.reserve(request_id, count) for request_id, count in plan]
+        if self.use_graphs and not self.cache.states and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
+            return self._decode_with_graph(reservations, entries)
         batch = build_step_batch(reservations, entries, self.cache, self.device)
         return self.forward(batch)
 
@@ -174,3 +241,61 @@ class ModelRunner:
             self.model.forward_without_logits(batch, self.cells)
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         return self.model.forward(batch, self.cells)
+
+    # ------------------------------------------------------------------ captured decode steps
+
+    @staticmethod
+    def _bucket(value: int) -> int:
+        size = 1
+        while size < value:
+            size *= 2
+        return size
+
+    @torch.inference_mode()
+    def _decode_with_graph(self, reservations: list[Reservation], entries: list[StepEntry]) -> torch.Tensor:
+        """A step of single tokens, one per request, replayed from a HIP graph: the launches
+        of a decode step cost more on the host than the step takes on the device.  Graphs are
+        kept per (requests rounded up to a power of two, block-table width likewise); the
+        step's index arrays go into the graph's static buffer and the same kernels run."""
+        requests = self._bucket(len(reservations))
+        blocks = max(-(-(r.start + 1) // self.cache.page_size) for r in reservations)
+        width = min(self._bucket(blocks), self._bucket(self.cache.max_blocks_per_sequence))
+        key = (requests, width)
+        packed, sizes, widths, facts = _pack_step(reservations, entries, self.cache, pad_to=requests, width=width)
+        graph = self._graphs.get(key)
+        if graph is None:
+            graph = self._capture(key, packed, sizes, widths, facts)
+        turn = graph.turn
+        graph.turn = 1 - turn
+        if graph.copied[turn] is not None:
+            graph.copied[turn].synchronize()  # the staging buffer's last copy has left it
+        graph.host[turn].copy_(torch.from_numpy(packed))
+        graph.static.copy_(graph.host[turn], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        graph.copied[turn] = event
+        graph.graph.replay()
+        return graph.logits[: len(reservations)]
+
+    def _capture(self, key, packed, sizes, widths, facts) -> _DecodeGraph:
+        requests, width = key
+        if len(self._graphs) >= 24:  # keep the newest; each holds only a step's activations
+            self._graphs.pop(next(iter(self._graphs)))
+        static = torch.from_numpy(packed).to(self.device)
+        chunks = [SequenceChunk(f"#{index}", 0, 0, 1) for index in range(requests)]
+        # the widest context these tables can describe decides how the attention splits its keys
+        facts = dict(facts, max_context_length=width * self.cache.page_size)
+        batch = _view_step(static, sizes, widths, facts, chunks, self.cache.page_size)
+        stream = torch.cuda.Stream(self.device)
+        stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(stream):
+            self.model.forward(batch, self.cells)  # loads libraries, builds the work lists kept on `batch`
+        torch.cuda.current_stream(self.device).wait_stream(stream)
+        torch.cuda.synchronize(self.device)
+        captured = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(captured):
+            logits = self.model.forward(batch, self.cells)
+        host = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        graph = _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)
+        self._graphs[key] = graph
+        return graph

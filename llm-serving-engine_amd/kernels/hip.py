@@ -73,13 +73,16 @@ class GatedLinearWeights:
 
 
 class HipKernels:
-    def __init__(self, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0") -> None:
+    def __init__(
+        self, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0", *, library_products: bool = True
+    ) -> None:
         if dtype not in (torch.bfloat16, torch.float32):
             raise KernelError(f"run dtype must be bfloat16 or float32, not {dtype}")
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine runs on an MI355X only and has no CPU path")
         self.dtype = dtype
         self.device = torch.device(device)
+        self.library_products = library_products
         name = torch.cuda.get_device_properties(self.device).gcnArchName
         if not name.startswith("gfx950"):
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
@@ -181,12 +184,28 @@ class HipKernels:
             and weights.in_features % 32 == 0
         )
 
+    def _library(self, x: torch.Tensor, weights: LinearWeights) -> bool:
+        """Whether the product goes to the BLAS library (hipBLASLt through torch), as the
+        reference's products go to its BLAS through nn.Linear: bfloat16 with more rows than
+        the weight-streaming kernel takes."""
+        return (
+            self.library_products
+            and x.dtype == torch.bfloat16
+            and weights.weight.dtype == torch.bfloat16
+            and x.shape[0] > 64
+        )
+
     def linear(self, x: torch.Tensor, weights: LinearWeights, out_dtype: torch.dtype | None = None) -> torch.Tensor:
         rows, inner = x.shape
         if inner != weights.in_features:
             raise KernelError(f"linear: x has {inner} columns, the weight {weights.in_features}")
-        out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
         bias = weights.bias
+        if self._library(x, weights):
+            out = torch.nn.functional.linear(x, weights.weight, bias if bias is None or bias.dtype == x.dtype else None)
+            if bias is not None and bias.dtype != x.dtype:
+                out = out.float() + bias
+            return out.to(out_dtype or self.dtype)
+        out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
         bias_is_float = _is_float(bias) if bias is not None else 0
         if self._skinny(x, weights):
             status = self._gemm_bf16.llmserve_gemm_skinny(
@@ -210,9 +229,9 @@ class HipKernels:
             )
             _check(status, "gated_linear")
             return out
-        both = self.linear(x, weights.both, out_dtype=torch.float32)
+        both = self.linear(x, weights.both, out_dtype=torch.bfloat16 if self._library(x, weights.both) else torch.float32)
         status = self._elementwise.llmserve_silu_mul(
-            _pointer(both), _pointer(out), _is_float(out), x.shape[0], weights.width, self._stream
+            _pointer(both), _is_float(both), _pointer(out), _is_float(out), x.shape[0], weights.width, self._stream
         )
         _check(status, "silu_mul")
         return out

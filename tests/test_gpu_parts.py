@@ -1,0 +1,221 @@
+"""Each part of a layer alone on the GPU against the plain functions, the toy architecture
+with a mixer that has state of its own, and generation through the entry points."""
+
+from __future__ import annotations
+
+import asyncio
+import json
+import math
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from llmserve_amd import CacheConfig, EngineCore, GenerationConfig, LLMEngine, ModelRunner, SchedulerConfig, StepEntry
+from llmserve_amd.parts import (
+    BLOCKS, FEED_FORWARDS, MIXERS, NORMS, AttentionSpec, GatedMLPSpec, PreNormBlockSpec, RMSNormSpec, RotarySpec,
+)
+from llmserve_amd.weights import load_model_folder, random_tensor
+from tests import toy
+from tests.gpu_helpers import ROOT
+from tests.plain import qwen2_plain as plain
+from tests.test_gpu_kernels import paged_case
+from tests.tiny import CONFIGS, random_tokens
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+TOLERANCE = {torch.float32: dict(atol=3e-5, rtol=1e-4), torch.bfloat16: dict(atol=3e-2, rtol=3e-2)}
+
+
+@pytest.fixture(scope="module")
+def kernels():
+    from llmserve_amd.kernels import HipKernels
+
+    return {dtype: HipKernels(dtype) for dtype in DTYPES}
+
+
+def draw(registry, spec, dtype, seed=1, **scales):
+    """Random tensors of a part: what the kernel gets (on the GPU) and what the plain function gets."""
+    on_gpu, exact = {}, {}
+    for name, tensor_spec in registry.tensors(spec).items():
+        value = random_tensor(name, tensor_spec, seed, std=0.08, norm_std=0.2, **scales).to(dtype)
+        on_gpu[name] = value.cuda()
+        exact[name] = value.double()
+    return on_gpu, exact
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_part(kernels, dtype):
+    spec = RMSNormSpec(136, 3e-4)
+    tensors, exact = draw(NORMS, spec, dtype)
+    part = NORMS.build(spec, tensors, kernels[dtype])
+    hidden, delta = torch.randn(5, 136), torch.randn(5, 136)
+    device_hidden = hidden.cuda()
+    out = part.forward(device_hidden, delta.cuda())
+    expected = plain.rms_norm((hidden + delta).double(), exact["weight"], 3e-4)
+    torch.testing.assert_close(out.cpu().double(), expected, **TOLERANCE[dtype])
+    torch.testing.assert_close(device_hidden.cpu(), hidden + delta)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_feed_forward_part(kernels, dtype):
+    spec = GatedMLPSpec(96, 208)
+    tensors, exact = draw(FEED_FORWARDS, spec, dtype)
+    part = FEED_FORWARDS.build(spec, tensors, kernels[dtype])
+    for rows in (3, 80):  # the decoding kernel and the one for long portions
+        x = torch.randn(rows, 96).to(dtype)
+        out = part.forward(x.cuda(), None)
+        assert out.dtype == torch.float32
+        expected = plain.swiglu(x.double(), exact["gate_proj.weight"], exact["up_proj.weight"], exact["down_proj.weight"])
+        torch.testing.assert_close(out.cpu().double(), expected, **TOLERANCE[dtype])
+
+
+def attention_reference(spec, exact, xs, pairing, theta):
+    outs = []
+    config = plain.PlainConfig(
+        vocab_size=1, hidden_size=spec.hidden_size, intermediate_size=1, num_layers=1, num_heads=spec.num_heads,
+        num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim, rope_theta=theta, rms_norm_eps=0.0,
+        attention_bias=spec.qkv_bias, tie_word_embeddings=True, rope_pairing=pairing,
+    )
+    for x in xs:
+        outs.append(plain.attention_layer(x, exact, "", config, torch.arange(x.shape[0]), spec.window))
+    return outs
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,window,pairing", [(6, 2, 32, None, "half"), (5, 1, 48, 9, "adjacent"), (4, 4, 64, None, "adjacent")])
+def test_attention_part(kernels, dtype, heads, kv_heads, dim, window, pairing):
+    hidden, page, theta = 72, 8, 3000.0
+    spec = AttentionSpec(hidden, heads, kv_heads, dim, 1 / math.sqrt(dim), RotarySpec(dim, theta, pairing), True, False, window)
+    tensors, exact = draw(MIXERS, spec, dtype, bias_std=0.1)
+    part = MIXERS.build(spec, tensors, kernels[dtype])
+    lengths = [21, 40, 1]
+    xs = [torch.randn(n, hidden).to(dtype) for n in lengths]
+    expected = attention_reference(spec, exact, [x.double() for x in xs], pairing, theta)
+    # first everything but each request's last three tokens, then those three: the second call reads the cache
+    batch, cell, _, _ = paged_case(lengths, lengths, heads, kv_heads, dim, page, dtype)
+    cell.keys.zero_()
+    cell.values.zero_()
+    whole = part.forward(torch.cat(xs).cuda(), batch, cell)
+    torch.testing.assert_close(whole.cpu().double(), torch.cat(expected), **TOLERANCE[dtype])
+    counts = [min(3, n) for n in lengths]
+    tail_batch, _, _, _ = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype)
+    tail = part.forward(torch.cat([x[-c:] for x, c in zip(xs, counts)]).cuda(), tail_batch, cell)
+    torch.testing.assert_close(tail.cpu().double(), torch.cat([e[-c:] for e, c in zip(expected, counts)]), **TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_block_part(kernels, dtype):
+    hidden, heads, kv_heads, dim, page = 64, 4, 2, 16, 16
+    norm = RMSNormSpec(hidden, 1e-5)
+    attention = AttentionSpec(hidden, heads, kv_heads, dim, 0.25, RotarySpec(dim, 10000.0, "adjacent"))
+    spec = PreNormBlockSpec(norm, attention, norm, GatedMLPSpec(hidden, 96))
+    tensors, exact = draw(BLOCKS, spec, dtype)
+    part = BLOCKS.build(spec, tensors, kernels[dtype])
+    lengths = [33, 6]
+    batch, cell, _, _ = paged_case(lengths, lengths, heads, kv_heads, dim, page, dtype)
+    h = [torch.randn(n, hidden) for n in lengths]
+    device_hidden = torch.cat(h).cuda()
+    delta = part.forward(device_hidden, None, batch, cell)
+    config = plain.PlainConfig(1, hidden, 96, 1, heads, kv_heads, dim, 10000.0, 1e-5, True, True, "adjacent")
+    weights = {"layers.0." + name: value for name, value in exact.items()}
+    expected = torch.cat([plain.decoder_layer(x.double(), weights, 0, config, torch.arange(x.shape[0])) for x in h])
+    torch.testing.assert_close((device_hidden + delta).cpu().double(), expected, **TOLERANCE[dtype])
+
+
+def test_toy_architecture_on_the_gpu(tmp_path, kernels):
+    toy.register_toy()
+    try:
+        folder = toy.write_toy_folder(tmp_path / "toy")
+        loaded = load_model_folder(folder, "float32")
+        runner = ModelRunner(loaded, kernels[torch.float32], CacheConfig(block_size=4, num_blocks=40, max_sequences=3))
+        tokens = random_tokens(30, toy.TOY.vocab_size, seed=8)
+        expected = toy.plain_toy_forward(folder, tokens)
+        rows, at = [], 0
+        for count in (7, 1, 1, 2, 19):
+            rows.append(runner.step([StepEntry("t", tokens[at : at + count], range(count))], create_missing=True).clone())
+            at += count
+        torch.testing.assert_close(torch.cat(rows).cpu().double(), expected, atol=2e-5, rtol=1e-4)
+    finally:
+        toy.unregister_toy()
+
+
+# ------------------------------------------------------------------------------- entry points
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(model_folders, dtype):
+    name = "B"
+    config, page = CONFIGS[name]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders[name]), plain.read_weights(model_folders[name])
+    prompts = [random_tokens(n, config.vocab_size, seed=n) for n in (2, 9, 23, 40, 64, 100)]
+    expected = [plain.generate(weights, plain_config, prompt, 12) for prompt in prompts]
+
+    async def run():
+        async with LLMEngine(str(model_folders[name]), cache_config=CacheConfig(page, 96, 8),
+                             scheduler_config=SchedulerConfig(4, 64), prefill_chunk_size=16, dtype=dtype) as engine:
+            streamed = [[] for _ in prompts]
+            outputs = await asyncio.gather(*[
+                engine.generate(prompt, GenerationConfig(max_new_tokens=12), streamed[index].append)
+                for index, prompt in enumerate(prompts)
+            ])
+            assert engine.cache.used_pages == 0
+            engine.runner.close()
+            return outputs, streamed
+
+    outputs, streamed = asyncio.run(run())
+    assert streamed == outputs
+    if dtype == "float32":
+        assert outputs == expected
+    else:  # bfloat16 may turn a near-tie; the tokens before the first such turn must agree
+        agreeing = sum(a == b for got, want in zip(outputs, expected) for a, b in zip(got, want))
+        assert agreeing >= 0.8 * 12 * len(prompts), (outputs, expected)
+
+
+def test_sampled_generation_is_the_plain_decoders(model_folders):
+    config, page = CONFIGS["B"]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders["B"]), plain.read_weights(model_folders["B"])
+    prompts = [random_tokens(n, config.vocab_size, seed=50 + n) for n in (9, 40)]
+    settings = [GenerationConfig(12, 0.8, 1.0, seed=5), GenerationConfig(12, 0.8, 0.9, seed=6)]
+    expected = [plain.generate(weights, plain_config, p, 12, s.temperature, s.top_p, s.seed) for p, s in zip(prompts, settings)]
+    from llmserve_amd.kernels import HipKernels
+
+    loaded = load_model_folder(model_folders["B"], "float32")
+    runner = ModelRunner(loaded, HipKernels(torch.float32), CacheConfig(page, 64, 4))
+    assert EngineCore(runner, SchedulerConfig(2, 64), prefill_chunk_size=16).generate(prompts, settings) == expected
+    runner.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(model_folders, dtype):
+    """300 tokens decoded one by one after a one-token prompt (the first tokens of a sequence,
+    then many captured steps, page after page), each step's logits against the plain forward."""
+    config, page = CONFIGS["A"]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders["A"]), plain.read_weights(model_folders["A"])
+    tokens = random_tokens(300, config.vocab_size, seed=4)
+    expected = plain.forward(weights, plain_config, tokens)
+    from llmserve_amd.kernels import HipKernels
+
+    loaded = load_model_folder(model_folders["A"], dtype)
+    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(page, 24, 2))
+    rows = [runner.step([StepEntry("r", [token], [0])], create_missing=True).clone() for token in tokens]
+    tolerance = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=4e-2, rtol=4e-2)
+    torch.testing.assert_close(torch.cat(rows).cpu().double(), expected, **tolerance)
+    runner.close()
+
+
+def test_command_line_generates(model_folders, tmp_path):
+    common = ["--model", str(model_folders["A"]), "--dtype", "float32", "--block-size", "16", "--num-blocks", "64"]
+    done = subprocess.run([sys.executable, str(ROOT / "bin" / "llmserve"), "generate", "--prompt-tokens", "5,17,3,200",
+                           "--max-tokens", "6", *common], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders["A"]), plain.read_weights(model_folders["A"])
+    assert json.loads(done.stdout.strip().splitlines()[-1])["token_ids"] == plain.generate(weights, plain_config, [5, 17, 3, 200], 6)
+    output = tmp_path / "bench.json"
+    done = subprocess.run([sys.executable, str(ROOT / "bin" / "llmserve"), "benchmark", "--config", "continuous",
+                           "--requests", "6", "--arrival-rate", "200", "--batch-size", "4", "--output", str(output),
+                           *common, "--num-blocks", "512"], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    summary = json.loads(output.read_text())["summary"]
+    assert summary["successful_requests"] == 6 and summary["throughput_tokens_per_s"] > 0

@@ -1,0 +1,67 @@
+"""A toy mixer with state of its own, and a toy architecture around it, are registered,
+built and stepped without a change to the framework's files (here with the torch stand-in
+for the kernels; tests/test_gpu_parts.py does the same on the GPU)."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from llmserve_amd import CacheConfig, ModelRunner, StepEntry
+from llmserve_amd.parts import FixedState, PagedKeyValue
+from llmserve_amd.weights import load_model_folder
+from tests import toy
+from tests.tiny import random_tokens
+from tests.torch_kernels import TorchKernels
+
+
+@pytest.fixture()
+def toy_folder(tmp_path):
+    toy.register_toy()
+    yield toy.write_toy_folder(tmp_path / "toy")
+    toy.unregister_toy()
+
+
+def test_toy_architecture_steps_like_its_plain_forward(toy_folder):
+    loaded = load_model_folder(toy_folder, "float32")
+    assert loaded.architecture.name == "ToyStateForCausalLM"
+    runner = ModelRunner(loaded, TorchKernels(torch.float32), CacheConfig(block_size=4, num_blocks=40, max_sequences=3))
+    cache = runner.cache
+    # two state cells (layer 0 runs twice), two paged groups (rotated and unrotated attention need the same pages:
+    # one group), the last run owns nothing and reads run 1's pages
+    assert [type(cell.need) for cell in runner.cells] == [FixedState, PagedKeyValue, PagedKeyValue, FixedState, PagedKeyValue]
+    assert len(cache.states) == 2 and len(cache.groups) == 1 and cache.groups[0].cells == [1, 2]
+    assert runner.cells[4].keys.data_ptr() == runner.cells[1].keys.data_ptr() and not runner.cells[4].writable
+
+    prompts = {name: random_tokens(n, toy.TOY.vocab_size, seed=n) for name, n in (("a", 37), ("b", 9), ("c", 22))}
+    expected = {name: toy.plain_toy_forward(toy_folder, tokens) for name, tokens in prompts.items()}
+    got = {name: [] for name in prompts}
+    fed = {name: 0 for name in prompts}
+    sizes = {"a": [5, 1, 1, 9, 2, 19], "b": [2, 7], "c": [1, 1, 1, 1, 18]}
+    for turn in range(6):
+        entries = []
+        for name, tokens in prompts.items():
+            if turn < len(sizes[name]):
+                count = sizes[name][turn]
+                entries.append(StepEntry(name, tokens[fed[name] : fed[name] + count], range(count)))
+                fed[name] += count
+        logits = runner.step(entries, create_missing=True)
+        at = 0
+        for entry in entries:
+            got[entry.request_id].append(logits[at : at + len(entry.tokens)])
+            at += len(entry.tokens)
+    for name in prompts:
+        torch.testing.assert_close(torch.cat(got[name]).double(), expected[name], atol=1e-5, rtol=1e-5)
+    # a freed slot's state is zeroed for the next request
+    runner.end_request("b")
+    again = runner.step([StepEntry("b2", prompts["b"], range(9))], create_missing=True)
+    torch.testing.assert_close(again.double(), expected["b"], atol=1e-5, rtol=1e-5)
+    cache.check_invariants()
+
+
+def test_unregistered_parts_are_refused(tmp_path):
+    toy.register_toy()
+    folder = toy.write_toy_folder(tmp_path / "toy")
+    toy.unregister_toy()
+    with pytest.raises(Exception, match="ToyStateForCausalLM"):
+        load_model_folder(folder, "float32")

@@ -1,0 +1,195 @@
+"""A toy architecture defined entirely in the tests, to show that parts and whole
+architectures are added by registering them, without a change to the framework's files:
+
+- a mixer with state of its own (a decaying sum per request, a fixed-size state slot),
+- beside attention layers, chosen layer by layer,
+- a run order that names one layer twice, and a run that reads another run's cache.
+
+It is never a model of anyone's: it exists to exercise the interfaces."""
+
+from __future__ import annotations
+
+import json
+import math
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Any, ClassVar
+
+import torch
+
+from llmserve_amd.config.model import ArchitectureConfig, KeyReader
+from llmserve_amd.parts import (
+    MIXERS, AttentionSpec, FixedState, GatedMLPSpec, LayerDefinition, LayerRun, Mixer, ModelSpec, NoPositionSpec,
+    PreNormBlockSpec, RMSNormSpec, RotarySpec, TensorSpec,
+)
+from llmserve_amd.registry import register_architecture, unregister_architecture
+
+
+@dataclass(frozen=True)
+class DecaySpec:
+    hidden_size: int
+    state_size: int
+    decay: float
+    kind: str = "toy_decay"
+
+
+class DecayMixer(Mixer):
+    """state <- decay * state + x W_in;  out = state W_out, token after token in order.
+    The state of a request lives in its slot of the cell, across steps."""
+
+    @classmethod
+    def tensors(cls, spec: DecaySpec) -> dict[str, TensorSpec]:
+        return {
+            "in_proj.weight": TensorSpec((spec.state_size, spec.hidden_size)),
+            "out_proj.weight": TensorSpec((spec.hidden_size, spec.state_size)),
+        }
+
+    @classmethod
+    def cache_need(cls, spec: DecaySpec) -> FixedState:
+        return FixedState((spec.state_size,))
+
+    def __init__(self, spec: DecaySpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.w_in = tensors["in_proj.weight"].float()
+        self.w_out = tensors["out_proj.weight"].float()
+
+    def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
+        pushed = x.float() @ self.w_in.T  # [T, state]
+        out = torch.empty(x.shape[0], self.spec.hidden_size, dtype=torch.float32, device=x.device)
+        row = 0
+        for chunk in batch.chunks:
+            state = cell.state[chunk.slot]
+            for _ in range(chunk.count):
+                state = self.spec.decay * state + pushed[row]
+                out[row] = state @ self.w_out.T
+                row += 1
+            if cell.writable:
+                cell.state[chunk.slot] = state
+        return out
+
+
+@dataclass(frozen=True)
+class ToyConfig(ArchitectureConfig):
+    architecture: ClassVar[str] = "ToyStateForCausalLM"
+    vocab_size: int = 0
+    hidden_size: int = 0
+    state_size: int = 0
+    decay: float = 0.0
+    num_heads: int = 0
+    head_dim: int = 0
+    ffn_size: int = 0
+    eps: float = 0.0
+    max_length: int = 0
+
+    @classmethod
+    def from_dict(cls, values: dict[str, Any]) -> "ToyConfig":
+        reader = KeyReader(values, "toy config")
+        return cls(
+            vocab_size=reader.integer("vocab_size"), hidden_size=reader.integer("hidden_size"),
+            state_size=reader.integer("state_size"), decay=reader.number("decay"),
+            num_heads=reader.integer("num_heads"), head_dim=reader.integer("head_dim"),
+            ffn_size=reader.integer("ffn_size"), eps=reader.number("eps"), max_length=reader.integer("max_length"),
+        )
+
+    @property
+    def max_position_embeddings(self) -> int:
+        return self.max_length
+
+    def to_config_json(self) -> dict[str, Any]:
+        return {"architectures": [self.architecture], **self.to_dict()}
+
+
+def toy_spec(config: ToyConfig) -> ModelSpec:
+    norm = RMSNormSpec(config.hidden_size, config.eps)
+    ffn = GatedMLPSpec(config.hidden_size, config.ffn_size)
+    decay = DecaySpec(config.hidden_size, config.state_size, config.decay)
+    attention = AttentionSpec(
+        config.hidden_size, config.num_heads, config.num_heads, config.head_dim, 1.0 / math.sqrt(config.head_dim),
+        RotarySpec(config.head_dim, 100.0, "half"), qkv_bias=False,
+    )
+    unrotated = AttentionSpec(
+        config.hidden_size, config.num_heads, config.num_heads, config.head_dim, 1.0 / math.sqrt(config.head_dim),
+        NoPositionSpec(), qkv_bias=False,
+    )
+    layers = (
+        LayerDefinition("layers.0.", PreNormBlockSpec(norm, decay, norm, ffn, mixer_name="mixer.")),
+        LayerDefinition("layers.1.", PreNormBlockSpec(norm, attention, norm, ffn, mixer_name="mixer.")),
+        LayerDefinition("layers.2.", PreNormBlockSpec(norm, unrotated, norm, ffn, mixer_name="mixer.")),
+    )
+    # layer 0 runs twice (two state cells), layer 1 runs twice, its second run reading the first's pages
+    run_order = (LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(0), LayerRun(1, reads=1))
+    return ModelSpec(
+        config.vocab_size, config.hidden_size, layers, run_order, norm, tie_embeddings=True,
+        embedding_name="embed.weight", final_norm_name="final_norm.",
+    )
+
+
+TOY = ToyConfig(vocab_size=97, hidden_size=48, state_size=20, decay=0.8, num_heads=3, head_dim=16, ffn_size=64,
+                eps=1e-5, max_length=256)
+
+
+def register_toy() -> None:
+    MIXERS.register("toy_decay")(DecayMixer)
+    register_architecture("ToyStateForCausalLM", ToyConfig, toy_spec)
+
+
+def unregister_toy() -> None:
+    MIXERS.unregister("toy_decay")
+    unregister_architecture("ToyStateForCausalLM")
+
+
+def write_toy_folder(folder: Path, seed: int = 3) -> Path:
+    from llmserve_amd.weights import write_model_folder
+
+    return write_model_folder(folder, TOY, seed, dtype=torch.float32, std=0.1, norm_std=0.1)
+
+
+# ----------------------------------------------------------------------------- the toy's own plain forward
+
+
+def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
+    """Whole sequence, no cache, float64; written apart from the parts above."""
+    from safetensors.torch import load_file
+
+    from tests.plain import qwen2_plain as plain
+
+    config = json.loads((folder / "config.json").read_text())
+    w = {name: value.double() for name, value in load_file(str(folder / "model.safetensors")).items()}
+    eps, dim, heads = config["eps"], config["head_dim"], config["num_heads"]
+    h = w["embed.weight"][tokens]
+    length = len(tokens)
+
+    def ffn(x, prefix):
+        return plain.swiglu(x, w[prefix + "mlp.gate_proj.weight"], w[prefix + "mlp.up_proj.weight"], w[prefix + "mlp.down_proj.weight"])
+
+    def decay_layer(h, prefix):
+        x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
+        state = torch.zeros(config["state_size"], dtype=torch.float64)
+        out = []
+        for t in range(length):
+            state = config["decay"] * state + w[prefix + "mixer.in_proj.weight"] @ x[t]
+            out.append(w[prefix + "mixer.out_proj.weight"] @ state)
+        h = h + torch.stack(out)
+        return h + ffn(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
+
+    def attention_layer(h, prefix, rotate, shared=None):
+        x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
+        q = (x @ w[prefix + "mixer.q_proj.weight"].T).view(length, heads, dim)
+        k = (x @ w[prefix + "mixer.k_proj.weight"].T).view(length, heads, dim)
+        v = (x @ w[prefix + "mixer.v_proj.weight"].T).view(length, heads, dim)
+        if rotate:
+            angles = plain.rope_angles(dim, 100.0, torch.arange(length))
+            q, k = plain.rope_half(q, angles), plain.rope_half(k, angles)
+        if shared is not None:
+            k, v = shared  # the run reads the keys and values another run stored
+        mixed = plain.causal_attention(q, k, v, 1.0 / math.sqrt(dim)).reshape(length, -1)
+        h = h + mixed @ w[prefix + "mixer.o_proj.weight"].T
+        h = h + ffn(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
+        return h, (k, v)
+
+    h = decay_layer(h, "layers.0.")
+    h, stored = attention_layer(h, "layers.1.", True)
+    h, _ = attention_layer(h, "layers.2.", False)
+    h = decay_layer(h, "layers.0.")
+    h, _ = attention_layer(h, "layers.1.", True, shared=stored)
+    return plain.rms_norm(h, w["final_norm.weight"], eps) @ w["embed.weight"].T
