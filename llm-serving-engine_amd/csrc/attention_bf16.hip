@@ -17,6 +17,11 @@
 // and a second kernel merges them (for few long requests).  A wave may carry several column
 // tiles (COLUMN_TILES) through the same keys, which divides the cache traffic of a long
 // prompt portion by as much.
+// When every request of the step brings one token (FUSED), the kernel also does what comes
+// before and after it in a decode step: it rotates the queries in registers, the workgroup
+// that owns the newest key rotates that key and stores key and value in their page first,
+// and with `splits` > 1 the workgroup that finishes last (a counter per tile tells) merges
+// the splits, in split order, instead of a second kernel.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -65,14 +70,28 @@ __device__ __forceinline__ f32x4 mfma_qk(const QkOperand& a, const QkOperand& b,
 }
 
 // work[tile] = {request index in the step, first token row, tokens in the tile, unused}
-template <int COLUMN_TILES>
+// pairing: 0 none, 1 adjacent pairs (2j, 2j+1), 2 half pairs (j, j + D/2)
+__device__ __forceinline__ void rotate_pair(float& a, float& b, float2 cos_sin) {
+  const float x = a * cos_sin.x - b * cos_sin.y, y = b * cos_sin.x + a * cos_sin.y;
+  a = x;
+  b = y;
+}
+
+struct FusedDecode {          // what the kernel needs to rotate and store; unused unless FUSED
+  const float2* table;        // [rows][D / 2] (cos, sin) of each token's angles, or null
+  int pairing;
+  const int* slots;           // [rows] page * page_size + offset of each token, negative: store nothing
+};
+
+template <int COLUMN_TILES, bool FUSED>
 __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
     const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
-    float* __restrict__ partial_ml, const bf16_t* __restrict__ keys, const bf16_t* __restrict__ values,
-    const int* __restrict__ block_tables, int table_width, const int* __restrict__ positions,
-    const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile, int page_size, float scale,
-    int window, int splits) {
+    float* __restrict__ partial_ml, int* __restrict__ counters, bf16_t* __restrict__ keys,
+    bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
+    const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
+    int page_size, float scale, int window, int splits, FusedDecode fused) {
   extern __shared__ float lds[];  // [WAVES][16 columns][D + 2]
+  __shared__ int ticket;
   const int group = heads / kv_heads;
   const int kv_head = blockIdx.y % kv_heads, head_tile = blockIdx.y / kv_heads;
   const int heads_here = min(group - head_tile * 16, 16);
@@ -100,6 +119,32 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
     const bf16_t* q_row = qkv + (size_t)(row0 + safe) * row_width + (size_t)head * D;
 #pragma unroll
     for (int s = 0; s < QK_STEPS; ++s) query[t][s] = load_qk(q_row, s, q);
+#if HEAD_DIM % 32 == 0
+    if (FUSED && fused.pairing != 0) {  // the queries come unrotated: rotate them here, in float32
+      const float2* angles = fused.table + (size_t)(row0 + safe) * (D / 2);
+      if (fused.pairing == 1) {
+#pragma unroll
+        for (int s = 0; s < QK_STEPS; ++s)
+#pragma unroll
+          for (int pair = 0; pair < 4; ++pair) {
+            float a = (float)query[t][s].v[2 * pair], b = (float)query[t][s].v[2 * pair + 1];
+            rotate_pair(a, b, angles[(s * 32 + q * 8) / 2 + pair]);
+            query[t][s].v[2 * pair] = (bf16_t)a;
+            query[t][s].v[2 * pair + 1] = (bf16_t)b;
+          }
+      } else {  // the partner of dim d is d + D/2: the same lane, QK_STEPS / 2 steps on (D % 64 == 0)
+#pragma unroll
+        for (int s = 0; s < QK_STEPS / 2; ++s)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            float a = (float)query[t][s].v[i], b = (float)query[t][s + QK_STEPS / 2].v[i];
+            rotate_pair(a, b, angles[s * 32 + q * 8 + i]);
+            query[t][s].v[i] = (bf16_t)a;
+            query[t][s + QK_STEPS / 2].v[i] = (bf16_t)b;
+          }
+      }
+    }
+#endif
   }
 
   float running_max[COLUMN_TILES], running_sum[COLUMN_TILES];
@@ -118,6 +163,29 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
   const int step_end = min(step_last + 1, step_begin + per_split);
   const size_t page_stride = (size_t)kv_heads * page_size * D;
   const size_t head_offset = (size_t)kv_head * page_size * D;
+
+  if (FUSED && step_last >= step_begin && step_last < step_end) {
+    // this workgroup reads the newest key: it stores it first (one token per tile when FUSED; with
+    // more than 16 query heads per kv head several workgroups store the same values)
+    const int slot = fused.slots[row0];
+    if (slot >= 0 && wave == 0) {
+      const bf16_t* k_row = qkv + (size_t)row0 * row_width + (size_t)(heads + kv_head) * D;
+      const bf16_t* v_row = k_row + (size_t)kv_heads * D;
+      bf16_t* k_page = keys + (size_t)(slot / page_size) * page_stride + head_offset + (size_t)(slot % page_size) * D;
+      bf16_t* v_page = values + (size_t)(slot / page_size) * page_stride + head_offset + slot % page_size;
+      const float2* angles = fused.table + (size_t)row0 * (D / 2);
+      for (int j = lane; j < D / 2; j += WAVE) {
+        const int ia = fused.pairing == 2 ? j : 2 * j, ib = fused.pairing == 2 ? j + D / 2 : 2 * j + 1;
+        float a = (float)k_row[ia], b = (float)k_row[ib];
+        if (fused.pairing != 0) rotate_pair(a, b, angles[j]);
+        k_page[ia] = (bf16_t)a;
+        k_page[ib] = (bf16_t)b;
+      }
+      for (int d = lane; d < D; d += WAVE) v_page[(size_t)d * page_size] = v_row[d];
+      __threadfence();
+    }
+    __syncthreads();
+  }
 
   for (int step = step_begin + wave; step < step_end; step += WAVES) {
     const int key0 = step * KEYS;
@@ -268,80 +336,113 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
     }
     __syncthreads();
   }
-}
+  if (splits == 1) return;
 
-// out[row, head] = sum_s acc_s * exp(m_s - m) / sum_s l_s * exp(m_s - m)
-__global__ void attention_merge_kernel(const float* __restrict__ partial_acc, const float* __restrict__ partial_ml,
-                                       bf16_t* __restrict__ out, int splits) {
-  const size_t pair = blockIdx.x;  // row * heads + head
-  const float* ml = partial_ml + pair * splits * 2;
-  float best = -INFINITY;
-  for (int s = 0; s < splits; ++s) best = fmaxf(best, ml[2 * s]);
-  float total = 0.f;
-  for (int s = 0; s < splits; ++s) total += ml[2 * s] == -INFINITY ? 0.f : ml[2 * s + 1] * __expf(ml[2 * s] - best);
-  const float inverse = total > 0.f ? 1.f / total : 0.f;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float sum = 0.f;
-    for (int s = 0; s < splits; ++s)
-      if (ml[2 * s] != -INFINITY) sum += partial_acc[(pair * splits + s) * D + d] * __expf(ml[2 * s] - best);
-    out[pair * D + d] = (bf16_t)(sum * inverse);
+  // The workgroup that finishes last merges the splits of its tile, in split order:
+  // out = sum_s acc_s * exp(m_s - m) / sum_s l_s * exp(m_s - m).  The counter returns to zero.
+  __threadfence();
+  __syncthreads();
+  int* counter = counters + (size_t)blockIdx.x * gridDim.y + blockIdx.y;
+  if (threadIdx.x == 0) ticket = atomicAdd(counter, 1);
+  __syncthreads();
+  if (ticket != splits - 1) return;
+  __threadfence();
+  for (int index = threadIdx.x; index < COLUMN_TILES * 16 * (D / 4); index += WAVES * 64) {
+    const int t = index / (16 * (D / 4)), rest = index % (16 * (D / 4));
+    const int column = rest / (D / 4), d4 = (rest % (D / 4)) * 4;
+    const int token = t * tokens_per_tile + column / heads_here;
+    if (token >= tokens || column / heads_here >= tokens_per_tile) continue;
+    const int head = kv_head * group + head_tile * 16 + column % heads_here;
+    const size_t pair = ((size_t)row0 + token) * heads + head;
+    const float* ml = partial_ml + pair * splits * 2;
+    float best = -INFINITY;
+    for (int sp = 0; sp < splits; ++sp) best = fmaxf(best, ml[2 * sp]);
+    float total = 0.f;
+    f32x4 merged = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < splits; ++sp) {
+      if (ml[2 * sp] == -INFINITY) continue;
+      const float factor = __expf(ml[2 * sp] - best);
+      total += ml[2 * sp + 1] * factor;
+      const float* theirs = partial_acc + (pair * splits + sp) * D + d4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) merged[i] += theirs[i] * factor;
+    }
+    const float inverse = total > 0.f ? 1.f / total : 0.f;
+    bf16_t* dst = out + pair * D + d4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
   }
+  if (threadIdx.x == 0) *counter = 0;
 }
 
-template <int COLUMN_TILES>
+template <int COLUMN_TILES, bool FUSED>
 static int launch_tiles(const void* qkv, int row_width, void* out, float* partial_acc, float* partial_ml,
-                        const void* keys, const void* values, const int* block_tables, int table_width,
+                        int* counters, void* keys, void* values, const int* block_tables, int table_width,
                         const int* positions, const int* work, int tiles, int heads, int kv_heads,
-                        int tokens_per_tile, int page_size, float scale, int window, int splits, hipStream_t stream) {
+                        int tokens_per_tile, int page_size, float scale, int window, int splits, FusedDecode fused,
+                        hipStream_t stream) {
   const int group = heads / kv_heads;
   const int head_tiles = (group + 15) / 16;
   const size_t shared = (size_t)WAVES * 16 * (D + 2) * sizeof(float);
   if (shared > 64 * 1024) {  // more dynamic LDS than a kernel gets by default: ask for it once
     static bool asked = false;
     if (!asked) {
-      if (hipFuncSetAttribute((const void*)attention_tiles_kernel<COLUMN_TILES>,
+      if (hipFuncSetAttribute((const void*)attention_tiles_kernel<COLUMN_TILES, FUSED>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shared) != hipSuccess)
         return ERR_BAD_ARGUMENT;
       asked = true;
     }
   }
-  hipLaunchKernelGGL(attention_tiles_kernel<COLUMN_TILES>, dim3(tiles, kv_heads * head_tiles, splits),
+  hipLaunchKernelGGL((attention_tiles_kernel<COLUMN_TILES, FUSED>), dim3(tiles, kv_heads * head_tiles, splits),
                      dim3(WAVES * 64), shared, stream, (const bf16_t*)qkv, row_width, (bf16_t*)out, partial_acc,
-                     partial_ml, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width, positions,
-                     work, heads, kv_heads, tokens_per_tile, page_size, scale, window, splits);
+                     partial_ml, counters, (bf16_t*)keys, (bf16_t*)values, block_tables, table_width, positions, work,
+                     heads, kv_heads, tokens_per_tile, page_size, scale, window, splits, fused);
   return LAUNCH_STATUS();
 }
 
 extern "C" int llmserve_attention_head_dim() { return D; }
 
+// Whether the fused decode form can rotate with this pairing at this head size.
+extern "C" int llmserve_attention_can_fuse(int pairing) {
+  if (pairing == 0) return 1;
+  if (D % 32 != 0) return 0;
+  return pairing == 1 || (pairing == 2 && D % 64 == 0);
+}
+
 // `work` holds `tiles` items of four ints; a tile covers `column_tiles * tokens_per_tile`
 // tokens at most, where tokens_per_tile = max(1, 16 / (heads / kv_heads)).  page_size must
-// be a multiple of 4.  With splits > 1, partial_acc is float32 [rows * heads * splits * D]
-// and partial_ml [rows * heads * splits * 2], rows being the step's token count.
+// be a multiple of 4.  With splits > 1, partial_acc is float32 [rows * heads * splits * D],
+// partial_ml [rows * heads * splits * 2] (rows being the step's token count) and counters
+// tiles * kv_heads * ceil(group / 16) ints that are zero before the call and after it.
+// With `fuse` every tile holds one token, qkv is as the projection left it, and the kernel
+// rotates (table of cos and sin per row, pairing) and stores the token's key and value at slots[row] itself.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
-                                        float* partial_ml, const void* keys, const void* values,
+                                        float* partial_ml, int* counters, void* keys, void* values,
                                         const int* block_tables, int table_width, const int* positions,
                                         const int* work, int tiles, int column_tiles, int rows, int heads,
-                                        int kv_heads, int page_size, float scale, int window, int splits,
+                                        int kv_heads, int page_size, float scale, int window, int splits, int fuse,
+                                        const float* table, int pairing, const int* slots,
                                         hipStream_t stream) {
   if (tiles <= 0) return 0;
-  if (heads % kv_heads || page_size % 4 || splits < 1 || (splits > 1 && (!partial_acc || !partial_ml)))
+  if (heads % kv_heads || page_size % 4 || splits < 1 || (splits > 1 && (!partial_acc || !partial_ml || !counters)))
     return ERR_BAD_ARGUMENT;
   const int group = heads / kv_heads;
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
-  int status;
+  FusedDecode fused = {(const float2*)table, pairing, slots};
+  if (fuse) {
+    if (column_tiles != 1 || !slots || !llmserve_attention_can_fuse(pairing) || (pairing != 0 && !table))
+      return ERR_BAD_ARGUMENT;
+    return launch_tiles<1, true>(qkv, row_width, out, partial_acc, partial_ml, counters, keys, values, block_tables,
+                                 table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
+                                 scale, window, splits, fused, stream);
+  }
   if (column_tiles == 1)
-    status = launch_tiles<1>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables, table_width,
-                             positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size, scale, window,
-                             splits, stream);
-  else if (column_tiles == 4)
-    status = launch_tiles<4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables, table_width,
-                             positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size, scale, window,
-                             splits, stream);
-  else
-    return ERR_BAD_ARGUMENT;
-  if (status != 0 || splits == 1) return status;
-  hipLaunchKernelGGL(attention_merge_kernel, dim3(rows * heads), dim3(64), 0, stream, partial_acc, partial_ml,
-                     (bf16_t*)out, splits);
-  return LAUNCH_STATUS();
+    return launch_tiles<1, false>(qkv, row_width, out, partial_acc, partial_ml, counters, keys, values, block_tables,
+                                  table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
+                                  scale, window, splits, fused, stream);
+  if (column_tiles == 4)
+    return launch_tiles<4, false>(qkv, row_width, out, partial_acc, partial_ml, counters, keys, values, block_tables,
+                                  table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
+                                  scale, window, splits, fused, stream);
+  return ERR_BAD_ARGUMENT;
 }

@@ -25,12 +25,14 @@ extern "C" int llmserve_embedding(const void* table, int table_is_float, const i
 }
 
 // ---------------------------------------------------------------------------- add + RMSNorm
-// hidden[t] += delta[t] (if delta); out[t] = hidden[t] * rsqrt(mean(hidden[t]^2) + eps) * weight
-// (reference model.py:20-23, :200-201).  One block per row; the sum of squares is added in
-// an order that depends only on the row length, so a row's result is the same in any batch.
+// hidden[t] += delta[0][t] + delta[1][t] + ... (if delta); out[t] = hidden[t] *
+// rsqrt(mean(hidden[t]^2) + eps) * weight   (reference model.py:20-23, :200-201).
+// `delta` may come as `parts` partial sums [parts, rows, width] (a product split over K leaves
+// them); they are added in order.  One block per row; the sum of squares is added in an order
+// that depends only on the row length, so a row's result is the same in any batch.
 template <typename TO>
-__global__ void add_rms_norm_kernel(float* __restrict__ hidden, const float* __restrict__ delta,
-                                    const void* __restrict__ weight, int weight_is_float,
+__global__ void add_rms_norm_kernel(float* __restrict__ hidden, const float* __restrict__ delta, int parts,
+                                    size_t part_stride, const void* __restrict__ weight, int weight_is_float,
                                     TO* __restrict__ out, int width, float eps) {
   __shared__ float shared[17];
   float* row = hidden + (size_t)blockIdx.x * width;
@@ -39,7 +41,7 @@ __global__ void add_rms_norm_kernel(float* __restrict__ hidden, const float* __r
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = row[i];
     if (add) {
-      v += add[i];
+      for (int p = 0; p < parts; ++p) v += add[p * part_stride + i];
       row[i] = v;
     }
     squares += v * v;
@@ -51,50 +53,144 @@ __global__ void add_rms_norm_kernel(float* __restrict__ hidden, const float* __r
     dst[i] = from_float<TO>(row[i] * scale * load_as_float(weight, weight_is_float, i));
 }
 
-extern "C" int llmserve_add_rms_norm(float* hidden, const float* delta, const void* weight, int weight_is_float,
-                                     void* out, int out_is_float, int rows, int width, float eps,
+// The same for rows of up to 256 * 4 * VECTORS floats whose length is a multiple of 4: the row
+// stays in registers between the two passes and moves in 16-byte pieces.
+#define NORM_VECTORS 8
+template <typename TO>
+__global__ __launch_bounds__(256) void add_rms_norm_vector_kernel(float* __restrict__ hidden,
+                                                                  const float* __restrict__ delta, int parts,
+                                                                  size_t part_stride,
+                                                                  const void* __restrict__ weight,
+                                                                  int weight_is_float, TO* __restrict__ out,
+                                                                  int width, float eps) {
+  __shared__ float shared[17];
+  const int quads = width / 4;
+  float4* row = (float4*)(hidden + (size_t)blockIdx.x * width);
+  const float* add = delta ? delta + (size_t)blockIdx.x * width : nullptr;
+  float4 v[NORM_VECTORS], w[NORM_VECTORS];
+  float squares = 0.f;
+#pragma unroll
+  for (int j = 0; j < NORM_VECTORS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < quads) {
+      v[j] = row[i];
+      if (weight_is_float) {
+        w[j] = ((const float4*)weight)[i];
+      } else {
+        const bf16_t* wb = (const bf16_t*)weight + 4 * i;
+        w[j] = make_float4((float)wb[0], (float)wb[1], (float)wb[2], (float)wb[3]);
+      }
+    }
+  }
+  if (add) {
+    for (int p = 0; p < parts; ++p) {
+      const float4* part = (const float4*)(add + p * part_stride);
+#pragma unroll
+      for (int j = 0; j < NORM_VECTORS; ++j) {
+        const int i = threadIdx.x + j * 256;
+        if (i < quads) {
+          const float4 d = part[i];
+          v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NORM_VECTORS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < quads) {
+      if (add) row[i] = v[j];
+      squares += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    }
+  }
+  const float total = block_sum(squares, shared);
+  const float scale = rsqrtf(total / (float)width + eps);
+  TO* dst = out + (size_t)blockIdx.x * width;
+#pragma unroll
+  for (int j = 0; j < NORM_VECTORS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < quads) {
+      dst[4 * i + 0] = from_float<TO>(v[j].x * scale * w[j].x);
+      dst[4 * i + 1] = from_float<TO>(v[j].y * scale * w[j].y);
+      dst[4 * i + 2] = from_float<TO>(v[j].z * scale * w[j].z);
+      dst[4 * i + 3] = from_float<TO>(v[j].w * scale * w[j].w);
+    }
+  }
+}
+
+extern "C" int llmserve_add_rms_norm(float* hidden, const float* delta, int parts, const void* weight,
+                                     int weight_is_float, void* out, int out_is_float, int rows, int width, float eps,
                                      hipStream_t stream) {
   if (rows <= 0) return 0;
+  if (delta && parts < 1) return ERR_BAD_ARGUMENT;
+  const size_t part_stride = (size_t)rows * width;
+  if (width % 4 == 0 && width <= 256 * 4 * NORM_VECTORS) {
+    if (out_is_float)
+      hipLaunchKernelGGL(add_rms_norm_vector_kernel<float>, dim3(rows), dim3(256), 0, stream, hidden, delta, parts,
+                         part_stride, weight, weight_is_float, (float*)out, width, eps);
+    else
+      hipLaunchKernelGGL(add_rms_norm_vector_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, hidden, delta, parts,
+                         part_stride, weight, weight_is_float, (bf16_t*)out, width, eps);
+    return LAUNCH_STATUS();
+  }
   const int threads = width >= 2048 ? 512 : 256;
   if (out_is_float)
-    hipLaunchKernelGGL(add_rms_norm_kernel<float>, dim3(rows), dim3(threads), 0, stream, hidden, delta, weight,
-                       weight_is_float, (float*)out, width, eps);
+    hipLaunchKernelGGL(add_rms_norm_kernel<float>, dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, weight_is_float, (float*)out, width, eps);
   else
-    hipLaunchKernelGGL(add_rms_norm_kernel<bf16_t>, dim3(rows), dim3(threads), 0, stream, hidden, delta, weight,
-                       weight_is_float, (bf16_t*)out, width, eps);
+    hipLaunchKernelGGL(add_rms_norm_kernel<bf16_t>, dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, weight_is_float, (bf16_t*)out, width, eps);
   return LAUNCH_STATUS();
 }
 
 // ---------------------------------------------------------------------------- rotary + cache write
+// table[t][j] = (cos, sin) of positions[t] * inverse[j], in float32 (reference model.py:29-33
+// builds the same numbers for every position at start-up).  Every layer of a step rotates by the
+// same angles, so they are computed once per step.
+__global__ void rotary_table_kernel(const int* __restrict__ positions, const float* __restrict__ inverse,
+                                    float2* __restrict__ table, int half) {
+  const float position = (float)positions[blockIdx.x];
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    float sine, cosine;
+    sincosf(position * inverse[j], &sine, &cosine);
+    table[(size_t)blockIdx.x * half + j] = make_float2(cosine, sine);
+  }
+}
+
+extern "C" int llmserve_rotary_table(const int* positions, const float* inverse, float* table, int tokens, int half,
+                                     hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  hipLaunchKernelGGL(rotary_table_kernel, dim3(tokens), dim3(64), 0, stream, positions, inverse, (float2*)table, half);
+  return LAUNCH_STATUS();
+}
+
 // A token's row of qkv is [q heads | k heads | v heads], each head `dim` wide.  q and k heads
-// are rotated in place by the token's position (reference model.py:35-43): the pair (a, b)
-// becomes (a cos - b sin, b cos + a sin) with angle = position * inverse[j], all in float32.
+// are rotated in place by the token's angles (reference model.py:35-43): the pair (a, b)
+// becomes (a cos - b sin, b cos + a sin), all in float32.
 // pairing 0: none, 1: adjacent pairs (2j, 2j+1), 2: half pairs (j, j + dim/2).
 // k (after rotation) and v are then written to the pages: slot = page * page_size + offset,
 // key pages laid out [page, kv_head, offset, dim], value pages transposed [page, kv_head,
-// dim, offset] (reference kv_cache.py:249-266 writes both as [page, offset, kv_head, dim]).  slots may be null (nothing is stored); a negative slot
-// skips the token.
+// dim, offset] (reference kv_cache.py:249-266 writes both as [page, offset, kv_head, dim]).
+// slots may be null (nothing is stored); a negative slot skips the token.
 template <typename T>
-__global__ void rotate_and_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
-                                        const float* __restrict__ inverse, int pairing, int heads, int kv_heads,
-                                        int dim, T* __restrict__ keys, T* __restrict__ values,
+__global__ void rotate_and_store_kernel(T* __restrict__ qkv, const float2* __restrict__ table, int pairing, int heads,
+                                        int kv_heads, int dim, T* __restrict__ keys, T* __restrict__ values,
                                         const int* __restrict__ slots, int page_size) {
   const int token = blockIdx.x;
   const int half = dim / 2;
   T* row = qkv + (size_t)token * (heads + 2 * kv_heads) * dim;
-  const float position = (float)positions[token];
   if (pairing != 0) {
+    const float2* angles = table + (size_t)token * half;
     const int pairs = (heads + kv_heads) * half;
     for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
       const int head = i / half, j = i % half;
-      float sine, cosine;
-      sincosf(position * inverse[j], &sine, &cosine);
+      const float2 cs = angles[j];
       T* h = row + head * dim;
       const int ia = pairing == 1 ? 2 * j : j;
       const int ib = pairing == 1 ? 2 * j + 1 : j + half;
       const float a = to_float(h[ia]), b = to_float(h[ib]);
-      h[ia] = from_float<T>(a * cosine - b * sine);
-      h[ib] = from_float<T>(b * cosine + a * sine);
+      h[ia] = from_float<T>(a * cs.x - b * cs.y);
+      h[ib] = from_float<T>(b * cs.x + a * cs.y);
     }
   }
   if (slots == nullptr) return;
@@ -112,17 +208,19 @@ __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const int* __restri
   }
 }
 
-extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const int* positions, const float* inverse,
-                                         int pairing, int tokens, int heads, int kv_heads, int dim, void* keys,
-                                         void* values, const int* slots, int page_size, hipStream_t stream) {
+extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const float* table, int pairing, int tokens,
+                                         int heads, int kv_heads, int dim, void* keys, void* values,
+                                         const int* slots, int page_size, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (dim % 2 || (pairing != 0 && inverse == nullptr) || pairing < 0 || pairing > 2) return ERR_BAD_ARGUMENT;
+  if (dim % 2 || (pairing != 0 && table == nullptr) || pairing < 0 || pairing > 2) return ERR_BAD_ARGUMENT;
   if (is_float)
-    hipLaunchKernelGGL(rotate_and_store_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float*)qkv, positions,
-                       inverse, pairing, heads, kv_heads, dim, (float*)keys, (float*)values, slots, page_size);
+    hipLaunchKernelGGL(rotate_and_store_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float*)qkv,
+                       (const float2*)table, pairing, heads, kv_heads, dim, (float*)keys, (float*)values, slots,
+                       page_size);
   else
-    hipLaunchKernelGGL(rotate_and_store_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t*)qkv, positions,
-                       inverse, pairing, heads, kv_heads, dim, (bf16_t*)keys, (bf16_t*)values, slots, page_size);
+    hipLaunchKernelGGL(rotate_and_store_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t*)qkv,
+                       (const float2*)table, pairing, heads, kv_heads, dim, (bf16_t*)keys, (bf16_t*)values, slots,
+                       page_size);
   return LAUNCH_STATUS();
 }
 
@@ -156,17 +254,24 @@ extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int
 }
 
 // ---------------------------------------------------------------------------- gather rows
-// out[r] = hidden[rows[r]] (+ delta[rows[r]])
-__global__ void gather_rows_kernel(const float* __restrict__ hidden, const float* __restrict__ delta,
-                                   const int* __restrict__ rows, float* __restrict__ out, int width) {
+// out[r] = hidden[rows[r]] (+ delta[0][rows[r]] + delta[1][rows[r]] + ...)
+__global__ void gather_rows_kernel(const float* __restrict__ hidden, const float* __restrict__ delta, int parts,
+                                   size_t part_stride, const int* __restrict__ rows, float* __restrict__ out,
+                                   int width) {
   const size_t src = (size_t)rows[blockIdx.x] * width;
   float* dst = out + (size_t)blockIdx.x * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = hidden[src + i] + (delta ? delta[src + i] : 0.f);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = hidden[src + i];
+    if (delta)
+      for (int p = 0; p < parts; ++p) v += delta[p * part_stride + src + i];
+    dst[i] = v;
+  }
 }
 
-extern "C" int llmserve_gather_rows(const float* hidden, const float* delta, const int* rows, float* out, int count,
-                                    int width, hipStream_t stream) {
+extern "C" int llmserve_gather_rows(const float* hidden, const float* delta, int parts, int total_rows,
+                                    const int* rows, float* out, int count, int width, hipStream_t stream) {
   if (count <= 0) return 0;
-  hipLaunchKernelGGL(gather_rows_kernel, dim3(count), dim3(256), 0, stream, hidden, delta, rows, out, width);
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(count), dim3(256), 0, stream, hidden, delta, parts,
+                     (size_t)total_rows * width, rows, out, width);
   return LAUNCH_STATUS();
 }

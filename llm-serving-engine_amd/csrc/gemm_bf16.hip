@@ -26,26 +26,29 @@ template <int WAVES, int MT, typename TO, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                  const bf16_t* __restrict__ w,
                                                                  const void* __restrict__ bias, int bias_is_float,
-                                                                 TO* __restrict__ out, int M, int N, int K) {
+                                                                 TO* __restrict__ out, int M, int N, int K,
+                                                                 int k_split) {
   extern __shared__ float partial[];  // [WAVES][MT][64 lanes][4]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
   const int n = min((int)blockIdx.x * 16 + r, N - 1);
-  const bf16_t* w_row = w + (size_t)n * K + g * 8;
+  // blockIdx.y picks a slice of K, `k_split` long; its sums go to its own copy of `out`
+  const int k_first = blockIdx.y * k_split;
+  const bf16_t* w_row = w + (size_t)n * K + k_first + g * 8;
   const bf16_t* x_row[MT];
   bool x_live[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + r;
     x_live[t] = m < M;
-    x_row[t] = x + (size_t)min(m, M - 1) * K + g * 8;
+    x_row[t] = x + (size_t)min(m, M - 1) * K + k_first + g * 8;
   }
   f32x4 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  const int groups = K / (STEP * GROUP);
+  const int groups = k_split / (STEP * GROUP);
   bf16x8 a[GROUP], a_next[GROUP];
   int group = wave;
   if (group < groups) {
@@ -71,7 +74,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     group = next;
   }
   // the steps left over when K is not a multiple of 128
-  for (int step = groups * GROUP + wave; step < K / STEP; step += WAVES) {
+  for (int step = groups * GROUP + wave; step < k_split / STEP; step += WAVES) {
     const bf16x8 a_tail = load8(w_row + step * STEP);
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -91,7 +94,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   const int m = t * 16 + r;
   const int n_first = blockIdx.x * 16 + g * 4;
   if (m >= M) return;
-  if (bias) {
+  if (bias && blockIdx.y == 0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       if (n_first + i < N) total[i] += load_as_float(bias, bias_is_float, n_first + i);
@@ -106,7 +109,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
       }
     }
   } else {
-    TO* dst = out + (size_t)m * N + n_first;
+    TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       if (n_first + i < N) dst[i] = from_float<TO>(total[i]);
@@ -115,42 +118,46 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 
 template <int WAVES, int MT, typename TO, bool GATED>
 static int launch_skinny(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
-                         int K, hipStream_t stream) {
+                         int K, int splits, hipStream_t stream) {
   const size_t lds = (size_t)WAVES * MT * 64 * 4 * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<WAVES, MT, TO, GATED>), dim3((N + 15) / 16), dim3(WAVES * 64), lds, stream,
-                     (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K);
+  hipLaunchKernelGGL((gemm_skinny_kernel<WAVES, MT, TO, GATED>), dim3((N + 15) / 16, splits), dim3(WAVES * 64), lds,
+                     stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K, K / splits);
   return LAUNCH_STATUS();
 }
 
 template <int WAVES, typename TO, bool GATED>
 static int pick_tiles(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
-                      hipStream_t stream) {
-  if (M <= 16) return launch_skinny<WAVES, 1, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
-  if (M <= 32) return launch_skinny<WAVES, 2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
-  return launch_skinny<WAVES, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+                      int splits, hipStream_t stream) {
+  if (M <= 16) return launch_skinny<WAVES, 1, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  if (M <= 32) return launch_skinny<WAVES, 2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  return launch_skinny<WAVES, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
 }
 
 template <typename TO, bool GATED>
 static int pick_waves(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
-                      hipStream_t stream) {
+                      int splits, hipStream_t stream) {
   // enough waves to cover the chip (about 2,048), but no more than there are 128-wide groups of K
-  const int tiles = (N + 15) / 16, groups = max(1, K / (STEP * GROUP));
+  const int tiles = (N + 15) / 16 * splits, groups = max(1, K / splits / (STEP * GROUP));
   int waves = 4;
   while (waves < 16 && waves * tiles < 2048 && waves * 2 <= groups) waves *= 2;
-  if (waves == 4) return pick_tiles<4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
-  if (waves == 8) return pick_tiles<8, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
-  return pick_tiles<16, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, stream);
+  if (waves == 4) return pick_tiles<4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  if (waves == 8) return pick_tiles<8, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  return pick_tiles<16, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
 }
 
 // x, w bfloat16; out bfloat16 or float32.  Needs 1 <= M <= 64, K a multiple of 32, and with
-// `gated` an even N.  Any N.
+// `gated` an even N.  Any N.  With splits > 1 (float32 out, not gated, K / splits a multiple of
+// 32) `out` is [splits, M, N]: slice s holds the sums over the s-th part of K (the bias in slice 0),
+// and whoever reads it adds the slices in order.
 extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
-                                    int out_is_float, int gated, int M, int N, int K, hipStream_t stream) {
+                                    int out_is_float, int gated, int M, int N, int K, int splits,
+                                    hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % STEP || (gated && N % 2)) return ERR_BAD_ARGUMENT;
+  if (M > 64 || K <= 0 || K % STEP || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
+  if (splits > 1 && (gated || !out_is_float || K % splits || (K / splits) % STEP)) return ERR_BAD_ARGUMENT;
   if (gated)
-    return out_is_float ? pick_waves<float, true>(x, w, bias, bias_is_float, out, M, N, K, stream)
-                        : pick_waves<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, stream);
-  return out_is_float ? pick_waves<float, false>(x, w, bias, bias_is_float, out, M, N, K, stream)
-                      : pick_waves<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, stream);
+    return out_is_float ? pick_waves<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                        : pick_waves<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+  return out_is_float ? pick_waves<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
+                      : pick_waves<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
 }

@@ -75,20 +75,61 @@ __device__ __forceinline__ void block_argmax(const float* row, int n, float* bes
   *best_index = shared_i[16];
 }
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __restrict__ logits,
-                                                                int* __restrict__ out, int vocab) {
+// Two stages, so that a few rows still fill the chip: each row is cut into `pieces` pieces,
+// a block finds the first maximum of its piece, and one more block per row picks among them.
+__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_pieces_kernel(const float* __restrict__ logits,
+                                                                       float* __restrict__ piece_values,
+                                                                       int* __restrict__ piece_indices, int vocab,
+                                                                       int pieces) {
   __shared__ float sv[17];
   __shared__ int si[17];
+  const int per = (vocab + pieces - 1) / pieces;
+  const int begin = min(vocab, (int)blockIdx.y * per), count = min(vocab, begin + per) - begin;
   float value;
   int index;
-  block_argmax(logits + (size_t)blockIdx.x * vocab, vocab, &value, &index, sv, si);
-  if (threadIdx.x == 0) out[blockIdx.x] = index;
+  block_argmax(logits + (size_t)blockIdx.x * vocab + begin, count, &value, &index, sv, si);
+  if (threadIdx.x == 0) {
+    piece_values[blockIdx.x * pieces + blockIdx.y] = count > 0 ? value : -INFINITY;
+    piece_indices[blockIdx.x * pieces + blockIdx.y] = count > 0 ? begin + index : 0x7fffffff;
+  }
 }
 
-extern "C" int llmserve_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+__global__ void argmax_pick_kernel(const float* __restrict__ piece_values, const int* __restrict__ piece_indices,
+                                   int* __restrict__ out, int pieces) {
+  // one wave per row; pieces ascend in index, so the first maximum among them is the row's
+  float value = -INFINITY;
+  int index = 0x7fffffff;
+  for (int i = threadIdx.x; i < pieces; i += WAVE) {
+    const float v = piece_values[blockIdx.x * pieces + i];
+    const int at = piece_indices[blockIdx.x * pieces + i];
+    if (at != 0x7fffffff && (v > value || index == 0x7fffffff)) {
+      value = v;
+      index = at;
+    }
+  }
+#pragma unroll
+  for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+    const float ov = __shfl_xor(value, offset, WAVE);
+    const int oi = __shfl_xor(index, offset, WAVE);
+    if (oi != 0x7fffffff && (index == 0x7fffffff || ov > value || (ov == value && oi < index))) {
+      value = ov;
+      index = oi;
+    }
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = index == 0x7fffffff ? 0 : index;
+}
+
+#define ARGMAX_PIECES 64
+
+// scratch: at least rows * 64 floats and rows * 64 ints
+extern "C" int llmserve_argmax(const float* logits, float* piece_values, int* piece_indices, int* out, int rows,
+                               int vocab, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) return ERR_BAD_ARGUMENT;
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, out, vocab);
+  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(rows, ARGMAX_PIECES), dim3(SAMPLE_THREADS), 0, stream, logits,
+                     piece_values, piece_indices, vocab, ARGMAX_PIECES);
+  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(WAVE), 0, stream, piece_values, piece_indices, out,
+                     ARGMAX_PIECES);
   return LAUNCH_STATUS();
 }
 

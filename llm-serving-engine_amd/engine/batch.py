@@ -58,8 +58,12 @@ class StepBatch:
     num_logit_rows: int
     max_query_length: int
     max_context_length: int
-    # Kernel libraries may keep per-step work lists here (built once, used by every layer).
+    # Kernel libraries may keep here what they derive from the step's shape on the host (work
+    # lists: built once, used by every layer, and still valid when a captured step is replayed) ...
     scratch: dict[str, Any] = field(default_factory=dict)
+    # ... and here what a kernel computes from the step's values (rotary angles): valid for one
+    # forward pass only, so a captured step records the kernel that fills it.
+    computed: dict[str, Any] = field(default_factory=dict)
 
     @property
     def num_sequences(self) -> int:

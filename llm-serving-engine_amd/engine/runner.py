@@ -292,6 +292,7 @@ class ModelRunner:
             self.model.forward(batch, self.cells)  # loads libraries, builds the work lists kept on `batch`
         torch.cuda.current_stream(self.device).wait_stream(stream)
         torch.cuda.synchronize(self.device)
+        batch.computed.clear()  # what kernels computed from the warm-up's values is recorded anew
         captured = torch.cuda.CUDAGraph()
         with torch.cuda.graph(captured):
             logits = self.model.forward(batch, self.cells)

@@ -91,6 +91,8 @@ class HipKernels:
         self._attention_generic = load_module("attention_generic")
         self._gemm_bf16 = load_module("gemm_bf16") if dtype == torch.bfloat16 else None
         self._attention_bf16: dict[int, ctypes.CDLL] = {}  # by head size, compiled when a model needs it
+        # one counter per attention tile that is split over its keys; zero between kernels
+        self._counters = torch.zeros(1 << 16, dtype=torch.int32, device=self.device)
         self._sampling = None
 
     # ------------------------------------------------------------------ helpers
@@ -121,12 +123,28 @@ class HipKernels:
         if hidden.dtype != torch.float32 or (delta is not None and delta.dtype != torch.float32):
             raise KernelError("add_rms_norm: the residual stream and what is added to it are float32")
         out = self._empty((rows, width), self.dtype)
+        parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]  # [parts, rows, width]: partial sums
         status = self._elementwise.llmserve_add_rms_norm(
-            _pointer(hidden), _pointer(delta), _pointer(weight), _is_float(weight), _pointer(out), _is_float(out),
-            rows, width, ctypes.c_float(eps), self._stream,
+            _pointer(hidden), _pointer(delta), parts, _pointer(weight), _is_float(weight), _pointer(out),
+            _is_float(out), rows, width, ctypes.c_float(eps), self._stream,
         )
         _check(status, "add_rms_norm")
         return out
+
+    def rotary_table(self, batch, inverse_frequencies: torch.Tensor) -> torch.Tensor:
+        """(cos, sin) [T, D/2, 2] float32 of position * frequency for the step's tokens.  Every
+        layer with the same frequencies shares it: it is computed once per step and kept on the batch."""
+        key = ("rotary_table", inverse_frequencies.data_ptr())
+        table = batch.computed.get(key)
+        if table is None:
+            tokens, half = batch.positions.shape[0], inverse_frequencies.shape[0]
+            table = self._empty((tokens, half, 2), torch.float32)
+            status = self._elementwise.llmserve_rotary_table(
+                _pointer(batch.positions), _pointer(inverse_frequencies), _pointer(table), tokens, half, self._stream
+            )
+            _check(status, "rotary_table")
+            batch.computed[key] = table
+        return table
 
     def rotate_and_store(self, qkv, layout, batch, cell, inverse_frequencies, pairing: str) -> None:
         tokens = qkv.shape[0]
@@ -136,19 +154,22 @@ class HipKernels:
         group = batch.groups[cell.group] if store else None
         if store and (cell.keys.dtype != qkv.dtype or cell.keys.shape[1:] != (layout.num_kv_heads, group.page_size, layout.head_dim)):
             raise KernelError("rotate_and_store: the cell's pages do not fit the layout")
+        table = self.rotary_table(batch, inverse_frequencies) if pairing != "none" else None
         status = self._elementwise.llmserve_rotate_and_store(
-            _pointer(qkv), _is_float(qkv), _pointer(batch.positions), _pointer(inverse_frequencies),
-            _PAIRINGS[pairing], tokens, layout.num_heads, layout.num_kv_heads, layout.head_dim,
-            _pointer(cell.keys if store else None), _pointer(cell.values if store else None),
-            _pointer(group.slot_mapping if store else None), group.page_size if store else 1, self._stream,
+            _pointer(qkv), _is_float(qkv), _pointer(table), _PAIRINGS[pairing], tokens, layout.num_heads,
+            layout.num_kv_heads, layout.head_dim, _pointer(cell.keys if store else None),
+            _pointer(cell.values if store else None), _pointer(group.slot_mapping if store else None),
+            group.page_size if store else 1, self._stream,
         )
         _check(status, "rotate_and_store")
 
     def gather_rows(self, hidden, delta, rows) -> torch.Tensor:
         count, width = rows.shape[0], hidden.shape[1]
         out = self._empty((count, width), torch.float32)
+        parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]
         status = self._elementwise.llmserve_gather_rows(
-            _pointer(hidden), _pointer(delta), _pointer(rows), _pointer(out), count, width, self._stream
+            _pointer(hidden), _pointer(delta), parts, hidden.shape[0], _pointer(rows), _pointer(out), count, width,
+            self._stream,
         )
         _check(status, "gather_rows")
         return out
@@ -180,43 +201,70 @@ class HipKernels:
         return (
             x.dtype == torch.bfloat16
             and weights.weight.dtype == torch.bfloat16
-            and 0 < x.shape[0] <= 64
+            and 0 < x.shape[0] <= (16 if self.library_products else 64)
             and weights.in_features % 32 == 0
         )
 
     def _library(self, x: torch.Tensor, weights: LinearWeights) -> bool:
         """Whether the product goes to the BLAS library (hipBLASLt through torch), as the
         reference's products go to its BLAS through nn.Linear: bfloat16 with more rows than
-        the weight-streaming kernel takes."""
+        the weight-streaming kernel is good at (one tile of 16)."""
         return (
             self.library_products
             and x.dtype == torch.bfloat16
             and weights.weight.dtype == torch.bfloat16
-            and x.shape[0] > 64
+            and x.shape[0] > 16
         )
 
-    def linear(self, x: torch.Tensor, weights: LinearWeights, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    @staticmethod
+    def _partial_splits(out_features: int, in_features: int) -> int:
+        """Into how many parts of K a weight-streaming product is cut when its float32 result
+        may stay in parts: a weight with few rows has too few 16-row tiles to fill the chip, so
+        K is cut (at most 8 ways, parts of at least 512) until about a thousand workgroups run."""
+        groups = in_features // 128
+        if in_features % 128 or groups < 8:
+            return 1
+        tiles = -(-out_features // 16)
+        best = 1
+        for splits in range(2, 9):
+            if groups % splits == 0 and groups // splits >= 4 and tiles * splits <= 1024:
+                best = splits
+        return best
+
+    def linear(
+        self, x: torch.Tensor, weights: LinearWeights, out_dtype: torch.dtype | None = None, *, partial: bool = False
+    ) -> torch.Tensor:
+        """`partial` allows a float32 result to come back as [parts, T, N] partial sums that
+        the reader adds up in order (`add_rms_norm` and `gather_rows` do)."""
         rows, inner = x.shape
         if inner != weights.in_features:
             raise KernelError(f"linear: x has {inner} columns, the weight {weights.in_features}")
         bias = weights.bias
         if self._library(x, weights):
-            out = torch.nn.functional.linear(x, weights.weight, bias if bias is None or bias.dtype == x.dtype else None)
+            if (out_dtype or self.dtype) == torch.float32:  # float32 straight from the accumulators
+                out = torch.mm(x, weights.weight.t(), out_dtype=torch.float32)
+                return out if bias is None else out.add_(bias.float())
             if bias is not None and bias.dtype != x.dtype:
-                out = out.float() + bias
-            return out.to(out_dtype or self.dtype)
-        out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
+                return (torch.mm(x, weights.weight.t(), out_dtype=torch.float32) + bias).to(torch.bfloat16)
+            return torch.nn.functional.linear(x, weights.weight, bias)
         bias_is_float = _is_float(bias) if bias is not None else 0
         if self._skinny(x, weights):
+            splits = 1
+            if partial and out_dtype == torch.float32:
+                splits = self._partial_splits(weights.out_features, inner)
+            shape = (rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features)
+            out = self._empty(shape, out_dtype or self.dtype)
             status = self._gemm_bf16.llmserve_gemm_skinny(
                 _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out), _is_float(out),
-                0, rows, weights.out_features, inner, self._stream,
+                0, rows, weights.out_features, inner, splits, self._stream,
             )
-        else:
-            status = self._gemm_generic.llmserve_gemm_generic(
-                _pointer(x), _is_float(x), _pointer(weights.weight), _is_float(weights.weight), _pointer(bias),
-                bias_is_float, _pointer(out), _is_float(out), rows, weights.out_features, inner, self._stream,
-            )
+            _check(status, "linear")
+            return out
+        out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
+        status = self._gemm_generic.llmserve_gemm_generic(
+            _pointer(x), _is_float(x), _pointer(weights.weight), _is_float(weights.weight), _pointer(bias),
+            bias_is_float, _pointer(out), _is_float(out), rows, weights.out_features, inner, self._stream,
+        )
         _check(status, "linear")
         return out
 
@@ -225,7 +273,7 @@ class HipKernels:
         if self._skinny(x, weights.both):
             status = self._gemm_bf16.llmserve_gemm_skinny(
                 _pointer(x), _pointer(weights.both.weight), _pointer(None), 0, _pointer(out), _is_float(out), 1,
-                x.shape[0], 2 * weights.width, x.shape[1], self._stream,
+                x.shape[0], 2 * weights.width, x.shape[1], 1, self._stream,
             )
             _check(status, "gated_linear")
             return out
@@ -285,9 +333,11 @@ class HipKernels:
         _check(status, "paged_attention")
         return out
 
-    def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int) -> None:
+    def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None) -> None:
         """The MFMA kernel: requests that bring a few tokens (decoding) one column tile per
-        wave, split over the keys when there are few of them; longer portions four tiles per wave."""
+        wave, split over the keys when there are few of them; longer portions four tiles per
+        wave.  `fuse` = (rotary table, pairing) lets a step of single tokens rotate and
+        store inside the same kernel."""
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
         per_tile = max(1, 16 // (heads // kv_heads))
@@ -300,20 +350,48 @@ class HipKernels:
             if items == 0:
                 continue
             splits, partial_acc, partial_ml = 1, None, None
-            if batch.max_query_length <= per_tile:  # only then does one launch cover every row
+            if batch.max_query_length <= per_tile:  # few tiles, maybe long: split the keys
                 blocks = items * kv_heads * head_tiles
                 steps = -(-batch.max_context_length // 32)
                 splits = max(1, min(-(-1024 // blocks), -(-steps // 4), 64))
                 if splits > 1:
                     partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), torch.float32)
                     partial_ml = self._empty((tokens * heads * splits * 2,), torch.float32)
+                    if blocks > self._counters.numel():
+                        self._counters = torch.zeros(2 * blocks, dtype=torch.int32, device=self.device)
+            table, pairing = fuse if fuse is not None else (None, "none")
             status = library.llmserve_attention_tiles(
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
-                _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width,
-                _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
-                group.page_size, ctypes.c_float(scale), window, splits, self._stream,
+                _pointer(self._counters), _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables),
+                group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
+                group.page_size, ctypes.c_float(scale), window, splits, 1 if fuse is not None else 0,
+                _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), self._stream,
             )
             _check(status, "paged_attention")
+
+    def rotate_store_attend(
+        self, qkv, layout, batch, cell, inverse_frequencies, pairing: str, scale: float, window: int | None
+    ) -> torch.Tensor:
+        """`rotate_and_store` followed by `paged_attention`; one kernel when every request of
+        the step brings a single token and the MFMA kernel takes the sizes."""
+        group = batch.groups[cell.group]
+        dim = layout.head_dim
+        if (
+            batch.max_query_length == 1
+            and cell.writable
+            and qkv.dtype == torch.bfloat16
+            and cell.keys.dtype == torch.bfloat16
+            and group.page_size % 4 == 0
+            and dim % 16 == 0
+            and 16 <= dim <= 256
+            and self._attention_library(dim).llmserve_attention_can_fuse(_PAIRINGS[pairing])
+        ):
+            out = self._empty((qkv.shape[0], layout.num_heads * dim), qkv.dtype)
+            table = self.rotary_table(batch, inverse_frequencies) if pairing != "none" else None
+            self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), fuse=(table, pairing))
+            return out
+        self.rotate_and_store(qkv, layout, batch, cell, inverse_frequencies, pairing)
+        return self.paged_attention(qkv, layout, batch, cell, scale, window)
 
     # ------------------------------------------------------------------ sampling
 
@@ -325,7 +403,11 @@ class HipKernels:
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         rows, vocab = logits.shape
         out = self._empty((rows,), torch.int32)
-        status = self._sampling_library().llmserve_argmax(_pointer(logits), _pointer(out), rows, vocab, self._stream)
+        piece_values = self._empty((rows * 64,), torch.float32)
+        piece_indices = self._empty((rows * 64,), torch.int32)
+        status = self._sampling_library().llmserve_argmax(
+            _pointer(logits), _pointer(piece_values), _pointer(piece_indices), _pointer(out), rows, vocab, self._stream
+        )
         _check(status, "argmax")
         return out
 

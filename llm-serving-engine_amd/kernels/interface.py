@@ -33,8 +33,11 @@ class Kernels(Protocol):
 
     def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor) -> Any: ...
 
-    def linear(self, x: torch.Tensor, weights: Any, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        """x [T, K] @ W^T + bias -> [T, N] in `out_dtype` (the run dtype if None)."""
+    def linear(
+        self, x: torch.Tensor, weights: Any, out_dtype: torch.dtype | None = None, *, partial: bool = False
+    ) -> torch.Tensor:
+        """x [T, K] @ W^T + bias -> [T, N] in `out_dtype` (the run dtype if None).  With
+        `partial`, a float32 result may be [parts, T, N] partial sums for the reader to add."""
 
     def gated_linear(self, x: torch.Tensor, weights: Any) -> torch.Tensor:
         """silu(x Wg^T) * (x Wu^T) -> [T, I] in the run dtype."""
@@ -49,6 +52,12 @@ class Kernels(Protocol):
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any, scale: float, window: int | None
     ) -> torch.Tensor:
         """Attention of the q heads of `qkv` over the cell's pages -> [T, heads * head_dim]."""
+
+    def rotate_store_attend(
+        self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any,
+        inverse_frequencies: torch.Tensor | None, pairing: str, scale: float, window: int | None,
+    ) -> torch.Tensor:
+        """`rotate_and_store` followed by `paged_attention` (a library may fuse them)."""
 
     def gather_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
         """float32 (hidden + delta)[rows]."""

@@ -14,7 +14,9 @@ from .position import HeadLayout
 class Mixer(Part):
     """A token mixer.  `forward(x, batch, cell)` takes the normed rows [T, hidden]
     in the run dtype and returns the float32 rows [T, hidden] to add to the
-    residual stream.  `cell` is what `cache_need` asked for."""
+    residual stream, or partial sums [parts, T, hidden] of them (whoever adds
+    them to the stream adds the parts in order).  `cell` is what `cache_need`
+    asked for."""
 
     def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
         raise NotImplementedError
@@ -80,8 +82,7 @@ class Attention(Mixer):
 
     def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
         qkv = self.kernels.linear(x, self.qkv)
-        self.position.encode_and_store(qkv, self.layout, batch, cell)
-        mixed = self.kernels.paged_attention(
+        mixed = self.position.encode_store_attend(
             qkv, self.layout, batch, cell, self.spec.scale, self.spec.window
         )
-        return self.kernels.linear(mixed, self.out, out_dtype=torch.float32)
+        return self.kernels.linear(mixed, self.out, out_dtype=torch.float32, partial=True)

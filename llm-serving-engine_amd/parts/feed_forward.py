@@ -11,7 +11,8 @@ from .base import FEED_FORWARDS, Part, TensorSpec
 
 class FeedForward(Part):
     """`forward(x)` takes the normed rows [T, hidden] in the run dtype and
-    returns the float32 rows to add to the residual stream."""
+    returns the float32 rows to add to the residual stream, or partial sums
+    [parts, T, hidden] of them."""
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         raise NotImplementedError
@@ -49,4 +50,4 @@ class GatedMLP(FeedForward):
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         activated = self.kernels.gated_linear(x, self.gate_up)
-        return self.kernels.linear(activated, self.down, out_dtype=torch.float32)
+        return self.kernels.linear(activated, self.down, out_dtype=torch.float32, partial=True)

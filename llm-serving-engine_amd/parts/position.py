@@ -41,6 +41,12 @@ class PositionEncoding(Part):
         position and, if `cell` is writable, stores k and v in the cell's pages."""
         raise NotImplementedError
 
+    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window) -> "torch.Tensor":
+        """`encode_and_store`, then attention over the cell's pages.  An encoding that
+        a kernel can apply on the way (rotary) overrides this to let the kernel library fuse the two."""
+        self.encode_and_store(qkv, layout, batch, cell)
+        return self.kernels.paged_attention(qkv, layout, batch, cell, scale, window)
+
 
 @POSITIONS.register("rotary")
 class Rotary(PositionEncoding):
@@ -53,12 +59,23 @@ class Rotary(PositionEncoding):
         super().__init__(spec, tensors, kernels)
         if spec.pairing not in ("half", "adjacent"):
             raise ValueError(f"unknown rotary pairing {spec.pairing!r}")
-        exponents = torch.arange(0, spec.head_dim, 2, dtype=torch.float32) / spec.head_dim
-        self.inverse_frequencies = kernels.to_device(1.0 / (spec.theta ** exponents))
+        # one tensor per (head size, theta) and kernel library: layers that rotate alike share it,
+        # and with it whatever the library derives from it per step
+        shared = kernels.__dict__.setdefault("_rotary_frequencies", {})
+        key = (spec.head_dim, spec.theta)
+        if key not in shared:
+            exponents = torch.arange(0, spec.head_dim, 2, dtype=torch.float32) / spec.head_dim
+            shared[key] = kernels.to_device(1.0 / (spec.theta ** exponents))
+        self.inverse_frequencies = shared[key]
 
     def encode_and_store(self, qkv, layout: HeadLayout, batch, cell) -> None:
         self.kernels.rotate_and_store(
             qkv, layout, batch, cell, self.inverse_frequencies, self.spec.pairing
+        )
+
+    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window):
+        return self.kernels.rotate_store_attend(
+            qkv, layout, batch, cell, self.inverse_frequencies, self.spec.pairing, scale, window
         )
 
 
@@ -68,3 +85,6 @@ class NoPosition(PositionEncoding):
 
     def encode_and_store(self, qkv, layout: HeadLayout, batch, cell) -> None:
         self.kernels.rotate_and_store(qkv, layout, batch, cell, None, "none")
+
+    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window):
+        return self.kernels.rotate_store_attend(qkv, layout, batch, cell, None, "none", scale, window)

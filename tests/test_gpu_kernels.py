@@ -300,3 +300,44 @@ def test_sampling_edges(kernels):
         got = k.sample(on_gpu(logits), on_gpu(torch.full((3,), 1.0)), on_gpu(torch.full((3,), 0.6)), on_gpu(torch.full((3,), u))).cpu().tolist()
         want = [plain.sample(logits[row], 1.0, 0.6, u) for row in range(3)]
         assert got == want, (u, got, want)
+
+
+@pytest.mark.parametrize("pairing", ["adjacent", "half", "none"])
+@pytest.mark.parametrize("heads,kv_heads,dim,page", [(12, 2, 128, 16), (6, 1, 64, 8), (5, 5, 32, 4), (4, 2, 48, 16), (40, 2, 64, 16)])
+def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
+    """A step of single tokens: rotation, the store of the new key and value, attention and the
+    merge of key splits in one kernel (or, where the sizes do not allow it, in the separate ones):
+    the result and the pages must be what the separate steps give."""
+    dtype = torch.bfloat16
+    lengths = [1, 2, page, page + 1, 33, 64, 65, 700, 301]
+    counts = [1] * len(lengths)
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=dim + page)
+    theta = 800.0
+    inverse = 1.0 / (theta ** (torch.arange(0, dim, 2).float() / dim))
+    rotate = {"adjacent": plain.rope_adjacent, "half": plain.rope_half, "none": lambda x, a: x}[pairing]
+    # the pages hold the earlier tokens' keys already rotated; the new token's slot holds garbage
+    expected = []
+    for index, (q, k, v) in enumerate(per_request):
+        angles = plain.rope_angles(dim, theta, torch.arange(q.shape[0]))
+        k_rot = rotate(rounded(k, dtype), angles).to(dtype).double()
+        q_rot = rotate(rounded(q, dtype), angles).to(dtype).double()
+        per_request[index] = (q, k_rot.float(), v)
+        full = plain.causal_attention(q_rot, k_rot, rounded(v, dtype), 0.2)
+        expected.append(full[-1:].flatten(1))
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    slots = batch.groups[0].slot_mapping.cpu().long()
+    cell.keys[slots // page, :, slots % page] = float("nan")
+    cell.values[slots // page, :, :, slots % page] = float("nan")
+    rows = []  # the step's rows carry unrotated q and k
+    for (q, k, v), original in zip(per_request, [p[1] for p in paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=dim + page)[2]]):
+        rows.append(torch.cat([q[-1:].flatten(1), original[-1:].flatten(1), v[-1:].flatten(1)], dim=1))
+    qkv = on_gpu(torch.cat(rows), dtype)
+    out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None if pairing == "none" else on_gpu(inverse), pairing, 0.2, None)
+    torch.testing.assert_close(out.cpu().double(), torch.cat(expected), **TOLERANCE[dtype])
+    stored_k = cell.keys.cpu().double()[slots // page, :, slots % page]
+    stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
+    want_k = torch.stack([p[1][-1].double() for p in per_request])
+    want_v = torch.stack([rounded(p[2][-1], dtype) for p in per_request])
+    torch.testing.assert_close(stored_k, want_k, **TOLERANCE[dtype])
+    torch.testing.assert_close(stored_v, want_v, atol=0, rtol=0)
+    assert int(kernels[dtype]._counters.abs().sum()) == 0  # the split counters are back at zero

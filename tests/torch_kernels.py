@@ -34,7 +34,7 @@ class TorchKernels:
 
     def add_rms_norm(self, hidden, delta, weight, eps):
         if delta is not None:
-            hidden += delta
+            hidden += delta if delta.ndim == 2 else delta.sum(0)
         variance = hidden.pow(2).mean(-1, keepdim=True)
         return (hidden * torch.rsqrt(variance + eps) * weight.float()).to(self.dtype)
 
@@ -46,7 +46,7 @@ class TorchKernels:
     def prepare_gated_linear(self, gate, up):
         return (_Linear(gate.float(), None), _Linear(up.float(), None))
 
-    def linear(self, x, weights, out_dtype=None):
+    def linear(self, x, weights, out_dtype=None, partial=False):
         y = x.float() @ weights.weight.T
         if weights.bias is not None:
             y = y + weights.bias
@@ -104,8 +104,14 @@ class TorchKernels:
                 row += 1
         return out.reshape(tokens, heads * dim).to(self.dtype)
 
+    def rotate_store_attend(self, qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window):
+        self.rotate_and_store(qkv, layout, batch, cell, inverse_frequencies, pairing)
+        return self.paged_attention(qkv, layout, batch, cell, scale, window)
+
     def gather_rows(self, hidden, delta, rows):
         picked = hidden[rows.long()]
+        if delta is not None and delta.ndim == 3:
+            delta = delta.sum(0)
         return picked + delta[rows.long()] if delta is not None else picked.clone()
 
     def argmax(self, logits):
