@@ -19,9 +19,7 @@
 // prompt portion by as much.
 // When every request of the step brings one token (FUSED), the kernel also does what comes
 // before and after it in a decode step: it rotates the queries in registers, the workgroup
-// that owns the newest key rotates that key and stores key and value in their page first,
-// and with `splits` > 1 the workgroup that finishes last (a counter per tile tells) merges
-// the splits, in split order, instead of a second kernel.
+// that owns the newest key rotates that key and stores key and value in their page first.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -40,7 +38,6 @@ constexpr int D = HEAD_DIM;
 constexpr int D_TILES = D / 16;
 constexpr bool WIDE = (D % 32 == 0);          // 32-wide MFMA steps over the head dimension
 constexpr int QK_STEPS = WIDE ? D / 32 : D / 16;
-constexpr int WAVES = 4;
 constexpr int KEYS = 32;                      // keys per step
 
 struct QkOperand {                            // one lane's share of a row for one MFMA step
@@ -83,15 +80,14 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
   const int* slots;           // [rows] page * page_size + offset of each token, negative: store nothing
 };
 
-template <int COLUMN_TILES, bool FUSED>
+template <int COLUMN_TILES, bool FUSED, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
     const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
-    float* __restrict__ partial_ml, int* __restrict__ counters, bf16_t* __restrict__ keys,
+    float* __restrict__ partial_ml, bf16_t* __restrict__ keys,
     bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
     int page_size, float scale, int window, int splits, FusedDecode fused) {
   extern __shared__ float lds[];  // [WAVES][16 columns][D + 2]
-  __shared__ int ticket;
   const int group = heads / kv_heads;
   const int kv_head = blockIdx.y % kv_heads, head_tile = blockIdx.y / kv_heads;
   const int heads_here = min(group - head_tile * 16, 16);
@@ -182,52 +178,54 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
         k_page[ib] = (bf16_t)b;
       }
       for (int d = lane; d < D; d += WAVE) v_page[(size_t)d * page_size] = v_row[d];
-      __threadfence();
+      __threadfence_block();  // read again below by this workgroup only
     }
     __syncthreads();
   }
 
-  for (int step = step_begin + wave; step < step_end; step += WAVES) {
-    const int key0 = step * KEYS;
-    // K rows of the two 16-key halves: lane (c, q) loads key c of each half, its q-th slice of the row
+  // One step's loads: the K rows of the two 16-key halves (lane (c, q) loads key c of each half,
+  // its q-th slice of the row) and the V^T rows (lane (c, q) loads, for row d = 16 * tile + c, keys
+  // 4q .. 4q+3 of each half).  Keys outside [first_key, last_key] are read from a key inside it
+  // (their weights are zero), so no page is touched that the request does not hold.
+  struct StepPages { int k_lo, k_hi, v_lo, v_hi; };
+  struct StepLoads {
     QkOperand k_lo[QK_STEPS], k_hi[QK_STEPS];
-    {
-      const int key_lo = min(max(key0 + c, first_key), last_key);
-      const int key_hi = min(max(key0 + 16 + c, first_key), last_key);
-      const bf16_t* row_lo = keys + (size_t)table[key_lo / page_size] * page_stride + head_offset +
-                             (size_t)(key_lo % page_size) * D;
-      const bf16_t* row_hi = keys + (size_t)table[key_hi / page_size] * page_stride + head_offset +
-                             (size_t)(key_hi % page_size) * D;
-#pragma unroll
-      for (int s = 0; s < QK_STEPS; ++s) {
-        k_lo[s] = load_qk(row_lo, s, q);
-        k_hi[s] = load_qk(row_hi, s, q);
-      }
-    }
-    // V^T rows: lane (c, q) loads, for row d = 16 * tile + c, keys 4q .. 4q+3 of each half
     bf16x4 v_lo[D_TILES], v_hi[D_TILES];
-    {
-      const int low_limit = first_key & ~3, high_limit = last_key & ~3;
-      const int start_lo = min(max(key0 + 4 * q, low_limit), high_limit);
-      const int start_hi = min(max(key0 + 16 + 4 * q, low_limit), high_limit);
-      const bf16_t* base_lo = values + (size_t)table[start_lo / page_size] * page_stride + head_offset +
-                              (start_lo % page_size);
-      const bf16_t* base_hi = values + (size_t)table[start_hi / page_size] * page_stride + head_offset +
-                              (start_hi % page_size);
+  };
+  const int low_limit = first_key & ~3, high_limit = last_key & ~3;
+  auto key_of = [&](int step, int half) { return min(max(step * KEYS + 16 * half + c, first_key), last_key); };
+  auto start_of = [&](int step, int half) { return min(max(step * KEYS + 16 * half + 4 * q, low_limit), high_limit); };
+  auto pages_of = [&](int step) {
+    return StepPages{table[key_of(step, 0) / page_size], table[key_of(step, 1) / page_size],
+                     table[start_of(step, 0) / page_size], table[start_of(step, 1) / page_size]};
+  };
+  auto fetch = [&](int step, const StepPages& pages, StepLoads& L) {
+    const bf16_t* row_lo = keys + (size_t)pages.k_lo * page_stride + head_offset + (size_t)(key_of(step, 0) % page_size) * D;
+    const bf16_t* row_hi = keys + (size_t)pages.k_hi * page_stride + head_offset + (size_t)(key_of(step, 1) % page_size) * D;
 #pragma unroll
-      for (int d = 0; d < D_TILES; ++d) {
-        v_lo[d] = *(const bf16x4*)(base_lo + (size_t)(d * 16 + c) * page_size);
-        v_hi[d] = *(const bf16x4*)(base_hi + (size_t)(d * 16 + c) * page_size);
-      }
-      if (key0 + KEYS - 1 > last_key) {  // slots after the last key were never written: keep them out of 0 * x
+    for (int s = 0; s < QK_STEPS; ++s) {
+      L.k_lo[s] = load_qk(row_lo, s, q);
+      L.k_hi[s] = load_qk(row_hi, s, q);
+    }
+    const bf16_t* base_lo = values + (size_t)pages.v_lo * page_stride + head_offset + start_of(step, 0) % page_size;
+    const bf16_t* base_hi = values + (size_t)pages.v_hi * page_stride + head_offset + start_of(step, 1) % page_size;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const bool dead_lo = start_lo + i > last_key, dead_hi = start_hi + i > last_key;  // the slots really read
+    for (int d = 0; d < D_TILES; ++d) {
+      L.v_lo[d] = *(const bf16x4*)(base_lo + (size_t)(d * 16 + c) * page_size);
+      L.v_hi[d] = *(const bf16x4*)(base_hi + (size_t)(d * 16 + c) * page_size);
+    }
+  };
+  auto compute = [&](int step, StepLoads& L) {
+    const int key0 = step * KEYS;
+    if (key0 + KEYS - 1 > last_key) {  // slots after the last key were never written: keep them out of 0 * x
+      const int start_lo = start_of(step, 0), start_hi = start_of(step, 1);
 #pragma unroll
-          for (int d = 0; d < D_TILES; ++d) {
-            if (dead_lo) v_lo[d][i] = (bf16_t)0.f;
-            if (dead_hi) v_hi[d][i] = (bf16_t)0.f;
-          }
+      for (int i = 0; i < 4; ++i) {
+        const bool dead_lo = start_lo + i > last_key, dead_hi = start_hi + i > last_key;  // the slots really read
+#pragma unroll
+        for (int d = 0; d < D_TILES; ++d) {
+          if (dead_lo) L.v_lo[d][i] = (bf16_t)0.f;
+          if (dead_hi) L.v_hi[d][i] = (bf16_t)0.f;
         }
       }
     }
@@ -236,8 +234,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
       f32x4 s_lo = {0.f, 0.f, 0.f, 0.f}, s_hi = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < QK_STEPS; ++s) {
-        s_lo = mfma_qk(k_lo[s], query[t][s], s_lo);
-        s_hi = mfma_qk(k_hi[s], query[t][s], s_hi);
+        s_lo = mfma_qk(L.k_lo[s], query[t][s], s_lo);
+        s_hi = mfma_qk(L.k_hi[s], query[t][s], s_hi);
       }
       // lane holds, for its column, keys key0 + 4q + i (lo) and key0 + 16 + 4q + i (hi)
       float score[8];
@@ -274,13 +272,22 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
         bf16x8 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          v[i] = v_lo[d][i];
-          v[4 + i] = v_hi[d][i];
+          v[i] = L.v_lo[d][i];
+          v[4 + i] = L.v_hi[d][i];
         }
         acc[t][d] *= correction;
         acc[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, weights, acc[t][d], 0, 0, 0);
       }
     }
+  };
+
+  // (Issuing a step's loads one step ahead was measured and does not pay: a step's arithmetic is
+  // short beside the latency of its loads, which scatter over the pool's pages; what hides that
+  // latency is many waves, each with a short walk.)
+  for (int step = step_begin + wave; step < step_end; step += WAVES) {
+    StepLoads loads;
+    fetch(step, pages_of(step), loads);
+    compute(step, loads);
   }
 
   // merge the waves, one column tile at a time: each wave leaves, per column, D sums, its
@@ -336,48 +343,32 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
     }
     __syncthreads();
   }
-  if (splits == 1) return;
-
-  // The workgroup that finishes last merges the splits of its tile, in split order:
-  // out = sum_s acc_s * exp(m_s - m) / sum_s l_s * exp(m_s - m).  The counter returns to zero.
-  __threadfence();
-  __syncthreads();
-  int* counter = counters + (size_t)blockIdx.x * gridDim.y + blockIdx.y;
-  if (threadIdx.x == 0) ticket = atomicAdd(counter, 1);
-  __syncthreads();
-  if (ticket != splits - 1) return;
-  __threadfence();
-  for (int index = threadIdx.x; index < COLUMN_TILES * 16 * (D / 4); index += WAVES * 64) {
-    const int t = index / (16 * (D / 4)), rest = index % (16 * (D / 4));
-    const int column = rest / (D / 4), d4 = (rest % (D / 4)) * 4;
-    const int token = t * tokens_per_tile + column / heads_here;
-    if (token >= tokens || column / heads_here >= tokens_per_tile) continue;
-    const int head = kv_head * group + head_tile * 16 + column % heads_here;
-    const size_t pair = ((size_t)row0 + token) * heads + head;
-    const float* ml = partial_ml + pair * splits * 2;
-    float best = -INFINITY;
-    for (int sp = 0; sp < splits; ++sp) best = fmaxf(best, ml[2 * sp]);
-    float total = 0.f;
-    f32x4 merged = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < splits; ++sp) {
-      if (ml[2 * sp] == -INFINITY) continue;
-      const float factor = __expf(ml[2 * sp] - best);
-      total += ml[2 * sp + 1] * factor;
-      const float* theirs = partial_acc + (pair * splits + sp) * D + d4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) merged[i] += theirs[i] * factor;
-    }
-    const float inverse = total > 0.f ? 1.f / total : 0.f;
-    bf16_t* dst = out + pair * D + d4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
-  }
-  if (threadIdx.x == 0) *counter = 0;
 }
 
-template <int COLUMN_TILES, bool FUSED>
+// Merges the key splits of one (token, head): out = sum_s acc_s * exp(m_s - m) / sum_s l_s *
+// exp(m_s - m), in split order.  A second kernel rather than "the last workgroup merges": a
+// workgroup that reads what others wrote needs the other chiplets' L2 written back first, and
+// that costs more than this launch.
+__global__ void attention_merge_kernel(const float* __restrict__ partial_acc, const float* __restrict__ partial_ml,
+                                       bf16_t* __restrict__ out, int splits) {
+  const size_t pair = blockIdx.x;  // row * heads + head
+  const float* ml = partial_ml + pair * splits * 2;
+  float best = -INFINITY;
+  for (int s = 0; s < splits; ++s) best = fmaxf(best, ml[2 * s]);
+  float total = 0.f;
+  for (int s = 0; s < splits; ++s) total += ml[2 * s] == -INFINITY ? 0.f : ml[2 * s + 1] * __expf(ml[2 * s] - best);
+  const float inverse = total > 0.f ? 1.f / total : 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float sum = 0.f;
+    for (int s = 0; s < splits; ++s)
+      if (ml[2 * s] != -INFINITY) sum += partial_acc[(pair * splits + s) * D + d] * __expf(ml[2 * s] - best);
+    out[pair * D + d] = (bf16_t)(sum * inverse);
+  }
+}
+
+template <int COLUMN_TILES, bool FUSED, int WAVES>
 static int launch_tiles(const void* qkv, int row_width, void* out, float* partial_acc, float* partial_ml,
-                        int* counters, void* keys, void* values, const int* block_tables, int table_width,
+                        void* keys, void* values, const int* block_tables, int table_width,
                         const int* positions, const int* work, int tiles, int heads, int kv_heads,
                         int tokens_per_tile, int page_size, float scale, int window, int splits, FusedDecode fused,
                         hipStream_t stream) {
@@ -387,20 +378,21 @@ static int launch_tiles(const void* qkv, int row_width, void* out, float* partia
   if (shared > 64 * 1024) {  // more dynamic LDS than a kernel gets by default: ask for it once
     static bool asked = false;
     if (!asked) {
-      if (hipFuncSetAttribute((const void*)attention_tiles_kernel<COLUMN_TILES, FUSED>,
+      if (hipFuncSetAttribute((const void*)attention_tiles_kernel<COLUMN_TILES, FUSED, WAVES>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shared) != hipSuccess)
         return ERR_BAD_ARGUMENT;
       asked = true;
     }
   }
-  hipLaunchKernelGGL((attention_tiles_kernel<COLUMN_TILES, FUSED>), dim3(tiles, kv_heads * head_tiles, splits),
+  hipLaunchKernelGGL((attention_tiles_kernel<COLUMN_TILES, FUSED, WAVES>), dim3(tiles, kv_heads * head_tiles, splits),
                      dim3(WAVES * 64), shared, stream, (const bf16_t*)qkv, row_width, (bf16_t*)out, partial_acc,
-                     partial_ml, counters, (bf16_t*)keys, (bf16_t*)values, block_tables, table_width, positions, work,
+                     partial_ml, (bf16_t*)keys, (bf16_t*)values, block_tables, table_width, positions, work,
                      heads, kv_heads, tokens_per_tile, page_size, scale, window, splits, fused);
   return LAUNCH_STATUS();
 }
 
 extern "C" int llmserve_attention_head_dim() { return D; }
+
 
 // Whether the fused decode form can rotate with this pairing at this head size.
 extern "C" int llmserve_attention_can_fuse(int pairing) {
@@ -412,37 +404,43 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // `work` holds `tiles` items of four ints; a tile covers `column_tiles * tokens_per_tile`
 // tokens at most, where tokens_per_tile = max(1, 16 / (heads / kv_heads)).  page_size must
 // be a multiple of 4.  With splits > 1, partial_acc is float32 [rows * heads * splits * D],
-// partial_ml [rows * heads * splits * 2] (rows being the step's token count) and counters
-// tiles * kv_heads * ceil(group / 16) ints that are zero before the call and after it.
+// partial_ml [rows * heads * splits * 2] (rows being the step's token count), and every row
+// of the step must lie in one of the tiles: a second kernel merges the splits of all rows.
 // With `fuse` every tile holds one token, qkv is as the projection left it, and the kernel
 // rotates (table of cos and sin per row, pairing) and stores the token's key and value at slots[row] itself.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
-                                        float* partial_ml, int* counters, void* keys, void* values,
+                                        float* partial_ml, void* keys, void* values,
                                         const int* block_tables, int table_width, const int* positions,
                                         const int* work, int tiles, int column_tiles, int rows, int heads,
                                         int kv_heads, int page_size, float scale, int window, int splits, int fuse,
                                         const float* table, int pairing, const int* slots,
                                         hipStream_t stream) {
   if (tiles <= 0) return 0;
-  if (heads % kv_heads || page_size % 4 || splits < 1 || (splits > 1 && (!partial_acc || !partial_ml || !counters)))
+  if (heads % kv_heads || page_size % 4 || splits < 1 || (splits > 1 && (!partial_acc || !partial_ml)))
     return ERR_BAD_ARGUMENT;
   const int group = heads / kv_heads;
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
   FusedDecode fused = {(const float2*)table, pairing, slots};
+  int status;
   if (fuse) {
     if (column_tiles != 1 || !slots || !llmserve_attention_can_fuse(pairing) || (pairing != 0 && !table))
       return ERR_BAD_ARGUMENT;
-    return launch_tiles<1, true>(qkv, row_width, out, partial_acc, partial_ml, counters, keys, values, block_tables,
-                                 table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
-                                 scale, window, splits, fused, stream);
+    status = launch_tiles<1, true, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
+                                        table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile,
+                                        page_size, scale, window, splits, fused, stream);
+  } else if (column_tiles == 1) {
+    status = launch_tiles<1, false, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
+                                    table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
+                                    scale, window, splits, fused, stream);
+  } else if (column_tiles == 4) {
+    status = launch_tiles<4, false, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
+                                    table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
+                                    scale, window, splits, fused, stream);
+  } else {
+    return ERR_BAD_ARGUMENT;
   }
-  if (column_tiles == 1)
-    return launch_tiles<1, false>(qkv, row_width, out, partial_acc, partial_ml, counters, keys, values, block_tables,
-                                  table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
-                                  scale, window, splits, fused, stream);
-  if (column_tiles == 4)
-    return launch_tiles<4, false>(qkv, row_width, out, partial_acc, partial_ml, counters, keys, values, block_tables,
-                                  table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
-                                  scale, window, splits, fused, stream);
-  return ERR_BAD_ARGUMENT;
+  if (status != 0 || splits == 1) return status;
+  hipLaunchKernelGGL(attention_merge_kernel, dim3(rows * heads), dim3(64), 0, stream, partial_acc, partial_ml,
+                     (bf16_t*)out, splits);
+  return LAUNCH_STATUS();
 }

@@ -91,8 +91,6 @@ class HipKernels:
         self._attention_generic = load_module("attention_generic")
         self._gemm_bf16 = load_module("gemm_bf16") if dtype == torch.bfloat16 else None
         self._attention_bf16: dict[int, ctypes.CDLL] = {}  # by head size, compiled when a model needs it
-        # one counter per attention tile that is split over its keys; zero between kernels
-        self._counters = torch.zeros(1 << 16, dtype=torch.int32, device=self.device)
         self._sampling = None
 
     # ------------------------------------------------------------------ helpers
@@ -351,19 +349,19 @@ class HipKernels:
                 continue
             splits, partial_acc, partial_ml = 1, None, None
             if batch.max_query_length <= per_tile:  # few tiles, maybe long: split the keys
+                # a wave walks its share of the keys step after step (32 keys each), and a walk of
+                # a few steps costs less than the second kernel that merges splits: split only when
+                # a wave would walk more than 8 steps and the chip has room for more workgroups
                 blocks = items * kv_heads * head_tiles
                 steps = -(-batch.max_context_length // 32)
-                splits = max(1, min(-(-1024 // blocks), -(-steps // 4), 64))
+                splits = max(1, min(-(-steps // 32), max(1, 2048 // blocks), 64))
                 if splits > 1:
                     partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), torch.float32)
                     partial_ml = self._empty((tokens * heads * splits * 2,), torch.float32)
-                    if blocks > self._counters.numel():
-                        self._counters = torch.zeros(2 * blocks, dtype=torch.int32, device=self.device)
             table, pairing = fuse if fuse is not None else (None, "none")
             status = library.llmserve_attention_tiles(
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
-                _pointer(self._counters), _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables),
-                group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
+                _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
                 group.page_size, ctypes.c_float(scale), window, splits, 1 if fuse is not None else 0,
                 _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), self._stream,
             )

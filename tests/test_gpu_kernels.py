@@ -340,4 +340,3 @@ def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
     want_v = torch.stack([rounded(p[2][-1], dtype) for p in per_request])
     torch.testing.assert_close(stored_k, want_k, **TOLERANCE[dtype])
     torch.testing.assert_close(stored_v, want_v, atol=0, rtol=0)
-    assert int(kernels[dtype]._counters.abs().sum()) == 0  # the split counters are back at zero
