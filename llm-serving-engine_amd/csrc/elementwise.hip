@@ -232,7 +232,7 @@ template <typename TI, typename TO>
 __global__ void silu_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out, int width) {
   const TI* row = in + (size_t)blockIdx.x * 2 * width;
   TO* dst = out + (size_t)blockIdx.x * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x) {
     const float gate = to_float(row[2 * i]), up = to_float(row[2 * i + 1]);
     dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
   }
@@ -241,7 +241,9 @@ __global__ void silu_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out,
 extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
                                  hipStream_t stream) {
   if (rows <= 0) return 0;
-  const dim3 grid(rows), block(256);
+  // a row is cut over several blocks when the rows alone would not fill the chip
+  const int pieces = rows >= 1024 ? 1 : max(1, min((width + 255) / 256, 1024 / rows));
+  const dim3 grid(rows, pieces), block(256);
   if (in_is_float && out_is_float)
     hipLaunchKernelGGL((silu_mul_kernel<float, float>), grid, block, 0, stream, (const float*)in, (float*)out, width);
   else if (in_is_float)

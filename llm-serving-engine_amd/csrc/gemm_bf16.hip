@@ -21,6 +21,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define GROUP 4   // MFMA steps a wave loads at once: 128 k, 256 bytes of each weight row
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *(const bf16x8*)p; }
+// The weight stream uses plain loads: non-temporal ones were measured 8-12 % slower here.
+__device__ __forceinline__ bf16x8 load8_stream(const bf16_t* p) { return *(const bf16x8*)p; }
+#ifndef TARGET_WAVES
+#define TARGET_WAVES 2048
+#endif
 
 template <int WAVES, int MT, typename TO, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
@@ -53,13 +58,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   int group = wave;
   if (group < groups) {
 #pragma unroll
-    for (int u = 0; u < GROUP; ++u) a[u] = load8(w_row + (group * GROUP + u) * STEP);
+    for (int u = 0; u < GROUP; ++u) a[u] = load8_stream(w_row + (group * GROUP + u) * STEP);
   }
   while (group < groups) {
     const int next = group + WAVES;
     if (next < groups) {
 #pragma unroll
-      for (int u = 0; u < GROUP; ++u) a_next[u] = load8(w_row + (next * GROUP + u) * STEP);
+      for (int u = 0; u < GROUP; ++u) a_next[u] = load8_stream(w_row + (next * GROUP + u) * STEP);
     }
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -75,7 +80,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   }
   // the steps left over when K is not a multiple of 128
   for (int step = groups * GROUP + wave; step < k_split / STEP; step += WAVES) {
-    const bf16x8 a_tail = load8(w_row + step * STEP);
+    const bf16x8 a_tail = load8_stream(w_row + step * STEP);
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const bf16x8 b_tail = x_live[t] ? load8(x_row[t] + step * STEP) : zero;
@@ -139,10 +144,157 @@ static int pick_waves(const void* x, const void* w, const void* bias, int bias_i
   // enough waves to cover the chip (about 2,048), but no more than there are 128-wide groups of K
   const int tiles = (N + 15) / 16 * splits, groups = max(1, K / splits / (STEP * GROUP));
   int waves = 4;
-  while (waves < 16 && waves * tiles < 2048 && waves * 2 <= groups) waves *= 2;
+  while (waves < 16 && waves * tiles < TARGET_WAVES && waves * 2 <= groups) waves *= 2;
   if (waves == 4) return pick_tiles<4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
   if (waves == 8) return pick_tiles<8, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
   return pick_tiles<16, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+}
+
+// ---------------------------------------------------------------------------- 16 < M <= 64
+// gemm_medium: the same product for up to 64 rows of x.  With more than one 16-row tile of x,
+// loading x per wave would cost more than streaming the weights, so a workgroup takes 64
+// weight rows (four waves, one 16-row tile each) times four slices of its K range (sixteen
+// waves), and the four waves of a K slice share the slice's 128 columns of x through LDS
+// (rows padded by 16 bytes, so that the 16-byte reads of an MFMA operand spread over all
+// banks).  K may be cut over workgroups too (blockIdx.y), leaving partial sums as above.
+#define MEDIUM_ROWS 64
+#define X_STRIDE (STEP * GROUP + 8)  // bf16 elements per staged row of x: 128 + padding
+
+template <int MT, typename TO, bool GATED>
+__global__ __launch_bounds__(1024) void gemm_medium_kernel(const bf16_t* __restrict__ x,
+                                                           const bf16_t* __restrict__ w,
+                                                           const void* __restrict__ bias, int bias_is_float,
+                                                           TO* __restrict__ out, int M, int N, int K,
+                                                           int groups_per_block) {
+  extern __shared__ float shared_medium[];
+  bf16_t* staged = (bf16_t*)shared_medium;  // [4 slices][MT * 16 rows][X_STRIDE]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row_tile = wave & 3, slice = wave >> 2;
+  const int r = lane & 15, g = lane >> 4;
+  const int n = min((int)blockIdx.x * MEDIUM_ROWS + row_tile * 16 + r, N - 1);
+  const int total_groups = K / (STEP * GROUP);
+  const int group_begin = blockIdx.y * groups_per_block;
+  const int group_end = min(total_groups, group_begin + groups_per_block);
+  const bf16_t* w_row = w + (size_t)n * K + g * 8;
+  bf16_t* my_stage = staged + (size_t)slice * (MT * 16) * X_STRIDE;
+  const int slice_thread = threadIdx.x & 255;  // index among the four waves of this K slice
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int rounds = (groups_per_block + 3) / 4;
+  for (int round = 0; round < rounds; ++round) {
+    const int group = group_begin + round * 4 + slice;
+    const bool live = group < group_end;
+    bf16x8 a[GROUP];
+    if (live) {
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) a[u] = load8_stream(w_row + (group * GROUP + u) * STEP);
+    }
+    __syncthreads();  // the previous round's reads of the staged x are done
+    if (live) {
+      // the slice's 256 threads bring x[0 .. MT*16)[group's 128 columns] in: 16 bytes each, MT * 16 * 16 pieces
+      for (int piece = slice_thread; piece < MT * 16 * 16; piece += 256) {
+        const int row = piece >> 4, part = piece & 15;
+        bf16x8 value = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (row < M) value = load8(x + (size_t)row * K + (size_t)group * (STEP * GROUP) + part * 8);
+        *(bf16x8*)(my_stage + (size_t)row * X_STRIDE + part * 8) = value;
+      }
+    }
+    __syncthreads();
+    if (live) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) {
+          const bf16x8 b = *(const bf16x8*)(my_stage + (size_t)(t * 16 + r) * X_STRIDE + u * STEP + g * 8);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[t], 0, 0, 0);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // add the four K slices of each row tile through LDS: [slice][row_tile][MT][64 lanes][4]
+  float* partial = shared_medium;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) *(f32x4*)(partial + (((slice * 4 + row_tile) * MT + t) * 64 + lane) * 4) = acc[t];
+  __syncthreads();
+  if (slice != 0) return;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    f32x4 total = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int v = 0; v < 4; ++v) total += *(const f32x4*)(partial + (((v * 4 + row_tile) * MT + t) * 64 + lane) * 4);
+    const int m = t * 16 + r;
+    const int n_first = blockIdx.x * MEDIUM_ROWS + row_tile * 16 + g * 4;
+    if (m >= M) continue;
+    if (bias && blockIdx.y == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n_first + i < N) total[i] += load_as_float(bias, bias_is_float, n_first + i);
+    }
+    if (GATED) {
+      TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (n_first + 2 * i + 1 < N) {
+          const float gate = total[2 * i], up = total[2 * i + 1];
+          dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+        }
+      }
+    } else {
+      TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n_first + i < N) dst[i] = from_float<TO>(total[i]);
+    }
+  }
+}
+
+template <int MT, typename TO, bool GATED>
+static int launch_medium(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
+                         int K, int splits, hipStream_t stream) {
+  const size_t stage = (size_t)4 * MT * 16 * X_STRIDE * sizeof(bf16_t);
+  const size_t merge = (size_t)4 * 4 * MT * 64 * 4 * sizeof(float);
+  const size_t lds = stage > merge ? stage : merge;
+  if (lds > 64 * 1024) {
+    static bool asked = false;
+    if (!asked) {
+      if (hipFuncSetAttribute((const void*)gemm_medium_kernel<MT, TO, GATED>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return ERR_BAD_ARGUMENT;
+      asked = true;
+    }
+  }
+  const int groups = K / (STEP * GROUP);
+  const int per_block = (groups + splits - 1) / splits;
+  hipLaunchKernelGGL((gemm_medium_kernel<MT, TO, GATED>), dim3((N + MEDIUM_ROWS - 1) / MEDIUM_ROWS, splits),
+                     dim3(1024), lds, stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N,
+                     K, per_block);
+  return LAUNCH_STATUS();
+}
+
+template <typename TO, bool GATED>
+static int pick_medium(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
+                       int K, int splits, hipStream_t stream) {
+  if (M <= 32) return launch_medium<2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  return launch_medium<4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+}
+
+// As llmserve_gemm_skinny, for 16 < M <= 64 and K a multiple of 128.  With splits > 1 the K
+// range is cut into `splits` runs of ceil(K / 128 / splits) groups of 128 and `out` is
+// [splits, M, N] partial sums.
+extern "C" int llmserve_gemm_medium(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
+                                    int out_is_float, int gated, int M, int N, int K, int splits,
+                                    hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % (STEP * GROUP) || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
+  if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
+  if (gated)
+    return out_is_float ? pick_medium<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                        : pick_medium<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+  return out_is_float ? pick_medium<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
+                      : pick_medium<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
 }
 
 // x, w bfloat16; out bfloat16 or float32.  Needs 1 <= M <= 64, K a multiple of 32, and with

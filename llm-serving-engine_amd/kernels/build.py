@@ -95,12 +95,14 @@ def build_module(module: str, defines: dict[str, object] | None = None, *, force
     for folder in _build_folders():
         try:
             folder.mkdir(parents=True, exist_ok=True)
+            if not os.access(folder, os.W_OK | os.X_OK):
+                raise PermissionError(f"{folder} is not writable")
             partial = folder / f".{name}.{os.getpid()}.tmp"
             command = [_hipcc(), *FLAGS, f"-I{CSRC}"]
             command += [f"-D{key}={value}" for key, value in sorted(defines.items())]
             command += [str(source), "-o", str(partial)]
-            tag = " ".join(f"{k}={v}" for k, v in sorted(defines.items()))
-            _say(f"compiling {module}.hip {tag}for gfx950 ...".replace("  ", " "))
+            tag = "".join(f" {k}={v}" for k, v in sorted(defines.items()))
+            _say(f"compiling {module}.hip{tag} for gfx950 ...")
             started = time.monotonic()
             process = subprocess.Popen(command, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
             while True:
@@ -113,6 +115,9 @@ def build_module(module: str, defines: dict[str, object] | None = None, *, force
                 partial.unlink(missing_ok=True)
                 raise BuildError(f"hipcc failed for {module}.hip:\n{output}")
             os.replace(partial, folder / name)
+            for stale in folder.glob(f"{name.rsplit('-', 1)[0]}-*.so"):  # older builds of the same source
+                if stale.name != name:
+                    stale.unlink(missing_ok=True)
             _say(f"  built {name} in {time.monotonic() - started:.1f} s")
             return folder / name
         except OSError as error:  # folder not writable: try the next one

@@ -194,23 +194,31 @@ class HipKernels:
         both = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
         return GatedLinearWeights(LinearWeights(both, None), gate.shape[0])
 
-    def _skinny(self, x: torch.Tensor, weights: LinearWeights) -> bool:
-        """Whether the weight-streaming MFMA kernel takes this product."""
-        return (
-            x.dtype == torch.bfloat16
-            and weights.weight.dtype == torch.bfloat16
-            and 0 < x.shape[0] <= (16 if self.library_products else 64)
-            and weights.in_features % 32 == 0
-        )
+    def _streaming(self, x: torch.Tensor, weights: LinearWeights) -> str | None:
+        """Which weight-streaming MFMA kernel takes this product: "skinny" (up to 16 rows of x),
+        "medium" (up to 64, x shared through LDS), or None."""
+        if x.dtype != torch.bfloat16 or weights.weight.dtype != torch.bfloat16:
+            return None
+        rows, inner = x.shape[0], weights.in_features
+        if 0 < rows <= 16 and inner % 32 == 0:
+            return "skinny"
+        if self.library_products:  # the library is faster than "medium" as it stands
+            return None
+        if 16 < rows <= 64 and inner % 128 == 0:
+            return "medium"
+        if 16 < rows <= 64 and inner % 32 == 0:
+            return "skinny"
+        return None
 
     def _library(self, x: torch.Tensor, weights: LinearWeights) -> bool:
         """Whether the product goes to the BLAS library (hipBLASLt through torch), as the
         reference's products go to its BLAS through nn.Linear: bfloat16 with more rows than
-        the weight-streaming kernel is good at (one tile of 16)."""
+        the weight-streaming kernels take."""
         return (
             self.library_products
             and x.dtype == torch.bfloat16
             and weights.weight.dtype == torch.bfloat16
+            and self._streaming(x, weights) is None
             and x.shape[0] > 16
         )
 
@@ -246,13 +254,15 @@ class HipKernels:
                 return (torch.mm(x, weights.weight.t(), out_dtype=torch.float32) + bias).to(torch.bfloat16)
             return torch.nn.functional.linear(x, weights.weight, bias)
         bias_is_float = _is_float(bias) if bias is not None else 0
-        if self._skinny(x, weights):
+        streaming = self._streaming(x, weights)
+        if streaming is not None:
             splits = 1
             if partial and out_dtype == torch.float32:
                 splits = self._partial_splits(weights.out_features, inner)
             shape = (rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features)
             out = self._empty(shape, out_dtype or self.dtype)
-            status = self._gemm_bf16.llmserve_gemm_skinny(
+            entry = self._gemm_bf16.llmserve_gemm_skinny if streaming == "skinny" else self._gemm_bf16.llmserve_gemm_medium
+            status = entry(
                 _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out), _is_float(out),
                 0, rows, weights.out_features, inner, splits, self._stream,
             )
@@ -268,8 +278,10 @@ class HipKernels:
 
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
         out = self._empty((x.shape[0], weights.width), self.dtype)
-        if self._skinny(x, weights.both):
-            status = self._gemm_bf16.llmserve_gemm_skinny(
+        streaming = self._streaming(x, weights.both)
+        if streaming is not None:
+            entry = self._gemm_bf16.llmserve_gemm_skinny if streaming == "skinny" else self._gemm_bf16.llmserve_gemm_medium
+            status = entry(
                 _pointer(x), _pointer(weights.both.weight), _pointer(None), 0, _pointer(out), _is_float(out), 1,
                 x.shape[0], 2 * weights.width, x.shape[1], 1, self._stream,
             )

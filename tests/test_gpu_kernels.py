@@ -26,6 +26,14 @@ def kernels():
     return {dtype: HipKernels(dtype) for dtype in DTYPES}
 
 
+@pytest.fixture(scope="module")
+def own_kernels():
+    """The library with every product on the hand-written kernels (none sent to the BLAS library)."""
+    from llmserve_amd.kernels import HipKernels
+
+    return HipKernels(torch.bfloat16, library_products=False)
+
+
 def on_gpu(tensor, dtype=None):
     return tensor.to("cuda", dtype) if dtype else tensor.to("cuda")
 
@@ -85,6 +93,25 @@ def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
     # a weight kept in 32-bit under a bfloat16 run
     wide = k.linear(on_gpu(x, dtype), k.prepare_linear([on_gpu(w)], None), out_dtype=torch.float32)
     torch.testing.assert_close(wide.cpu().double(), rounded(x, dtype) @ w.double().T, atol=1e-4, rtol=1e-4)
+    up = torch.randn(outer, inner) / math.sqrt(inner)
+    gated = k.gated_linear(on_gpu(x, dtype), k.prepare_gated_linear(on_gpu(w, dtype), on_gpu(up, dtype)))
+    want = F.silu(rounded(x, dtype) @ rounded(w, dtype).T) * (rounded(x, dtype) @ rounded(up, dtype).T)
+    torch.testing.assert_close(gated.cpu().double(), want, **TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("rows,inner,outer", [(17, 128, 64), (32, 256, 100), (33, 1536, 272), (64, 1280, 130), (64, 8960, 48),
+                                              (40, 96, 77), (64, 160, 2048), (100, 256, 40)])
+def test_products_without_the_library(own_kernels, rows, inner, outer):
+    """17 to 64 rows: the kernel that shares x through LDS (K a multiple of 128), else the
+    weight-streaming one with several tiles of x, else the generic one; with partial sums too."""
+    k, dtype = own_kernels, torch.bfloat16
+    x, w, b = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer)
+    expected = rounded(x, dtype) @ rounded(w, dtype).T + rounded(b, dtype)
+    handle = k.prepare_linear([on_gpu(w, dtype)], [on_gpu(b, dtype)])
+    torch.testing.assert_close(k.linear(on_gpu(x, dtype), handle).cpu().double(), expected, **TOLERANCE[dtype])
+    parts = k.linear(on_gpu(x, dtype), handle, out_dtype=torch.float32, partial=True)
+    summed = parts if parts.ndim == 2 else parts.sum(0)
+    torch.testing.assert_close(summed.cpu().double(), expected, atol=1e-4, rtol=1e-4)
     up = torch.randn(outer, inner) / math.sqrt(inner)
     gated = k.gated_linear(on_gpu(x, dtype), k.prepare_gated_linear(on_gpu(w, dtype), on_gpu(up, dtype)))
     want = F.silu(rounded(x, dtype) @ rounded(w, dtype).T) * (rounded(x, dtype) @ rounded(up, dtype).T)
