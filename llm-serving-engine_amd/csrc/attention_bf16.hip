@@ -93,7 +93,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
   const int heads_here = min(group - head_tile * 16, 16);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, q = lane >> 4;
-  const int* item = work + (size_t)blockIdx.x * 4;
+  // the work list runs from early to late tokens; late ones walk more keys, so they start first
+  const int* item = work + (size_t)(gridDim.x - 1 - blockIdx.x) * 4;
   const int request = item[0], row0 = item[1], tokens = item[2];
   const int position0 = positions[row0];
   const int last_key = position0 + tokens - 1;

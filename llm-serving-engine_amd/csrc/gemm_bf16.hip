@@ -183,33 +183,56 @@ __global__ __launch_bounds__(1024) void gemm_medium_kernel(const bf16_t* __restr
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  const int rounds = (groups_per_block + 3) / 4;
-  for (int round = 0; round < rounds; ++round) {
-    const int group = group_begin + round * 4 + slice;
-    const bool live = group < group_end;
-    bf16x8 a[GROUP];
-    if (live) {
+  // The slice's 256 threads bring x[0 .. MT*16)[a group's 128 columns] into LDS, 16 bytes a piece,
+  // MT pieces a thread: first into registers (issued a round ahead), then into LDS.
+  bf16x8 x_piece[MT];
+  auto fetch_x = [&](int group) {
 #pragma unroll
-      for (int u = 0; u < GROUP; ++u) a[u] = load8_stream(w_row + (group * GROUP + u) * STEP);
+    for (int i = 0; i < MT; ++i) {
+      const int piece = slice_thread + i * 256, row = piece >> 4, part = piece & 15;
+      x_piece[i] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+      if (row < M) x_piece[i] = load8(x + (size_t)row * K + (size_t)group * (STEP * GROUP) + part * 8);
     }
-    __syncthreads();  // the previous round's reads of the staged x are done
-    if (live) {
-      // the slice's 256 threads bring x[0 .. MT*16)[group's 128 columns] in: 16 bytes each, MT * 16 * 16 pieces
-      for (int piece = slice_thread; piece < MT * 16 * 16; piece += 256) {
-        const int row = piece >> 4, part = piece & 15;
-        bf16x8 value = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (row < M) value = load8(x + (size_t)row * K + (size_t)group * (STEP * GROUP) + part * 8);
-        *(bf16x8*)(my_stage + (size_t)row * X_STRIDE + part * 8) = value;
+  };
+  auto stage_x = [&]() {
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int piece = slice_thread + i * 256, row = piece >> 4, part = piece & 15;
+      *(bf16x8*)(my_stage + (size_t)row * X_STRIDE + part * 8) = x_piece[i];
+    }
+  };
+  // Rounds go in runs of three whose weights are all requested before the first is used, so the
+  // weight stream never waits for the arithmetic or for x.
+  constexpr int RUN = 3;
+  const int rounds = (groups_per_block + 3) / 4;
+  auto group_of = [&](int round) { return group_begin + round * 4 + slice; };
+  if (rounds > 0 && group_of(0) < group_end) fetch_x(group_of(0));
+  for (int base = 0; base < rounds; base += RUN) {
+    bf16x8 a[RUN][GROUP];
+#pragma unroll
+    for (int j = 0; j < RUN; ++j) {
+      if (base + j < rounds && group_of(base + j) < group_end) {
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) a[j][u] = load8_stream(w_row + (group_of(base + j) * GROUP + u) * STEP);
       }
     }
-    __syncthreads();
-    if (live) {
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
+    for (int j = 0; j < RUN; ++j) {
+      const int round = base + j;
+      if (round >= rounds) break;
+      const bool live = group_of(round) < group_end;
+      __syncthreads();  // the previous round's reads of the staged x are done
+      if (live) stage_x();
+      if (round + 1 < rounds && group_of(round + 1) < group_end) fetch_x(group_of(round + 1));
+      __syncthreads();
+      if (live) {
 #pragma unroll
-        for (int u = 0; u < GROUP; ++u) {
-          const bf16x8 b = *(const bf16x8*)(my_stage + (size_t)(t * 16 + r) * X_STRIDE + u * STEP + g * 8);
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[t], 0, 0, 0);
+        for (int t = 0; t < MT; ++t) {
+#pragma unroll
+          for (int u = 0; u < GROUP; ++u) {
+            const bf16x8 b = *(const bf16x8*)(my_stage + (size_t)(t * 16 + r) * X_STRIDE + u * STEP + g * 8);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][u], b, acc[t], 0, 0, 0);
+          }
         }
       }
     }

@@ -246,7 +246,21 @@ class HipKernels:
         if inner != weights.in_features:
             raise KernelError(f"linear: x has {inner} columns, the weight {weights.in_features}")
         bias = weights.bias
-        if self._library(x, weights):
+        streaming = self._streaming(x, weights)
+        if (
+            streaming is None
+            and partial
+            and out_dtype == torch.float32
+            and x.dtype == torch.bfloat16
+            and weights.weight.dtype == torch.bfloat16
+            and 16 < rows <= 64
+            and inner % 128 == 0
+            and self._partial_splits(weights.out_features, inner) >= 4
+        ):
+            # a long K over few weight rows (the down projection): cut over K into partial sums, the
+            # hand-written kernel is ahead of the library (16 against 25 us at 64 rows of the 1.5B sizes)
+            streaming = "medium"
+        if streaming is None and self._library(x, weights):
             if (out_dtype or self.dtype) == torch.float32:  # float32 straight from the accumulators
                 out = torch.mm(x, weights.weight.t(), out_dtype=torch.float32)
                 return out if bias is None else out.add_(bias.float())
@@ -254,7 +268,6 @@ class HipKernels:
                 return (torch.mm(x, weights.weight.t(), out_dtype=torch.float32) + bias).to(torch.bfloat16)
             return torch.nn.functional.linear(x, weights.weight, bias)
         bias_is_float = _is_float(bias) if bias is not None else 0
-        streaming = self._streaming(x, weights)
         if streaming is not None:
             splits = 1
             if partial and out_dtype == torch.float32:
