@@ -84,6 +84,7 @@ class CacheManager:
         self.sequences: dict[str, SequenceRecord] = {}
         self._free_slots: deque[int] = deque(range(config.max_sequences))
         self._tick = 0
+        self._used_tokens = 0  # tokens cached over all live requests
         self._high_water = {"pages": 0, "used_tokens": 0, "sequences": 0}
 
         self.groups: list[PageGroup] = []
@@ -216,43 +217,50 @@ class CacheManager:
             short += max(0, -balance)
         return short
 
-    def reserve(self, request_id: str, count: int) -> Reservation:
+    def reserve(self, request_id: str, count: int, *, checked: bool = False) -> Reservation:
         """Takes the cache entries of the request's next `count` tokens
         (reference `kv_cache.py:145-179`).  Pages that a window has passed are
         given back first.  Raises `CacheFullError`, holding nothing new, if a
-        pool runs dry or the request would outgrow the longest sequence."""
+        pool runs dry or the request would outgrow the longest sequence;
+        `checked` says that the caller has asked `fits` for this already."""
         if count <= 0:
             raise ValueError("count must be positive")
         record = self.sequences[request_id]
         start = record.length
-        if start + count > self.max_sequence_length:
-            raise CacheFullError("sequence exceeds the longest sequence the cache was built for")
-        if not self.fits([(request_id, count)]):
-            raise CacheFullError("paged cache has no free pages")
+        if not checked:
+            if start + count > self.max_sequence_length:
+                raise CacheFullError("sequence exceeds the longest sequence the cache was built for")
+            if not self.fits([(request_id, count)]):
+                raise CacheFullError("paged cache has no free pages")
         page_size = self.page_size
-        positions = np.arange(start, start + count)
+        first_new = -(-start // page_size)
+        end_new = -(-(start + count) // page_size)
         slots = []
         for index, group in enumerate(self.groups):
             table = group.tables[record.slot]
-            first = min(self._first_needed_block(group, start), math.ceil(start / page_size))
-            for block in range(record.released[index], first):
-                group.pool.free(int(table[block]), request_id)
-                table[block] = -1
-            record.released[index] = max(record.released[index], first)
-            for block in range(math.ceil(start / page_size), math.ceil((start + count) / page_size)):
+            if group.need.window is not None:
+                first = min(self._first_needed_block(group, start), first_new)
+                for block in range(record.released[index], first):
+                    group.pool.free(int(table[block]), request_id)
+                    table[block] = -1
+                if first > record.released[index]:
+                    record.released[index] = first
+            for block in range(first_new, end_new):
                 table[block] = group.pool.allocate(request_id)
-            group.peak_pages = max(group.peak_pages, group.pool.used_pages)
-            pages = table[positions // page_size].astype(np.int64)
-            slots.append((pages * page_size + positions % page_size).astype(np.int32))
+            if group.pool.used_pages > group.peak_pages:
+                group.peak_pages = group.pool.used_pages
+            if count == 1:  # a decoded token: no arrays on the way
+                slots.append(np.array([int(table[start // page_size]) * page_size + start % page_size], np.int32))
+            else:
+                positions = np.arange(start, start + count)
+                pages = table[positions // page_size].astype(np.int64)
+                slots.append((pages * page_size + positions % page_size).astype(np.int32))
         record.length = start + count
+        self._used_tokens += count
         self._touch(record)
-        used = sum(group.pool.used_pages for group in self.groups)
+        used = self.used_pages
         if used >= self._high_water["pages"]:
-            self._high_water = {
-                "pages": used,
-                "used_tokens": sum(item.length for item in self.sequences.values()),
-                "sequences": len(self.sequences),
-            }
+            self._high_water = {"pages": used, "used_tokens": self._used_tokens, "sequences": len(self.sequences)}
         return Reservation(request_id, record.slot, start, count, tuple(slots))
 
     def block_table(self, request_id: str, group: int = 0) -> list[int]:
@@ -263,6 +271,7 @@ class CacheManager:
     def free(self, request_id: str) -> None:
         """Gives back everything the request holds (reference `kv_cache.py:344-350`)."""
         record = self.sequences.pop(request_id)
+        self._used_tokens -= record.length
         for group in self.groups:
             table = group.tables[record.slot]
             for page in table[table >= 0].tolist():
@@ -336,10 +345,12 @@ class CacheManager:
                     raise AssertionError(f"group {index}: free slot {slot} still holds pages")
         if len(self._free_slots) + len(self.sequences) != self.config.max_sequences:
             raise AssertionError("request slots lost")
+        if self._used_tokens != sum(record.length for record in self.sequences.values()):
+            raise AssertionError("token count drifted")
 
     def stats(self, contiguous_max_length: int | None = None) -> dict[str, float]:
         """The reference's accounting (`kv_cache.py:386-413`), summed over groups."""
-        used_tokens = sum(record.length for record in self.sequences.values())
+        used_tokens = self._used_tokens
         used = self.used_pages
         total = sum(group.pool.num_pages for group in self.groups)
         held_tokens = 0

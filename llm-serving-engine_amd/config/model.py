@@ -110,7 +110,8 @@ class Qwen2Config(ArchitectureConfig):
     `config.py:30-32`, which stays the default), the sliding-window keys of
     Qwen2's config.json (the reference drops them silently), and
     `rope_pairing`.  `attention_bias` and `tie_word_embeddings` default to True
-    when absent, as in the reference (`config.py:21-22`).
+    when absent, as in the reference (`config.py:21-22`), and the rotation is the
+    reference's unless the folder comes from transformers (see `rope_pairing`).
     """
 
     architecture: ClassVar[str] = "Qwen2ForCausalLM"
@@ -128,10 +129,13 @@ class Qwen2Config(ArchitectureConfig):
     rms_norm_eps: float
     attention_bias: bool = True
     tie_word_embeddings: bool = True
-    # "half": pairs (j, j + D/2), the layout of published Qwen2 checkpoints.
     # "adjacent": pairs (2j, 2j+1), the rotation the reference applies
-    # (`model.py:39-42`).  The two agree after permuting each head's q/k rows.
-    rope_pairing: str = "half"
+    # (`model.py:39-42`), and so the default.  "half": pairs (j, j + D/2), the
+    # layout of published Qwen2 checkpoints; `from_dict` chooses it for a
+    # config.json that transformers wrote (it carries `transformers_version`)
+    # unless `rope_pairing` says otherwise.  The two agree after permuting each
+    # head's q/k rows.
+    rope_pairing: str = "adjacent"
     # Layers with index >= max_window_layers see only the last `sliding_window`
     # keys when use_sliding_window is set; the others see all of them.
     use_sliding_window: bool = False
@@ -189,7 +193,11 @@ class Qwen2Config(ArchitectureConfig):
             rms_norm_eps=reader.number("rms_norm_eps"),
             attention_bias=reader.boolean("attention_bias", default=True),
             tie_word_embeddings=reader.boolean("tie_word_embeddings", default=True),
-            rope_pairing=reader.choice("rope_pairing", choices=("half", "adjacent"), default="half"),
+            rope_pairing=reader.choice(
+                "rope_pairing",
+                choices=("half", "adjacent"),
+                default="half" if "transformers_version" in values else "adjacent",
+            ),
             use_sliding_window=use_window,
             sliding_window=reader.integer("sliding_window") if use_window else None,
             max_window_layers=reader.integer("max_window_layers", minimum=0) if use_window else None,

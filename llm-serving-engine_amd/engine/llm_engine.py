@@ -156,12 +156,12 @@ class EngineCore:
 
         entries, sampled = [], []
         for request, count in planned:
-            tokens = request.all_tokens[request.processed_tokens : request.processed_tokens + count]
+            tokens = request.tokens_between(request.processed_tokens, request.processed_tokens + count)
             last = request.processed_tokens + count == len(request.prompt_token_ids) + len(request.generated_token_ids)
             entries.append(StepEntry(request.request_id, tokens, (count - 1,) if last else ()))
             if last:  # otherwise: a portion of a prompt, or a replay after preemption
                 sampled.append(request)
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, fits_checked=True)
         for request, count in planned:
             request.processed_tokens += count
         if not sampled:

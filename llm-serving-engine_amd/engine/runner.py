@@ -193,12 +193,13 @@ class ModelRunner:
     def has_request(self, request_id: str) -> bool:
         return request_id in self.cache.sequences
 
-    def step(self, entries: list[StepEntry], *, create_missing: bool = False) -> torch.Tensor:
+    def step(self, entries: list[StepEntry], *, create_missing: bool = False, fits_checked: bool = False) -> torch.Tensor:
         """Runs the entries as one batch; returns float32 logits [wanted, vocab]
         in the order of the entries and of each entry's `want`.  The tensor may be a
         view of a buffer that the next step overwrites: use it, or copy it, before then.
 
-        Nothing is reserved if the batch does not fit (`CacheFullError`)."""
+        Nothing is reserved if the batch does not fit (`CacheFullError`); `fits_checked`
+        says that the caller has asked the cache's `fits` for exactly these entries."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
@@ -211,9 +212,8 @@ class ModelRunner:
             for place in entry.want:
                 if not 0 <= place < len(entry.tokens):
                     raise ValueError(f"request {entry.request_id!r}: wanted place {place} is outside its tokens")
-            for token in entry.tokens:
-                if not 0 <= token < self.vocab_size:
-                    raise ValueError(f"request {entry.request_id!r}: token {token} is outside the vocabulary")
+            if min(entry.tokens) < 0 or max(entry.tokens) >= self.vocab_size:
+                raise ValueError(f"request {entry.request_id!r}: a token is outside the vocabulary")
         created = []
         try:
             for entry in entries:
@@ -223,13 +223,13 @@ class ModelRunner:
                     self.add_request(entry.request_id)
                     created.append(entry.request_id)
             plan = [(entry.request_id, len(entry.tokens)) for entry in entries]
-            if not self.cache.fits(plan):
+            if not fits_checked and not self.cache.fits(plan):
                 raise CacheFullError("the step's tokens do not fit the cache")
         except Exception:
             for request_id in created:
                 self.end_request(request_id)
             raise
-        reservations = [self.cache.reserve(request_id, count) for request_id, count in plan]
+        reservations = [self.cache.reserve(request_id, count, checked=True) for request_id, count in plan]
         if self.use_graphs and not self.cache.states and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
             return self._decode_with_graph(reservations, entries)
         batch = build_step_batch(reservations, entries, self.cache, self.device)

@@ -41,6 +41,15 @@ class RequestState:
     def all_tokens(self) -> list[int]:
         return self.prompt_token_ids + self.generated_token_ids
 
+    def tokens_between(self, start: int, end: int) -> list[int]:
+        """all_tokens[start:end] without joining the two lists (a decode step asks for one token)."""
+        prompt = len(self.prompt_token_ids)
+        if start >= prompt:
+            return self.generated_token_ids[start - prompt : end - prompt]
+        if end <= prompt:
+            return self.prompt_token_ids[start:end]
+        return self.prompt_token_ids[start:] + self.generated_token_ids[: end - prompt]
+
     @property
     def remaining_input_tokens(self) -> int:
         return len(self.prompt_token_ids) + len(self.generated_token_ids) - self.processed_tokens

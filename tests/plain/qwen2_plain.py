@@ -35,7 +35,7 @@ class PlainConfig:
     rms_norm_eps: float
     attention_bias: bool
     tie_word_embeddings: bool
-    rope_pairing: str = "half"
+    rope_pairing: str = "adjacent"  # the reference's (`model.py:39-42`)
     # window[i] is None (all earlier keys) or the number of keys layer i sees.
     windows: tuple = ()
 
@@ -60,7 +60,7 @@ class PlainConfig:
             rms_norm_eps=float(values["rms_norm_eps"]),
             attention_bias=values.get("attention_bias", True),
             tie_word_embeddings=values.get("tie_word_embeddings", True),
-            rope_pairing=values.get("rope_pairing", "half"),
+            rope_pairing=values.get("rope_pairing", "adjacent"),
             windows=tuple(windows),
         )
 

@@ -20,13 +20,17 @@ QWEN_1_5B = {
     "num_attention_heads": 12, "num_key_value_heads": 2, "max_position_embeddings": 32768,
     "rope_theta": 1000000.0, "rms_norm_eps": 1e-06, "tie_word_embeddings": True,
     "sliding_window": 32768, "max_window_layers": 21, "use_sliding_window": False, "torch_dtype": "bfloat16",
+    "transformers_version": "4.43.1",
 }
 
 
 def test_reads_the_architectures_own_keys():
     config = Qwen2Config.from_dict(QWEN_1_5B)
     assert (config.num_layers, config.head_dim, config.attention_bias) == (28, 128, True)
-    assert config.rope_pairing == "half" and config.layer_window(27) is None
+    assert config.rope_pairing == "half" and config.layer_window(27) is None  # a published checkpoint's config
+    plain_folder = {k: v for k, v in QWEN_1_5B.items() if k != "transformers_version"}
+    assert Qwen2Config.from_dict(plain_folder).rope_pairing == "adjacent"  # the reference's rotation (model.py:39-42)
+    assert Qwen2Config.from_dict({**plain_folder, "rope_pairing": "half"}).rope_pairing == "half"
     # the reference's aliases (config.py:46-54)
     aliased = dict(QWEN_1_5B)
     aliased["num_layers"] = aliased.pop("num_hidden_layers")
