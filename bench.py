@@ -137,8 +137,9 @@ def main() -> int:
             seconds, _ = decode(batch, short, min(args.warmup, 8))
             points[f"decode_b{batch}"] = round(batch * short / seconds, 1)
 
+    label = Path(args.config).stem.replace("qwen", "Qwen").replace("b", "B")
     record = {
-        "metric": "decode tok/s at batch 8, 512-token prompts (Qwen2.5-1.5B shape)",
+        "metric": f"decode tok/s at batch {args.batch}, {args.prompt_len}-token prompts ({label} shape)",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -151,7 +152,7 @@ def main() -> int:
         "dtype": "bf16" if dtype == torch.bfloat16 else "fp32",
         "data": "synthetic: seeded random weights, uniform random token ids",
         "config": {
-            "model": "Qwen2.5-1.5B layer sizes, random weights",
+            "model": f"{label} layer sizes, random weights",
             "layers": config.num_layers,
             "layers_full": full.num_layers,
             "hidden": config.hidden_size,

@@ -96,3 +96,11 @@ def test_byte_tokenizer_round_trip():
     ids = tokenizer.encode("héllo")
     assert min(ids) >= 4 and max(ids) < 260 and tokenizer.vocab_size == 260 and tokenizer.eos_token_id == 2
     assert tokenizer.decode(ids + [0, 1, 2]) == "héllo"
+
+
+def test_bench_measures_one_gpu_only():
+    import subprocess
+    import sys
+
+    done = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 2 and len(done.stdout.strip().splitlines()) == 1 and "one GPU" in done.stdout
