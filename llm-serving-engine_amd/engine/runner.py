@@ -10,6 +10,7 @@ counterpart is the second half of `LLMEngine._step` plus
 
 from __future__ import annotations
 
+import contextlib
 from dataclasses import dataclass, field
 from typing import Any
 
@@ -235,12 +236,17 @@ class ModelRunner:
         batch = build_step_batch(reservations, entries, self.cache, self.device)
         return self.forward(batch)
 
+    def _stream_scope(self):
+        scope = getattr(self.kernels, "stream_scope", None)
+        return scope() if scope is not None else contextlib.nullcontext()
+
     @torch.inference_mode()
     def forward(self, batch: StepBatch) -> torch.Tensor:
-        if batch.num_logit_rows == 0:
-            self.model.forward_without_logits(batch, self.cells)
-            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
-        return self.model.forward(batch, self.cells)
+        with self._stream_scope():
+            if batch.num_logit_rows == 0:
+                self.model.forward_without_logits(batch, self.cells)
+                return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+            return self.model.forward(batch, self.cells)
 
     # ------------------------------------------------------------------ captured decode steps
 
@@ -288,13 +294,13 @@ class ModelRunner:
         batch = _view_step(static, sizes, widths, facts, chunks, self.cache.page_size)
         stream = torch.cuda.Stream(self.device)
         stream.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(stream):
+        with torch.cuda.stream(stream), self._stream_scope():
             self.model.forward(batch, self.cells)  # loads libraries, builds the work lists kept on `batch`
         torch.cuda.current_stream(self.device).wait_stream(stream)
         torch.cuda.synchronize(self.device)
         batch.computed.clear()  # what kernels computed from the warm-up's values is recorded anew
         captured = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(captured):
+        with torch.cuda.graph(captured), self._stream_scope():
             logits = self.model.forward(batch, self.cells)
         host = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         graph = _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)

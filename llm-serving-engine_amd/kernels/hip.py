@@ -8,6 +8,7 @@ torch's current stream, so a step can be captured into a HIP graph.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from dataclasses import dataclass
 from typing import Any
@@ -31,12 +32,43 @@ def _is_float(tensor: torch.Tensor) -> int:
     raise KernelError(f"kernels take float32 or bfloat16 tensors, not {tensor.dtype}")
 
 
-def _pointer(tensor: torch.Tensor | None) -> ctypes.c_void_p:
+def _pointer(tensor: torch.Tensor | None) -> int | None:
+    """The tensor's device address (None: a null pointer) for an argument declared as a pointer."""
     if tensor is None:
-        return ctypes.c_void_p(0)
+        return None
     if not tensor.is_contiguous():
         raise KernelError("kernels take contiguous tensors")
-    return ctypes.c_void_p(tensor.data_ptr())
+    return tensor.data_ptr()
+
+
+# Argument types of every entry point: p pointer, i int, f float.  Declared once, so that a call
+# costs no guessing: a decode step is replayed from a graph, but every other step pays per launch.
+_SIGNATURES = {
+    "llmserve_embedding": "pippiip",
+    "llmserve_add_rms_norm": "ppipipiiifp",
+    "llmserve_rotary_table": "pppiip",
+    "llmserve_rotate_and_store": "pipiiiiipppip",
+    "llmserve_silu_mul": "pipiiip",
+    "llmserve_gather_rows": "ppiippiip",
+    "llmserve_gemm_generic": "pipipipiiiip",
+    "llmserve_gemm_skinny": "pppipiiiiiip",
+    "llmserve_gemm_medium": "pppipiiiiiip",
+    "llmserve_attention_generic": "pipipppippiiiiifip",
+    "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
+    "llmserve_attention_can_fuse": "i",
+    "llmserve_argmax": "ppppiip",
+    "llmserve_sample": "ppppppiip",
+}
+_TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
+
+
+def _declared(library: ctypes.CDLL) -> ctypes.CDLL:
+    for name, signature in _SIGNATURES.items():
+        if hasattr(library, name):
+            entry = getattr(library, name)
+            entry.argtypes = [_TYPES[code] for code in signature]
+            entry.restype = ctypes.c_int
+    return library
 
 
 def _check(status: int, what: str) -> None:
@@ -86,18 +118,32 @@ class HipKernels:
         name = torch.cuda.get_device_properties(self.device).gcnArchName
         if not name.startswith("gfx950"):
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
-        self._elementwise = load_module("elementwise")
-        self._gemm_generic = load_module("gemm_generic")
-        self._attention_generic = load_module("attention_generic")
-        self._gemm_bf16 = load_module("gemm_bf16") if dtype == torch.bfloat16 else None
+        self._elementwise = _declared(load_module("elementwise"))
+        self._gemm_generic = _declared(load_module("gemm_generic"))
+        self._attention_generic = _declared(load_module("attention_generic"))
+        self._gemm_bf16 = _declared(load_module("gemm_bf16")) if dtype == torch.bfloat16 else None
+        self._pinned_stream: int | None = None
         self._attention_bf16: dict[int, ctypes.CDLL] = {}  # by head size, compiled when a model needs it
         self._sampling = None
 
     # ------------------------------------------------------------------ helpers
 
     @property
-    def _stream(self) -> ctypes.c_void_p:
-        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+    def _stream(self) -> int:
+        if self._pinned_stream is not None:
+            return self._pinned_stream
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    @contextlib.contextmanager
+    def stream_scope(self):
+        """Within the scope every kernel goes to the stream that is current at its start (asked
+        once instead of per launch); the caller must not switch streams inside."""
+        previous = self._pinned_stream
+        self._pinned_stream = torch.cuda.current_stream(self.device).cuda_stream
+        try:
+            yield
+        finally:
+            self._pinned_stream = previous
 
     def to_device(self, tensor: torch.Tensor) -> torch.Tensor:
         return tensor.to(self.device).contiguous()
@@ -124,7 +170,7 @@ class HipKernels:
         parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]  # [parts, rows, width]: partial sums
         status = self._elementwise.llmserve_add_rms_norm(
             _pointer(hidden), _pointer(delta), parts, _pointer(weight), _is_float(weight), _pointer(out),
-            _is_float(out), rows, width, ctypes.c_float(eps), self._stream,
+            _is_float(out), rows, width, eps, self._stream,
         )
         _check(status, "add_rms_norm")
         return out
@@ -196,13 +242,16 @@ class HipKernels:
 
     def _streaming(self, x: torch.Tensor, weights: LinearWeights) -> str | None:
         """Which weight-streaming MFMA kernel takes this product: "skinny" (up to 16 rows of x),
-        "medium" (up to 64, x shared through LDS), or None."""
+        "medium" (up to 64, x shared through LDS), or None (the BLAS library, or the generic kernel)."""
         if x.dtype != torch.bfloat16 or weights.weight.dtype != torch.bfloat16:
             return None
         rows, inner = x.shape[0], weights.in_features
         if 0 < rows <= 16 and inner % 32 == 0:
             return "skinny"
-        if self.library_products:  # the library is faster than "medium" as it stands
+        if self.library_products and (rows > 64 or torch.cuda.is_current_stream_capturing()):
+            # On the device the library is ahead of "medium" as it stands, so a captured step (which
+            # costs the host nothing per launch) takes the library; a step launched kernel by kernel
+            # is bound by the host, where a torch call costs four times one of ours.
             return None
         if 16 < rows <= 64 and inner % 128 == 0:
             return "medium"
@@ -311,7 +360,7 @@ class HipKernels:
 
     def _attention_library(self, head_dim: int):
         if head_dim not in self._attention_bf16:
-            self._attention_bf16[head_dim] = load_module("attention_bf16", {"HEAD_DIM": head_dim})
+            self._attention_bf16[head_dim] = _declared(load_module("attention_bf16", {"HEAD_DIM": head_dim}))
         return self._attention_bf16[head_dim]
 
     def _attention_work(self, batch, tokens_per_item: int, longer_than: int, up_to: int | None):
@@ -351,7 +400,7 @@ class HipKernels:
             _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
             _pointer(group.block_tables), group.width, _pointer(batch.token_sequence), _pointer(batch.positions),
             tokens, layout.num_heads, layout.num_kv_heads, dim, group.page_size,
-            ctypes.c_float(scale), int(window or 0), self._stream,
+            scale, int(window or 0), self._stream,
         )
         _check(status, "paged_attention")
         return out
@@ -387,7 +436,7 @@ class HipKernels:
             status = library.llmserve_attention_tiles(
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
                 _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
-                group.page_size, ctypes.c_float(scale), window, splits, 1 if fuse is not None else 0,
+                group.page_size, scale, window, splits, 1 if fuse is not None else 0,
                 _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), self._stream,
             )
             _check(status, "paged_attention")
@@ -420,7 +469,7 @@ class HipKernels:
 
     def _sampling_library(self):
         if self._sampling is None:
-            self._sampling = load_module("sampling")
+            self._sampling = _declared(load_module("sampling"))
         return self._sampling
 
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
