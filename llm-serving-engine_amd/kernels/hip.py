@@ -53,6 +53,7 @@ _SIGNATURES = {
     "llmserve_gemm_generic": "pipipipiiiip",
     "llmserve_gemm_skinny": "pppipiiiiiip",
     "llmserve_gemm_medium": "pppipiiiiiip",
+    "llmserve_gemm_tiled": "pppipiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifip",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
     "llmserve_attention_can_fuse": "i",
@@ -241,8 +242,9 @@ class HipKernels:
         return GatedLinearWeights(LinearWeights(both, None), gate.shape[0])
 
     def _streaming(self, x: torch.Tensor, weights: LinearWeights) -> str | None:
-        """Which weight-streaming MFMA kernel takes this product: "skinny" (up to 16 rows of x),
-        "medium" (up to 64, x shared through LDS), or None (the BLAS library, or the generic kernel)."""
+        """Which MFMA kernel takes this product: "skinny" (up to 16 rows of x, weights streamed),
+        "medium" (up to 64, x shared through LDS), "tiled" (any number, both operands through LDS),
+        or None (the BLAS library, or the generic kernel)."""
         if x.dtype != torch.bfloat16 or weights.weight.dtype != torch.bfloat16:
             return None
         rows, inner = x.shape[0], weights.in_features
@@ -257,6 +259,8 @@ class HipKernels:
             return "medium"
         if 16 < rows <= 64 and inner % 32 == 0:
             return "skinny"
+        if rows > 64 and inner % 32 == 0:
+            return "tiled"
         return None
 
     def _library(self, x: torch.Tensor, weights: LinearWeights) -> bool:
@@ -319,15 +323,21 @@ class HipKernels:
         bias_is_float = _is_float(bias) if bias is not None else 0
         if streaming is not None:
             splits = 1
-            if partial and out_dtype == torch.float32:
+            if partial and out_dtype == torch.float32 and streaming != "tiled":
                 splits = self._partial_splits(weights.out_features, inner)
             shape = (rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features)
             out = self._empty(shape, out_dtype or self.dtype)
-            entry = self._gemm_bf16.llmserve_gemm_skinny if streaming == "skinny" else self._gemm_bf16.llmserve_gemm_medium
-            status = entry(
-                _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out), _is_float(out),
-                0, rows, weights.out_features, inner, splits, self._stream,
-            )
+            if streaming == "tiled":
+                status = self._gemm_bf16.llmserve_gemm_tiled(
+                    _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out),
+                    _is_float(out), 0, rows, weights.out_features, inner, self._stream,
+                )
+            else:
+                entry = self._gemm_bf16.llmserve_gemm_skinny if streaming == "skinny" else self._gemm_bf16.llmserve_gemm_medium
+                status = entry(
+                    _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out),
+                    _is_float(out), 0, rows, weights.out_features, inner, splits, self._stream,
+                )
             _check(status, "linear")
             return out
         out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
@@ -342,6 +352,13 @@ class HipKernels:
         out = self._empty((x.shape[0], weights.width), self.dtype)
         streaming = self._streaming(x, weights.both)
         if streaming is not None:
+            if streaming == "tiled":
+                status = self._gemm_bf16.llmserve_gemm_tiled(
+                    _pointer(x), _pointer(weights.both.weight), None, 0, _pointer(out), _is_float(out), 1,
+                    x.shape[0], 2 * weights.width, x.shape[1], self._stream,
+                )
+                _check(status, "gated_linear")
+                return out
             entry = self._gemm_bf16.llmserve_gemm_skinny if streaming == "skinny" else self._gemm_bf16.llmserve_gemm_medium
             status = entry(
                 _pointer(x), _pointer(weights.both.weight), _pointer(None), 0, _pointer(out), _is_float(out), 1,
