@@ -5,13 +5,13 @@
 // of up to 16 "columns": the (token, query head) pairs of a few consecutive tokens of one
 // request that share one kv head.  A wave computes, for steps of 32 cached keys,
 //   S^T[key][column] = K[key][:] . Q[column][:]          v_mfma_f32_16x16x32_bf16, A = K rows
-//   P = exp(S * scale - running max), masked per column to the keys (p - window, p]
+//   P = exp(S * scale - the column's reference maximum), masked per column to the keys (p - window, p]
 //   O^T[d][column] += V^T[d][key] * P^T[key][column]      A = rows of the transposed V page
 // so each lane owns one column: its running maximum, its sum and four rows of every 16-row
 // tile of O^T.  Value pages are stored transposed ([page, kv_head, dim, offset]) so that the
 // keys, the contraction index of the second product, are contiguous for the A operand; the
-// two 16-key halves of a step are interleaved in groups of four keys so that the layout S
-// comes out in is already the layout P goes in with, without a shuffle.
+// keys of a step are dealt to the rows of the first product in groups of four so that the
+// layout S comes out in is already the layout P goes in with, without a shuffle.
 // The four waves of a workgroup take the steps of the tile's key range in turn and merge
 // their partial results through LDS; with `splits` > 1 several workgroups share a key range
 // and a second kernel merges them (for few long requests).  A wave may carry several column
@@ -39,6 +39,7 @@ constexpr int D_TILES = D / 16;
 constexpr bool WIDE = (D % 32 == 0);          // 32-wide MFMA steps over the head dimension
 constexpr int QK_STEPS = WIDE ? D / 32 : D / 16;
 constexpr int KEYS = 32;                      // keys per step
+constexpr float RESCALE_STEP = 8.f;           // log2 units a column's maximum may run ahead of its reference
 
 struct QkOperand {                            // one lane's share of a row for one MFMA step
 #if HEAD_DIM % 32 == 0
@@ -81,17 +82,18 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
 };
 
 template <int COLUMN_TILES, bool FUSED, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
+__global__ __launch_bounds__(WAVES * 64, COLUMN_TILES > 2 ? 1 : 2) void attention_tiles_kernel(
     const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
     float* __restrict__ partial_ml, bf16_t* __restrict__ keys,
     bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
-    int page_size, float scale, int window, int splits, FusedDecode fused) {
+    int page_size, int page_shift, float scale, int window, int splits, FusedDecode fused) {
   extern __shared__ float lds[];  // [WAVES][16 columns][D + 2]
   const int group = heads / kv_heads;
   const int kv_head = blockIdx.y % kv_heads, head_tile = blockIdx.y / kv_heads;
   const int heads_here = min(group - head_tile * 16, 16);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in all lanes: kept in a scalar register
   const int c = lane & 15, q = lane >> 4;
   // the work list runs from early to late tokens; late ones walk more keys, so they start first
   const int* item = work + (size_t)(gridDim.x - 1 - blockIdx.x) * 4;
@@ -158,8 +160,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
   const int per_split = (step_last - step_first + 1 + splits - 1) / splits;
   const int step_begin = step_first + blockIdx.z * per_split;
   const int step_end = min(step_last + 1, step_begin + per_split);
-  const size_t page_stride = (size_t)kv_heads * page_size * D;
-  const size_t head_offset = (size_t)kv_head * page_size * D;
+  const unsigned page_stride = (unsigned)kv_heads * page_size * D;  // elements of one page: checked to fit by the host
+  const unsigned head_offset = (unsigned)kv_head * page_size * D;
 
   if (FUSED && step_last >= step_begin && step_last < step_end) {
     // this workgroup reads the newest key: it stores it first (one token per tile when FUSED; with
@@ -184,111 +186,155 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
     __syncthreads();
   }
 
-  // One step's loads: the K rows of the two 16-key halves (lane (c, q) loads key c of each half,
-  // its q-th slice of the row) and the V^T rows (lane (c, q) loads, for row d = 16 * tile + c, keys
-  // 4q .. 4q+3 of each half).  Keys outside [first_key, last_key] are read from a key inside it
-  // (their weights are zero), so no page is touched that the request does not hold.
-  struct StepPages { int k_lo, k_hi, v_lo, v_hi; };
+  // One step's loads.  The 32 keys of a step are dealt to the two 16-row tiles of the first product
+  // so that a lane ends up with the scores of eight consecutive keys: row r of the "lo" tile is key
+  // 8 * (r / 4) + r % 4 of the step, of the "hi" tile four keys further, and lane (c, q), which gets
+  // rows 4q .. 4q+3 of both, holds keys 8q .. 8q+7.  That is the order the second product wants its
+  // weights in, and its other operand is then one 16-byte piece of a row of the transposed V page
+  // (row d = 16 * tile + c, keys 8q .. 8q+7; a page holds a multiple of 8 keys).  Keys outside
+  // [first_key, last_key] are read from a key inside it (their weights are zero), so no page is
+  // touched that the request does not hold.
   struct StepLoads {
     QkOperand k_lo[QK_STEPS], k_hi[QK_STEPS];
-    bf16x4 v_lo[D_TILES], v_hi[D_TILES];
+    bf16x8 v[D_TILES];
   };
-  const int low_limit = first_key & ~3, high_limit = last_key & ~3;
-  auto key_of = [&](int step, int half) { return min(max(step * KEYS + 16 * half + c, first_key), last_key); };
-  auto start_of = [&](int step, int half) { return min(max(step * KEYS + 16 * half + 4 * q, low_limit), high_limit); };
+  const int row_key = 8 * (c >> 2) + (c & 3);  // this lane's K row within a step (lo tile; hi: + 4)
+  const int low_limit = first_key & ~7, high_limit = last_key & ~7;
+  // Where a step's rows lie: the page numbers come from the block table (a load of their own,
+  // requested two steps ahead so that the loads of the rows never wait for it), the offsets
+  // within the pages are arithmetic.
+  struct StepPages { int k, k_hi, v; };
+  struct StepKeys { int k, k_hi, v; };
+  auto keys_of = [&](int step) {  // the keys this lane reads in a step
+    const int key0 = step * KEYS;
+    StepKeys at = {key0 + row_key, key0 + row_key + 4, key0 + 8 * q};
+    if (key0 < first_key || key0 + KEYS - 1 > last_key) {
+      at.k = min(max(at.k, first_key), last_key);
+      at.k_hi = min(max(at.k_hi, first_key), last_key);
+      at.v = min(max(at.v, low_limit), high_limit);
+    }
+    return at;
+  };
+  auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
   auto pages_of = [&](int step) {
-    return StepPages{table[key_of(step, 0) / page_size], table[key_of(step, 1) / page_size],
-                     table[start_of(step, 0) / page_size], table[start_of(step, 1) / page_size]};
+    const StepKeys at = keys_of(step);
+    return StepPages{table[page_index(at.k)], table[page_index(at.k_hi)], table[page_index(at.v)]};
   };
-  auto fetch = [&](int step, const StepPages& pages, StepLoads& L) {
-    const bf16_t* row_lo = keys + (size_t)pages.k_lo * page_stride + head_offset + (size_t)(key_of(step, 0) % page_size) * D;
-    const bf16_t* row_hi = keys + (size_t)pages.k_hi * page_stride + head_offset + (size_t)(key_of(step, 1) % page_size) * D;
+  auto fetch_keys = [&](int step, const StepPages& P, StepLoads& L) {
+    const StepKeys at = keys_of(step);
+    const int offset = at.k - page_index(at.k) * page_size, offset_hi = at.k_hi - page_index(at.k_hi) * page_size;
+    const bf16_t* row_lo = keys + (size_t)(unsigned)P.k * page_stride + (head_offset + (unsigned)offset * D);
+    const bf16_t* row_hi = keys + (size_t)(unsigned)P.k_hi * page_stride + (head_offset + (unsigned)offset_hi * D);
 #pragma unroll
     for (int s = 0; s < QK_STEPS; ++s) {
       L.k_lo[s] = load_qk(row_lo, s, q);
       L.k_hi[s] = load_qk(row_hi, s, q);
     }
-    const bf16_t* base_lo = values + (size_t)pages.v_lo * page_stride + head_offset + start_of(step, 0) % page_size;
-    const bf16_t* base_hi = values + (size_t)pages.v_hi * page_stride + head_offset + start_of(step, 1) % page_size;
-#pragma unroll
-    for (int d = 0; d < D_TILES; ++d) {
-      L.v_lo[d] = *(const bf16x4*)(base_lo + (size_t)(d * 16 + c) * page_size);
-      L.v_hi[d] = *(const bf16x4*)(base_hi + (size_t)(d * 16 + c) * page_size);
-    }
   };
-  auto compute = [&](int step, StepLoads& L) {
-    const int key0 = step * KEYS;
-    if (key0 + KEYS - 1 > last_key) {  // slots after the last key were never written: keep them out of 0 * x
-      const int start_lo = start_of(step, 0), start_hi = start_of(step, 1);
+  auto fetch_values = [&](int step, const StepPages& P, StepLoads& L) {
+    const StepKeys at = keys_of(step);
+    const bf16_t* base = values + (size_t)(unsigned)P.v * page_stride + (head_offset + (unsigned)(at.v - page_index(at.v) * page_size));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const bool dead_lo = start_lo + i > last_key, dead_hi = start_hi + i > last_key;  // the slots really read
-#pragma unroll
-        for (int d = 0; d < D_TILES; ++d) {
-          if (dead_lo) L.v_lo[d][i] = (bf16_t)0.f;
-          if (dead_hi) L.v_hi[d][i] = (bf16_t)0.f;
-        }
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < COLUMN_TILES; ++t) {
-      f32x4 s_lo = {0.f, 0.f, 0.f, 0.f}, s_hi = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < QK_STEPS; ++s) {
-        s_lo = mfma_qk(L.k_lo[s], query[t][s], s_lo);
-        s_hi = mfma_qk(L.k_hi[s], query[t][s], s_hi);
-      }
-      // lane holds, for its column, keys key0 + 4q + i (lo) and key0 + 16 + 4q + i (hi)
-      float score[8];
-      float tile_max = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int key = key0 + (i < 4 ? 4 * q + i : 16 + 4 * q + (i - 4));
-        const bool seen = key <= column_position[t] && key >= column_first[t];
-        score[i] = seen ? (i < 4 ? s_lo[i] : s_hi[i - 4]) * scale : -INFINITY;
-        tile_max = fmaxf(tile_max, score[i]);
-      }
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-      const float next_max = fmaxf(running_max[t], tile_max);
-      float correction = 1.f;
-      bf16x8 weights;
-      float added = 0.f;
-      if (next_max == -INFINITY) {  // nothing seen yet by this column
-#pragma unroll
-        for (int i = 0; i < 8; ++i) weights[i] = (bf16_t)0.f;
-      } else {
-        correction = __expf(running_max[t] - next_max);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float p = __expf(score[i] - next_max);  // exp(-inf) = 0 for masked keys
-          added += p;
-          weights[i] = (bf16_t)p;
-        }
-      }
-      running_sum[t] = running_sum[t] * correction + added;
-      running_max[t] = next_max;
-#pragma unroll
-      for (int d = 0; d < D_TILES; ++d) {
-        bf16x8 v;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          v[i] = L.v_lo[d][i];
-          v[4 + i] = L.v_hi[d][i];
-        }
-        acc[t][d] *= correction;
-        acc[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, weights, acc[t][d], 0, 0, 0);
-      }
-    }
+    for (int d = 0; d < D_TILES; ++d) L.v[d] = *(const bf16x8*)(base + (unsigned)(d * 16 + c) * page_size);
   };
 
-  // (Issuing a step's loads one step ahead was measured and does not pay: a step's arithmetic is
-  // short beside the latency of its loads, which scatter over the pool's pages; what hides that
-  // latency is many waves, each with a short walk.)
-  for (int step = step_begin + wave; step < step_end; step += WAVES) {
+  // Scores are kept in units of log2 (scale * log2 e is folded into one multiply-add, weights are
+  // exp2 of differences to the column's reference).  The reference is the column's maximum at
+  // some earlier step; it moves only when a score exceeds it by more than RESCALE_STEP, so weights
+  // reach 2^RESCALE_STEP at most, the accumulators are rescaled rarely, and the common step needs
+  // no exchange between the four lanes of a column: each checks its own eight scores.
+  const float scale_log2 = scale * 1.44269504088896f;
+  // first product of a step, for all column tiles: after it the K rows are no longer needed
+  auto scores_of = [&](const StepLoads& L, f32x4* s_lo, f32x4* s_hi) {
+#pragma unroll
+    for (int t = 0; t < COLUMN_TILES; ++t) {
+      s_lo[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      s_hi[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < QK_STEPS; ++s) {
+        s_lo[t] = mfma_qk(L.k_lo[s], query[t][s], s_lo[t]);
+        s_hi[t] = mfma_qk(L.k_hi[s], query[t][s], s_hi[t]);
+      }
+    }
+  };
+  // softmax weights and second product of a step
+  auto weigh_and_add = [&](int step, StepLoads& L, const f32x4* s_lo, const f32x4* s_hi) {
+    const int key0 = step * KEYS;
+    const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
+    bf16x8 weights[COLUMN_TILES];
+#pragma unroll
+    for (int t = 0; t < COLUMN_TILES; ++t) {
+      // lane holds, for its column, keys key0 + 8q + i
+      const bool unset = running_max[t] == -INFINITY;  // nothing seen yet by this column
+      const float reference = unset ? 0.f : running_max[t];
+      float x[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = fmaf(i < 4 ? s_lo[t][i] : s_hi[t][i - 4], scale_log2, -reference);
+      if (!interior) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int key = key0 + 8 * q + i;
+          if (key > column_position[t] || key < column_first[t]) x[i] = -INFINITY;
+        }
+      }
+      const float highest = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+      if (__any(highest > (unset ? -INFINITY : RESCALE_STEP))) {
+        float column_highest = fmaxf(highest, __shfl_xor(highest, 16, WAVE));
+        column_highest = fmaxf(column_highest, __shfl_xor(column_highest, 32, WAVE));
+        if (column_highest > (unset ? -INFINITY : RESCALE_STEP)) {  // the same answer in the four lanes of a column
+          const float correction = unset ? 0.f : __builtin_amdgcn_exp2f(-column_highest);
+          running_max[t] = reference + column_highest;
+          running_sum[t] *= correction;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) x[i] -= column_highest;
+#pragma unroll
+          for (int d = 0; d < D_TILES; ++d) acc[t][d] *= correction;
+        }
+      }
+      float added = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float p = __builtin_amdgcn_exp2f(x[i]);  // exp2(-inf) = 0 for keys the column does not see
+        added += p;
+        weights[t][i] = (bf16_t)p;
+      }
+      running_sum[t] += added;
+    }
+    if (key0 + KEYS - 1 > last_key) {  // slots after the last key were never written: keep them out of 0 * x
+      const int start = min(max(key0 + 8 * q, low_limit), high_limit);  // the slots really read
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (start + i > last_key) {
+#pragma unroll
+          for (int d = 0; d < D_TILES; ++d) L.v[d][i] = (bf16_t)0.f;
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < COLUMN_TILES; ++t)
+#pragma unroll
+      for (int d = 0; d < D_TILES; ++d)
+        acc[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(L.v[d], weights[t], acc[t][d], 0, 0, 0);
+  };
+
+  // A wave's next step is requested into the registers of the current one as soon as they are
+  // free: the K rows after the first product, the V rows after the second; the page numbers of a
+  // step are looked up a step before its rows are requested.
+  if (step_begin + wave < step_end) {
+    const int step0 = step_begin + wave;
     StepLoads loads;
-    fetch(step, pages_of(step), loads);
-    compute(step, loads);
+    StepPages pages = pages_of(step0);
+    fetch_keys(step0, pages, loads);
+    fetch_values(step0, pages, loads);
+    if (step0 + WAVES < step_end) pages = pages_of(step0 + WAVES);
+    for (int step = step0; step < step_end; step += WAVES) {
+      const bool more = step + WAVES < step_end;
+      f32x4 s_lo[COLUMN_TILES], s_hi[COLUMN_TILES];
+      scores_of(loads, s_lo, s_hi);
+      if (more) fetch_keys(step + WAVES, pages, loads);
+      weigh_and_add(step, loads, s_lo, s_hi);
+      if (more) fetch_values(step + WAVES, pages, loads);
+      if (step + 2 * WAVES < step_end) pages = pages_of(step + 2 * WAVES);
+    }
   }
 
   // merge the waves, one column tile at a time: each wave leaves, per column, D sums, its
@@ -319,7 +365,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
       f32x4 merged = {0.f, 0.f, 0.f, 0.f};
       for (int w = 0; w < WAVES; ++w) {
         const float* theirs = lds + ((size_t)w * 16 + column) * STRIDE;
-        const float factor = theirs[D] == -INFINITY ? 0.f : __expf(theirs[D] - best);
+        const float factor = theirs[D] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(theirs[D] - best);
         total += theirs[D + 1] * factor;
 #pragma unroll
         for (int i = 0; i < 4; ++i) merged[i] += theirs[d4 + i] * factor;
@@ -346,8 +392,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_tiles_kernel(
   }
 }
 
-// Merges the key splits of one (token, head): out = sum_s acc_s * exp(m_s - m) / sum_s l_s *
-// exp(m_s - m), in split order.  A second kernel rather than "the last workgroup merges": a
+// Merges the key splits of one (token, head): out = sum_s acc_s * 2^(m_s - m) / sum_s l_s *
+// 2^(m_s - m), in split order (the maxima are kept in units of log2).  A second kernel rather than "the last workgroup merges": a
 // workgroup that reads what others wrote needs the other chiplets' L2 written back first, and
 // that costs more than this launch.
 __global__ void attention_merge_kernel(const float* __restrict__ partial_acc, const float* __restrict__ partial_ml,
@@ -357,12 +403,12 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial_acc, co
   float best = -INFINITY;
   for (int s = 0; s < splits; ++s) best = fmaxf(best, ml[2 * s]);
   float total = 0.f;
-  for (int s = 0; s < splits; ++s) total += ml[2 * s] == -INFINITY ? 0.f : ml[2 * s + 1] * __expf(ml[2 * s] - best);
+  for (int s = 0; s < splits; ++s) total += ml[2 * s] == -INFINITY ? 0.f : ml[2 * s + 1] * exp2f(ml[2 * s] - best);
   const float inverse = total > 0.f ? 1.f / total : 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float sum = 0.f;
     for (int s = 0; s < splits; ++s)
-      if (ml[2 * s] != -INFINITY) sum += partial_acc[(pair * splits + s) * D + d] * __expf(ml[2 * s] - best);
+      if (ml[2 * s] != -INFINITY) sum += partial_acc[(pair * splits + s) * D + d] * exp2f(ml[2 * s] - best);
     out[pair * D + d] = (bf16_t)(sum * inverse);
   }
 }
@@ -374,6 +420,7 @@ static int launch_tiles(const void* qkv, int row_width, void* out, float* partia
                         int tokens_per_tile, int page_size, float scale, int window, int splits, FusedDecode fused,
                         hipStream_t stream) {
   const int group = heads / kv_heads;
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
   const int head_tiles = (group + 15) / 16;
   const size_t shared = (size_t)WAVES * 16 * (D + 2) * sizeof(float);
   if (shared > 64 * 1024) {  // more dynamic LDS than a kernel gets by default: ask for it once
@@ -388,7 +435,7 @@ static int launch_tiles(const void* qkv, int row_width, void* out, float* partia
   hipLaunchKernelGGL((attention_tiles_kernel<COLUMN_TILES, FUSED, WAVES>), dim3(tiles, kv_heads * head_tiles, splits),
                      dim3(WAVES * 64), shared, stream, (const bf16_t*)qkv, row_width, (bf16_t*)out, partial_acc,
                      partial_ml, (bf16_t*)keys, (bf16_t*)values, block_tables, table_width, positions, work,
-                     heads, kv_heads, tokens_per_tile, page_size, scale, window, splits, fused);
+                     heads, kv_heads, tokens_per_tile, page_size, page_shift, scale, window, splits, fused);
   return LAUNCH_STATUS();
 }
 
@@ -404,7 +451,7 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 
 // `work` holds `tiles` items of four ints; a tile covers `column_tiles * tokens_per_tile`
 // tokens at most, where tokens_per_tile = max(1, 16 / (heads / kv_heads)).  page_size must
-// be a multiple of 4.  With splits > 1, partial_acc is float32 [rows * heads * splits * D],
+// be a multiple of 8.  With splits > 1, partial_acc is float32 [rows * heads * splits * D],
 // partial_ml [rows * heads * splits * 2] (rows being the step's token count), and every row
 // of the step must lie in one of the tiles: a second kernel merges the splits of all rows.
 // With `fuse` every tile holds one token, qkv is as the projection left it, and the kernel
@@ -417,8 +464,9 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
                                         const float* table, int pairing, const int* slots,
                                         hipStream_t stream) {
   if (tiles <= 0) return 0;
-  if (heads % kv_heads || page_size % 4 || splits < 1 || (splits > 1 && (!partial_acc || !partial_ml)))
+  if (heads % kv_heads || page_size % 8 || splits < 1 || (splits > 1 && (!partial_acc || !partial_ml)))
     return ERR_BAD_ARGUMENT;
+  if ((long)kv_heads * page_size * D >= (1L << 31)) return ERR_BAD_ARGUMENT;  // a page's elements are counted in 32 bits
   const int group = heads / kv_heads;
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
   FusedDecode fused = {(const float2*)table, pairing, slots};
@@ -431,6 +479,10 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
                                         page_size, scale, window, splits, fused, stream);
   } else if (column_tiles == 1) {
     status = launch_tiles<1, false, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
+                                    table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
+                                    scale, window, splits, fused, stream);
+  } else if (column_tiles == 2) {
+    status = launch_tiles<2, false, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
                                     table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
                                     scale, window, splits, fused, stream);
   } else if (column_tiles == 4) {

@@ -321,107 +321,112 @@ extern "C" int llmserve_gemm_medium(const void* x, const void* w, const void* bi
 }
 
 // ---------------------------------------------------------------------------- many rows
-// gemm_tiled: the same product for any number of rows of x (prompt portions), a classic tiled
-// product: a workgroup computes 128 weight rows x 128 rows of x, steps of 32 over K go through
-// LDS (two buffers: the next step's 16-byte pieces are requested before the current step is
-// multiplied), and each of the four waves owns 64 x 64 of the result as 2 x 2 tiles of
-// v_mfma_f32_32x32x16_bf16.  As in the kernels above the weights are the A operand, so a lane
-// ends up with four consecutive weight rows n of one row m of x: bias, SiLU(gate) * up over
-// interleaved rows, and the stores work the same way.
+// gemm_tiled: the same product for any number of rows of x (prompt portions), a tiled product:
+// a workgroup of four waves (2 x 2) computes a square tile of 64 * WT weight rows by 64 * WT rows
+// of x; steps of 32 over K go through LDS (two buffers: the next step's 16-byte pieces are
+// requested before the current step is multiplied); each wave owns WT x WT tiles of
+// v_mfma_f32_32x32x16_bf16.  WT = 4 (256 x 256, 128 x 128 a wave) halves the LDS traffic per
+// multiply of WT = 2 and is used when the product has enough such tiles to fill the chip.
+// As in the kernels above the weights are the A operand, so a lane ends up with four consecutive
+// weight rows n of one row m of x: bias, SiLU(gate) * up over interleaved rows, and the stores
+// work the same way; K may be cut over workgroups (blockIdx.z) into partial sums.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-#define TILE_MN 128
 #define TILE_K 32
 #define TILE_STRIDE (TILE_K + 8)  // bf16 elements per staged row: 64 bytes + 16 of padding
 
-template <typename TO, bool GATED>
+template <int WT, typename TO, bool GATED>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                          const void* __restrict__ bias, int bias_is_float,
-                                                         TO* __restrict__ out, int M, int N, int K) {
-  __shared__ __attribute__((aligned(16))) bf16_t staged_w[2][TILE_MN * TILE_STRIDE];
-  __shared__ __attribute__((aligned(16))) bf16_t staged_x[2][TILE_MN * TILE_STRIDE];
+                                                         TO* __restrict__ out, int M, int N, int K, int k_split) {
+  constexpr int TILE = 64 * WT;          // rows of each operand in the workgroup's tile
+  constexpr int PIECES = TILE * 4 / 256;  // 16-byte pieces of an operand's step each thread moves
+  extern __shared__ __attribute__((aligned(16))) bf16_t staged[];  // [2 buffers][w, x][TILE][TILE_STRIDE]
+  auto staged_w = [&](int buffer) { return staged + (size_t)(buffer * 2) * TILE * TILE_STRIDE; };
+  auto staged_x = [&](int buffer) { return staged + (size_t)(buffer * 2 + 1) * TILE * TILE_STRIDE; };
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wave_n = wave & 1, wave_m = wave >> 1;  // which 64 x 64 quarter of the 128 x 128 tile
-  const int n0 = blockIdx.x * TILE_MN, m0 = blockIdx.y * TILE_MN;
+  const int wave_n = wave & 1, wave_m = wave >> 1;
+  const int n0 = blockIdx.x * TILE, m0 = blockIdx.y * TILE;
+  const int k_first = blockIdx.z * k_split;
   const int r32 = lane & 31, half = lane >> 5;
 
-  // each thread moves two 16-byte pieces of each operand per step: piece -> (row, 8-element part)
-  int piece_row[2], piece_part[2];
-  const bf16_t* w_src[2];
-  const bf16_t* x_src[2];
-  bool w_live[2], x_live[2];
+  const bf16_t* w_src[PIECES];
+  const bf16_t* x_src[PIECES];
+  bool w_live[PIECES], x_live[PIECES];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int piece = threadIdx.x + i * 256;
-    piece_row[i] = piece >> 2;
-    piece_part[i] = piece & 3;
-    w_live[i] = n0 + piece_row[i] < N;
-    x_live[i] = m0 + piece_row[i] < M;
-    w_src[i] = w + (size_t)min(n0 + piece_row[i], N - 1) * K + piece_part[i] * 8;
-    x_src[i] = x + (size_t)min(m0 + piece_row[i], M - 1) * K + piece_part[i] * 8;
+  for (int i = 0; i < PIECES; ++i) {
+    const int piece = threadIdx.x + i * 256, row = piece >> 2, part = piece & 3;
+    w_live[i] = n0 + row < N;
+    x_live[i] = m0 + row < M;
+    w_src[i] = w + (size_t)min(n0 + row, N - 1) * K + k_first + part * 8;
+    x_src[i] = x + (size_t)min(m0 + row, M - 1) * K + k_first + part * 8;
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  bf16x8 w_piece[2], x_piece[2];
+  bf16x8 w_piece[PIECES], x_piece[PIECES];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < PIECES; ++i) {
       w_piece[i] = w_live[i] ? load8(w_src[i] + k0) : zero;
       x_piece[i] = x_live[i] ? load8(x_src[i] + k0) : zero;
     }
   };
   auto stage = [&](int buffer) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      *(bf16x8*)(staged_w[buffer] + piece_row[i] * TILE_STRIDE + piece_part[i] * 8) = w_piece[i];
-      *(bf16x8*)(staged_x[buffer] + piece_row[i] * TILE_STRIDE + piece_part[i] * 8) = x_piece[i];
+    for (int i = 0; i < PIECES; ++i) {
+      const int piece = threadIdx.x + i * 256, row = piece >> 2, part = piece & 3;
+      *(bf16x8*)(staged_w(buffer) + row * TILE_STRIDE + part * 8) = w_piece[i];
+      *(bf16x8*)(staged_x(buffer) + row * TILE_STRIDE + part * 8) = x_piece[i];
     }
   };
 
-  f32x16 acc[2][2];  // [tile of weight rows][tile of x rows]
+  f32x16 acc[WT][WT];  // [tile of weight rows][tile of x rows]
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WT; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WT; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int steps = K / TILE_K;
+  const int steps = k_split / TILE_K;
   fetch(0);
   stage(0);
   for (int step = 0; step < steps; ++step) {
     const int buffer = step & 1;
     __syncthreads();
     if (step + 1 < steps) fetch((step + 1) * TILE_K);
+    const bf16_t* from_w = staged_w(buffer) + (size_t)(wave_n * 32 * WT + r32) * TILE_STRIDE + half * 8;
+    const bf16_t* from_x = staged_x(buffer) + (size_t)(wave_m * 32 * WT + r32) * TILE_STRIDE + half * 8;
 #pragma unroll
     for (int kk = 0; kk < TILE_K / 16; ++kk) {
-      bf16x8 a[2], b[2];
+      bf16x8 a[WT], b[WT];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        a[i] = *(const bf16x8*)(staged_w[buffer] + (wave_n * 64 + i * 32 + r32) * TILE_STRIDE + kk * 16 + half * 8);
-        b[i] = *(const bf16x8*)(staged_x[buffer] + (wave_m * 64 + i * 32 + r32) * TILE_STRIDE + kk * 16 + half * 8);
+      for (int i = 0; i < WT; ++i) {
+        a[i] = *(const bf16x8*)(from_w + (size_t)i * 32 * TILE_STRIDE + kk * 16);
+        b[i] = *(const bf16x8*)(from_x + (size_t)i * 32 * TILE_STRIDE + kk * 16);
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < WT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
     if (step + 1 < steps) stage(buffer ^ 1);  // read last in step - 1: everyone has passed this step's barrier since
   }
 
   // D[n][m] of a 32 x 32 tile: lane holds column m = lane % 32 and rows n = 8 * (e / 4) + 4 * (lane / 32) + e % 4
+  const bool with_bias = bias && blockIdx.z == 0;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int m = m0 + wave_m * 64 + j * 32 + r32;
+  for (int j = 0; j < WT; ++j) {
+    const int m = m0 + wave_m * 32 * WT + j * 32 + r32;
     if (m >= M) continue;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < WT; ++i) {
 #pragma unroll
       for (int quad = 0; quad < 4; ++quad) {
-        const int n_first = n0 + wave_n * 64 + i * 32 + quad * 8 + half * 4;
+        const int n_first = n0 + wave_n * 32 * WT + i * 32 + quad * 8 + half * 4;
         float value[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           value[e] = acc[i][j][quad * 4 + e];
-          if (bias && n_first + e < N) value[e] += load_as_float(bias, bias_is_float, n_first + e);
+          if (with_bias && n_first + e < N) value[e] += load_as_float(bias, bias_is_float, n_first + e);
         }
         if (GATED) {
           TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
@@ -429,7 +434,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
           for (int e = 0; e < 2; ++e)
             if (n_first + 2 * e + 1 < N) dst[e] = from_float<TO>(value[2 * e] / (1.f + expf(-value[2 * e])) * value[2 * e + 1]);
         } else {
-          TO* dst = out + (size_t)m * N + n_first;
+          TO* dst = out + ((size_t)blockIdx.z * M + m) * N + n_first;
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (n_first + e < N) dst[e] = from_float<TO>(value[e]);
@@ -439,24 +444,48 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   }
 }
 
-template <typename TO, bool GATED>
+template <int WT, typename TO, bool GATED>
 static int launch_tiled(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
-                        int K, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm_tiled_kernel<TO, GATED>), dim3((N + TILE_MN - 1) / TILE_MN, (M + TILE_MN - 1) / TILE_MN),
-                     dim3(256), 0, stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K);
+                        int K, int splits, hipStream_t stream) {
+  constexpr int TILE = 64 * WT;
+  const size_t lds = (size_t)4 * TILE * TILE_STRIDE * sizeof(bf16_t);
+  if (lds > 64 * 1024) {
+    static bool asked = false;
+    if (!asked) {
+      if (hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, TO, GATED>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return ERR_BAD_ARGUMENT;
+      asked = true;
+    }
+  }
+  hipLaunchKernelGGL((gemm_tiled_kernel<WT, TO, GATED>), dim3((N + TILE - 1) / TILE, (M + TILE - 1) / TILE, splits),
+                     dim3(256), lds, stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K,
+                     K / splits);
   return LAUNCH_STATUS();
 }
 
+template <typename TO, bool GATED>
+static int pick_tiled(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
+                      int splits, hipStream_t stream) {
+  // the big tile when there are enough of them for every CU (256) to get one
+  const long big_tiles = (long)((N + 255) / 256) * ((M + 255) / 256) * splits;
+  if (big_tiles >= 200) return launch_tiled<4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  return launch_tiled<2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+}
+
 // x, w bfloat16; out bfloat16 or float32; any M and N, K a multiple of 32, an even N with `gated`.
+// With splits > 1 (float32 out, not gated, K / splits a multiple of 32) `out` is [splits, M, N]
+// partial sums, the bias in the first.
 extern "C" int llmserve_gemm_tiled(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
-                                   int out_is_float, int gated, int M, int N, int K, hipStream_t stream) {
+                                   int out_is_float, int gated, int M, int N, int K, int splits, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || K % TILE_K || (gated && N % 2)) return ERR_BAD_ARGUMENT;
+  if (K <= 0 || K % TILE_K || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
+  if (splits > 1 && (gated || !out_is_float || K % splits || (K / splits) % TILE_K)) return ERR_BAD_ARGUMENT;
   if (gated)
-    return out_is_float ? launch_tiled<float, true>(x, w, bias, bias_is_float, out, M, N, K, stream)
-                        : launch_tiled<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, stream);
-  return out_is_float ? launch_tiled<float, false>(x, w, bias, bias_is_float, out, M, N, K, stream)
-                      : launch_tiled<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, stream);
+    return out_is_float ? pick_tiled<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                        : pick_tiled<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+  return out_is_float ? pick_tiled<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
+                      : pick_tiled<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
 }
 
 // x, w bfloat16; out bfloat16 or float32.  Needs 1 <= M <= 64, K a multiple of 32, and with

@@ -53,7 +53,7 @@ _SIGNATURES = {
     "llmserve_gemm_generic": "pipipipiiiip",
     "llmserve_gemm_skinny": "pppipiiiiiip",
     "llmserve_gemm_medium": "pppipiiiiiip",
-    "llmserve_gemm_tiled": "pppipiiiiip",
+    "llmserve_gemm_tiled": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifip",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
     "llmserve_attention_can_fuse": "i",
@@ -290,6 +290,18 @@ class HipKernels:
                 best = splits
         return best
 
+    @staticmethod
+    def _tiled_splits(rows: int, out_features: int, in_features: int) -> int:
+        """Into how many parts of K the tiled product is cut when its float32 result may stay in
+        parts: as many (at most 8, K / parts a multiple of 256) as it takes for the 256 x 256 tiles
+        to number about 256, one for every CU."""
+        tiles = -(-rows // 256) * -(-out_features // 256)
+        best = 1
+        for splits in range(2, 9):
+            if in_features % (splits * 256) == 0 and tiles * (splits - 1) < 256:
+                best = splits
+        return best
+
     def linear(
         self, x: torch.Tensor, weights: LinearWeights, out_dtype: torch.dtype | None = None, *, partial: bool = False
     ) -> torch.Tensor:
@@ -323,14 +335,17 @@ class HipKernels:
         bias_is_float = _is_float(bias) if bias is not None else 0
         if streaming is not None:
             splits = 1
-            if partial and out_dtype == torch.float32 and streaming != "tiled":
-                splits = self._partial_splits(weights.out_features, inner)
+            if partial and out_dtype == torch.float32:
+                if streaming == "tiled":
+                    splits = self._tiled_splits(rows, weights.out_features, inner)
+                else:
+                    splits = self._partial_splits(weights.out_features, inner)
             shape = (rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features)
             out = self._empty(shape, out_dtype or self.dtype)
             if streaming == "tiled":
                 status = self._gemm_bf16.llmserve_gemm_tiled(
                     _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out),
-                    _is_float(out), 0, rows, weights.out_features, inner, self._stream,
+                    _is_float(out), 0, rows, weights.out_features, inner, splits, self._stream,
                 )
             else:
                 entry = self._gemm_bf16.llmserve_gemm_skinny if streaming == "skinny" else self._gemm_bf16.llmserve_gemm_medium
@@ -355,7 +370,7 @@ class HipKernels:
             if streaming == "tiled":
                 status = self._gemm_bf16.llmserve_gemm_tiled(
                     _pointer(x), _pointer(weights.both.weight), None, 0, _pointer(out), _is_float(out), 1,
-                    x.shape[0], 2 * weights.width, x.shape[1], self._stream,
+                    x.shape[0], 2 * weights.width, x.shape[1], 1, self._stream,
                 )
                 _check(status, "gated_linear")
                 return out
@@ -410,7 +425,7 @@ class HipKernels:
             raise KernelError("paged_attention: queries and pages differ in type")
         out = self._empty((tokens, layout.num_heads * layout.head_dim), qkv.dtype)
         dim = layout.head_dim
-        if qkv.dtype == torch.bfloat16 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
+        if qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
             self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0))
             return out
         status = self._attention_generic.llmserve_attention_generic(
@@ -424,8 +439,8 @@ class HipKernels:
 
     def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None) -> None:
         """The MFMA kernel: requests that bring a few tokens (decoding) one column tile per
-        wave, split over the keys when there are few of them; longer portions four tiles per
-        wave.  `fuse` = (rotary table, pairing) lets a step of single tokens rotate and
+        wave, split over the keys when there are few of them; longer portions two or four
+        tiles per wave.  `fuse` = (rotary table, pairing) lets a step of single tokens rotate and
         store inside the same kernel."""
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
@@ -434,7 +449,10 @@ class HipKernels:
         tokens = qkv.shape[0]
         launches = [(1, *self._attention_work(batch, per_tile, 0, per_tile))]
         if batch.max_query_length > per_tile:
-            launches.append((4, *self._attention_work(batch, 4 * per_tile, per_tile, None)))
+            # four column tiles a wave halve the cache traffic of two, at one wave a SIMD instead of
+            # two: that pays once the keys no longer fit the chiplets' L2
+            wide = 4 if batch.max_context_length >= 4096 else 2
+            launches.append((wide, *self._attention_work(batch, wide * per_tile, per_tile, None)))
         for column_tiles, work, items in launches:
             if items == 0:
                 continue
@@ -470,7 +488,7 @@ class HipKernels:
             and cell.writable
             and qkv.dtype == torch.bfloat16
             and cell.keys.dtype == torch.bfloat16
-            and group.page_size % 4 == 0
+            and group.page_size % 8 == 0
             and dim % 16 == 0
             and 16 <= dim <= 256
             and self._attention_library(dim).llmserve_attention_can_fuse(_PAIRINGS[pairing])

@@ -101,11 +101,13 @@ def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
 
 @pytest.mark.parametrize("rows,inner,outer", [(17, 128, 64), (32, 256, 100), (33, 1536, 272), (64, 1280, 130), (64, 8960, 48),
                                               (40, 96, 77), (64, 160, 2048), (100, 256, 40), (65, 32, 128), (130, 1536, 272),
-                                              (300, 96, 1000), (2048, 512, 384), (129, 129, 50)])
+                                              (300, 96, 1000), (2048, 512, 384), (129, 129, 50), (2000, 64, 6500), (2048, 2048, 1500),
+                                              (1100, 2048, 700)])
 def test_products_without_the_library(own_kernels, rows, inner, outer):
     """17 to 64 rows: the kernel that shares x through LDS (K a multiple of 128), else the
-    weight-streaming one with several tiles of x; more rows: the tiled one (K a multiple of 32);
-    else the generic one; with partial sums too."""
+    weight-streaming one with several tiles of x; more rows: the tiled one (K a multiple of 32; its
+    256 x 256 tiles where there are 200 of them, K cut into partial sums where a float32 result
+    may stay in parts); else the generic one."""
     k, dtype = own_kernels, torch.bfloat16
     x, w, b = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer)
     expected = rounded(x, dtype) @ rounded(w, dtype).T + rounded(b, dtype)
@@ -177,7 +179,7 @@ def step_rows(per_request, counts, heads, kv_heads, dim):
 ATTENTION_SHAPES = [  # heads, kv_heads, dim, page
     (12, 2, 32, 16),  # the reference's own test shape (tests/test_triton_paged_attention.py:24)
     (6, 1, 48, 8),
-    (5, 5, 80, 4),
+    (5, 5, 80, 24),  # a page that is no power of two
     (8, 2, 128, 16),
     (3, 1, 112, 64),
     (4, 4, 16, 1),
@@ -251,6 +253,27 @@ def test_paged_attention_finds_a_far_key_among_hundreds(kernels, dtype):
         full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), 1.0)[-1]
         torch.testing.assert_close(out, full, **TOLERANCE[dtype])
         torch.testing.assert_close(out[0], rounded(v, dtype)[far, 0], atol=5e-2, rtol=0)
+
+
+@pytest.mark.parametrize("window", [None, 1500])
+def test_paged_attention_portion_of_a_long_context(kernels, window):
+    """Beyond 4,096 keys the bfloat16 kernel carries four column tiles a wave: a portion at the end of
+    such a context, with a far key that dominates and, with a window, lies just inside it."""
+    heads, kv_heads, dim, page, dtype = 6, 2, 64, 16, torch.bfloat16
+    lengths, counts = [4200, 37], [150, 37]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=3)
+    q, k, v = per_request[0]
+    far = 4199 - 1499 if window else 1
+    k[far] = 3.0 * q[-1, ::3]  # for heads 0 and 3 of the last query this key dominates
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    out = kernels[dtype].paged_attention(qkv, layout, batch, cell, 1.0, window).cpu().double()
+    expected = []
+    for (q, k, v), count in zip(per_request, counts):
+        full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), 1.0, window)
+        expected.append(full[-count:].flatten(1))
+    torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
+    torch.testing.assert_close(out[149].view(heads, dim)[0], rounded(per_request[0][2], dtype)[far, 0], atol=5e-2, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
