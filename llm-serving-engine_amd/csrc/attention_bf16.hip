@@ -96,8 +96,10 @@ __global__ __launch_bounds__(WAVES * 64, COLUMN_TILES > 2 ? 1 : 2) void attentio
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in all lanes: kept in a scalar register
   const int c = lane & 15, q = lane >> 4;
   // the work list runs from early to late tokens; late ones walk more keys, so they start first
+  // (when FUSED every request brings one token: tile i is request i and row i, nothing to look up)
   const int* item = work + (size_t)(gridDim.x - 1 - blockIdx.x) * 4;
-  const int request = item[0], row0 = item[1], tokens = item[2];
+  const int request = FUSED ? (int)blockIdx.x : item[0], row0 = FUSED ? (int)blockIdx.x : item[1];
+  const int tokens = FUSED ? 1 : item[2];
   const int position0 = positions[row0];
   const int last_key = position0 + tokens - 1;
   const int first_key = window > 0 ? max(0, position0 - window + 1) : 0;
@@ -454,7 +456,7 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // be a multiple of 8.  With splits > 1, partial_acc is float32 [rows * heads * splits * D],
 // partial_ml [rows * heads * splits * 2] (rows being the step's token count), and every row
 // of the step must lie in one of the tiles: a second kernel merges the splits of all rows.
-// With `fuse` every tile holds one token, qkv is as the projection left it, and the kernel
+// With `fuse` tile i is row i, the one token of request i (`work` is not read), qkv is as the projection left it, and the kernel
 // rotates (table of cos and sin per row, pairing) and stores the token's key and value at slots[row] itself.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
                                         float* partial_ml, void* keys, void* values,
@@ -472,7 +474,7 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   FusedDecode fused = {(const float2*)table, pairing, slots};
   int status;
   if (fuse) {
-    if (column_tiles != 1 || !slots || !llmserve_attention_can_fuse(pairing) || (pairing != 0 && !table))
+    if (column_tiles != 1 || tiles != rows || !slots || !llmserve_attention_can_fuse(pairing) || (pairing != 0 && !table))
       return ERR_BAD_ARGUMENT;
     status = launch_tiles<1, true, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
                                         table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile,
