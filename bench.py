@@ -55,17 +55,14 @@ def main() -> int:
     from llmserve_amd import CacheConfig, EngineCore, GenerationConfig, ModelRunner, Qwen2Config, SchedulerConfig, StepEntry
     from llmserve_amd.engine import RequestState
     from llmserve_amd.kernels import HipKernels
-    from llmserve_amd.registry import ARCHITECTURES
-    from llmserve_amd.weights import LoadedModel, random_tensors, run_dtype
+    from llmserve_amd.weights import random_model, run_dtype
 
     full = Qwen2Config.from_json_file(args.config)
     config = dataclasses.replace(full, num_layers=args.layers) if args.layers else full
     dtype = run_dtype(args.dtype)
-    architecture = ARCHITECTURES[config.architecture]
-    spec = architecture.build_spec(config)
     device = torch.device("cuda:0")
-    tensors = random_tensors(spec, args.seed, dtype=dtype, device=device)
-    loaded = LoadedModel(architecture, config, spec, tensors, dtype)
+    loaded = random_model(config, args.seed, dtype=dtype, device=device)
+    tensors = loaded.tensors
     kernels = HipKernels(dtype, device)
     page = 16
     most = max(64, args.batch)

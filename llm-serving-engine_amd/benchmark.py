@@ -32,8 +32,19 @@ class LengthDistribution:
 
 
 @dataclass(frozen=True)
+class RequestGroup:
+    """A run of consecutive requests with length distributions of their own."""
+
+    requests: int
+    prompt: LengthDistribution
+    output: LengthDistribution
+
+
+@dataclass(frozen=True)
 class LoadProfile:
-    """`workload.py:25-46` and configs/benchmark-sharegpt.yaml."""
+    """`workload.py:25-46` and configs/benchmark-sharegpt.yaml.  `groups`, which the reference
+    does not have, makes a mix: the first group's requests arrive first, then the second's, all
+    on the one arrival process; `requests` is then the groups' total."""
 
     requests: int = 100
     arrival_rate: float = 2.0
@@ -41,6 +52,28 @@ class LoadProfile:
     output: LengthDistribution = LengthDistribution(64, 0.7, 4, 256)
     seed: int = 7
     vocabulary_size: int = 32_000
+    groups: tuple[RequestGroup, ...] = ()
+
+    def __post_init__(self) -> None:
+        if self.groups and sum(group.requests for group in self.groups) != self.requests:
+            raise ValueError("requests must be the sum of the groups' requests")
+
+    def distributions(self) -> list[tuple[LengthDistribution, LengthDistribution]]:
+        """(prompt, output) distributions of every request, in arrival order."""
+        if not self.groups:
+            return [(self.prompt, self.output)] * self.requests
+        return [(group.prompt, group.output) for group in self.groups for _ in range(group.requests)]
+
+    def fitted(self, longest_sequence: int) -> "LoadProfile":
+        """The same profile with prompts clipped so that prompt plus output fit `longest_sequence`."""
+        from dataclasses import replace
+
+        def clip(prompt: LengthDistribution, output: LengthDistribution) -> LengthDistribution:
+            return replace(prompt, maximum=max(1, min(prompt.maximum, longest_sequence - output.maximum)),
+                           minimum=max(1, min(prompt.minimum, longest_sequence - output.maximum)))
+
+        groups = tuple(replace(group, prompt=clip(group.prompt, group.output)) for group in self.groups)
+        return replace(self, prompt=clip(self.prompt, self.output), groups=groups)
 
     @classmethod
     def from_yaml(cls, path: str | Path) -> "LoadProfile":
@@ -48,13 +81,19 @@ class LoadProfile:
 
         with Path(path).open() as handle:
             values = yaml.safe_load(handle)
+        groups = tuple(
+            RequestGroup(group["requests"], LengthDistribution(**group["prompt"]), LengthDistribution(**group["output"]))
+            for group in values.get("groups", ())
+        )
+        defaults = cls()
         return cls(
-            requests=values["requests"],
+            requests=values.get("requests", sum(group.requests for group in groups) or defaults.requests),
             arrival_rate=values["arrival_rate"],
-            prompt=LengthDistribution(**values["prompt"]),
-            output=LengthDistribution(**values["output"]),
+            prompt=LengthDistribution(**values["prompt"]) if "prompt" in values else defaults.prompt,
+            output=LengthDistribution(**values["output"]) if "output" in values else defaults.output,
             seed=values.get("seed", 7),
             vocabulary_size=values.get("vocabulary_size", 32_000),
+            groups=groups,
         )
 
     def to_dict(self) -> dict[str, object]:
@@ -78,11 +117,11 @@ def generate_workload(profile: LoadProfile) -> list[RequestSpec]:
     rng = random.Random(profile.seed)
     at = 0.0
     specs = []
-    for index in range(profile.requests):
+    for index, (prompt_lengths, output_lengths) in enumerate(profile.distributions()):
         if index:
             at += rng.expovariate(profile.arrival_rate)
-        prompt_length = profile.prompt.sample(rng)
-        output_length = profile.output.sample(rng)
+        prompt_length = prompt_lengths.sample(rng)
+        output_length = output_lengths.sample(rng)
         prompt = tuple(rng.randrange(4, profile.vocabulary_size) for _ in range(prompt_length))
         specs.append(RequestSpec(f"request-{index:06d}", at, prompt, output_length))
     return specs

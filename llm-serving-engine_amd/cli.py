@@ -24,12 +24,18 @@ ROOT = Path(__file__).resolve().parent.parent
 
 
 def _load_runtime(args):
-    """A model folder, or without --model the bundled tiny configuration with weights drawn
-    from --seed and the byte tokenizer (`cli.py:22-45`)."""
+    """A model folder; or weights drawn from --seed at the sizes of a config.json
+    (--random-weights, made on the device: no folder is written); or without either the
+    bundled tiny configuration with such weights and the byte tokenizer (`cli.py:22-45`)."""
     from .config import Qwen2Config
     from .engine.tokenizer import ByteTokenizer, FileTokenizer
-    from .weights import load_model_folder, write_model_folder
+    from .weights import load_model_folder, random_model, write_model_folder
 
+    if args.model and getattr(args, "random_weights", None):
+        raise SystemExit("give --model or --random-weights, not both")
+    if getattr(args, "random_weights", None):
+        device = args.device if args.device != "auto" else "cuda:0"
+        return random_model(args.random_weights, args.seed, dtype=args.dtype, device=device), ByteTokenizer()
     if args.model:
         loaded = load_model_folder(args.model, args.dtype)
         try:
@@ -67,14 +73,14 @@ async def _benchmark(args) -> None:
 
     loaded, tokenizer = _load_runtime(args)
     profile = LoadProfile.from_yaml(args.profile)
-    longest = loaded.config.max_position_embeddings
+    if args.requests and profile.groups:
+        raise SystemExit("--requests cannot change a profile made of groups")
     profile = replace(
         profile,
         requests=args.requests or profile.requests,
         arrival_rate=args.arrival_rate or profile.arrival_rate,
         vocabulary_size=loaded.config.vocab_size,
-        prompt=replace(profile.prompt, maximum=min(profile.prompt.maximum, longest - profile.output.maximum)),
-    )
+    ).fitted(loaded.config.max_position_embeddings)
     harness = BenchmarkHarness(profile)
     batch_size = 1 if args.config in ("naive", "paged") else args.batch_size
     engine = _engine(args, loaded, tokenizer, batch_size=batch_size, mode="static" if args.config == "static" else "continuous")
@@ -147,6 +153,8 @@ def _random_model(args) -> None:
 
 def _engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--model", help="model folder with config.json and safetensors files")
+    parser.add_argument("--random-weights", metavar="CONFIG_JSON",
+                        help="instead of --model: weights drawn from --seed at the sizes of this config.json")
     parser.add_argument("--device", default="auto")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--block-size", type=int, default=16)

@@ -69,6 +69,33 @@ def random_tensors(
     return tensors
 
 
+def random_model(
+    config: ArchitectureConfig | dict | str | Path,
+    seed: int,
+    *,
+    dtype: Any = torch.bfloat16,
+    device: str | torch.device = "cpu",
+    **scales: float,
+):
+    """A model with seeded random weights made in memory, on `device`: `config` is a typed
+    configuration, the mapping of a config.json, or the path of one (its architecture is
+    resolved as for a model folder).  Large configurations need no folder on disk this way."""
+    from ..registry import resolve_architecture
+    from .loader import LoadedModel, run_dtype
+
+    if isinstance(config, (str, Path)):
+        config = json.loads(Path(config).read_text())
+    if isinstance(config, dict):
+        architecture = resolve_architecture(config)
+        config = architecture.config_class.from_dict(config)
+    else:
+        architecture = ARCHITECTURES[config.architecture]
+    dtype = run_dtype(dtype)
+    spec = architecture.build_spec(config)
+    tensors = random_tensors(spec, seed, dtype=dtype, device=device, **scales)
+    return LoadedModel(architecture, config, spec, tensors, dtype)
+
+
 def write_model_folder(
     folder: str | Path,
     config: ArchitectureConfig,

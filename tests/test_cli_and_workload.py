@@ -104,3 +104,26 @@ def test_bench_measures_one_gpu_only():
 
     done = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert done.returncode == 2 and len(done.stdout.strip().splitlines()) == 1 and "one GPU" in done.stdout
+
+
+def test_workload_groups_arrive_in_order_and_fit_the_context():
+    """A profile made of groups: the groups' requests come one group after the other on the one
+    arrival process, lengths from each group's own distributions; `fitted` clips prompts so that
+    prompt plus output stay within the longest sequence."""
+    from llmserve_amd.benchmark import LengthDistribution, LoadProfile, RequestGroup, generate_workload
+
+    short = RequestGroup(5, LengthDistribution(20, 0.5, 4, 40), LengthDistribution(100, 0.1, 90, 110))
+    long = RequestGroup(3, LengthDistribution(600, 0.0, 600, 600), LengthDistribution(8, 0.0, 8, 8))
+    profile = LoadProfile(requests=8, arrival_rate=10.0, groups=(short, long), vocabulary_size=50)
+    specs = generate_workload(profile)
+    assert [len(spec.prompt_token_ids) <= 40 for spec in specs] == [True] * 5 + [False] * 3
+    assert [len(spec.prompt_token_ids) for spec in specs[5:]] == [600] * 3
+    assert all(90 <= spec.max_new_tokens <= 110 for spec in specs[:5]) and all(spec.max_new_tokens == 8 for spec in specs[5:])
+    assert [spec.arrival_offset_s for spec in specs] == sorted(spec.arrival_offset_s for spec in specs)
+    assert specs == generate_workload(profile)
+    fitted = generate_workload(profile.fitted(500))
+    assert [len(spec.prompt_token_ids) for spec in fitted[5:]] == [492] * 3
+    with pytest.raises(ValueError):
+        LoadProfile(requests=7, groups=(short, long))
+    mix = LoadProfile.from_yaml(ROOT / "configs" / "workload-long-context-mix.yaml")
+    assert mix.requests == 64 and [group.requests for group in mix.groups] == [48, 16]
