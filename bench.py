@@ -62,7 +62,7 @@ def main() -> int:
     dtype = run_dtype(args.dtype)
     device = torch.device("cuda:0")
     loaded = random_model(config, args.seed, dtype=dtype, device=device)
-    tensors = loaded.tensors
+    tensors, spec = loaded.tensors, loaded.spec
     kernels = HipKernels(dtype, device)
     page = 16
     most = max(64, args.batch)
