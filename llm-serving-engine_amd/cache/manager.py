@@ -263,6 +263,23 @@ class CacheManager:
             self._high_water = {"pages": used, "used_tokens": self._used_tokens, "sequences": len(self.sequences)}
         return Reservation(request_id, record.slot, start, count, tuple(slots))
 
+    def cancel(self, reservation: Reservation) -> None:
+        """Takes back the request's latest reservation, whose entries were never written: the
+        request is as long as before, and pages that the reservation began are free again.
+        (Pages that a window had passed stay given back: no later query reads them.)"""
+        record = self.sequences[reservation.request_id]
+        if record.length != reservation.start + reservation.count:
+            raise ValueError(f"not the latest reservation of {reservation.request_id!r}")
+        first_new = -(-reservation.start // self.page_size)
+        end_new = -(-record.length // self.page_size)
+        for group in self.groups:
+            table = group.tables[record.slot]
+            for block in range(first_new, end_new):
+                group.pool.free(int(table[block]), reservation.request_id)
+                table[block] = -1
+        record.length = reservation.start
+        self._used_tokens -= reservation.count
+
     def block_table(self, request_id: str, group: int = 0) -> list[int]:
         record = self.sequences[request_id]
         blocks = math.ceil(record.length / self.page_size)

@@ -44,6 +44,7 @@ class EngineCore:
         scheduler_mode: str = "continuous",
         prefill_chunk_size: int = 16,
         collect_iteration_metrics: bool = False,
+        look_ahead: bool = True,
     ) -> None:
         scheduler_config = scheduler_config or SchedulerConfig()
         if prefill_chunk_size <= 0:
@@ -58,6 +59,8 @@ class EngineCore:
         self.prefill_chunk_size = prefill_chunk_size
         self.sampler = Sampler(runner.kernels)
         self.collect_iteration_metrics = collect_iteration_metrics
+        self.look_ahead = look_ahead  # prepare the next decode step on the host while the device runs this one
+        self._expected: list[RequestState] | None = None  # the requests of the step that is prepared
         self.generation_configs: dict[str, GenerationConfig] = {}
         self.finished: list[RequestState] = []
         self._cpu_ms = {"prefill": 0.0, "decode": 0.0, "mixed": 0.0}
@@ -136,23 +139,17 @@ class EngineCore:
                     self._events[phase].append(events)
 
     def _run_iteration(self, active: list[RequestState]) -> list[TokenEvent]:
-        planned = plan_iteration(active, self.scheduler_config.max_tokens_per_step, self.prefill_chunk_size)
-        cache = self.runner.cache
-
-        def as_plan(items):
-            return [(request.request_id, count) for request, count in items]
-
-        # Pages run out: requests give way (never the oldest) until the rest fits.
-        while not cache.fits(as_plan(planned)) and len(planned) > 1:
-            victim = choose_victim(planned, self.scheduler_config.preemption)
-            self.runner.end_request(victim.request_id)
-            self.scheduler.preempt(victim)
-            planned = [item for item in planned if item[0] is not victim]
-        if not cache.fits(as_plan(planned)):
-            self.finish(planned[0][0], CacheFullError("one sequence exceeds total KV cache capacity"))
-            return []
+        expected, self._expected = self._expected, None
+        if expected is not None and len(expected) == len(active) and all(a is b for a, b in zip(expected, active)):
+            # the step that was prepared while the last one ran: every request brings the token it
+            # has just been given, and the runner holds the cache entries already
+            planned = [(request, 1) for request in active]
+        else:
+            planned = self._plan(active)
+            if planned is None:
+                return []
         if self.step_log is not None:
-            self.step_log.append(as_plan(planned))
+            self.step_log.append([(request.request_id, count) for request, count in planned])
 
         entries, sampled = [], []
         for request, count in planned:
@@ -168,6 +165,13 @@ class EngineCore:
             return []
         configs = [self.generation_configs[request.request_id] for request in sampled]
         steps = [len(request.generated_token_ids) for request in sampled]
+        if self.look_ahead and len(sampled) == len(planned) == len(active) and not self.scheduler.waiting:
+            # Every running request has just decoded and nothing waits: unless a stop token comes,
+            # the next step is these requests again, less those at their last token.  The runner does
+            # its host work for that step now, while the device is still busy with this one.
+            staying = [r for r in sampled if len(r.generated_token_ids) + 1 < r.max_new_tokens]
+            if self.runner.prepare_decode([r.request_id for r in staying]):
+                self._expected = staying
         tokens = self.sampler.sample(logits, configs, steps)
         produced = []
         for request, config, token in zip(sampled, configs, tokens):
@@ -176,6 +180,24 @@ class EngineCore:
             if len(request.generated_token_ids) >= request.max_new_tokens or token in config.stop_token_ids:
                 self.finish(request)
         return produced
+
+    def _plan(self, active: list[RequestState]) -> list[tuple[RequestState, int]] | None:
+        """Who brings how many tokens to this step; requests give way until it fits the cache."""
+        planned = plan_iteration(active, self.scheduler_config.max_tokens_per_step, self.prefill_chunk_size)
+
+        def as_plan(items):
+            return [(request.request_id, count) for request, count in items]
+
+        # Pages run out: requests give way (never the oldest) until the rest fits.
+        while not self.runner.fits(as_plan(planned)) and len(planned) > 1:
+            victim = choose_victim(planned, self.scheduler_config.preemption)
+            self.runner.end_request(victim.request_id)
+            self.scheduler.preempt(victim)
+            planned = [item for item in planned if item[0] is not victim]
+        if not self.runner.fits(as_plan(planned)):
+            self.finish(planned[0][0], CacheFullError("one sequence exceeds total KV cache capacity"))
+            return None
+        return planned
 
     # ------------------------------------------------------------------ synchronous use
 

@@ -178,9 +178,14 @@ class ModelRunner:
         self.vocab_size = loaded.spec.vocab_size
         self.use_graphs = self.device.type == "cuda" if use_graphs is None else use_graphs
         self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        # What `prepare_decode` has done for the step to come: each request's reservation of one
+        # token, and, where decode steps replay a graph, the step's index arrays already packed.
+        self._ahead: dict[str, Reservation] = {}
+        self._packed_ahead: tuple | None = None
 
     def close(self) -> None:
         """Drops the captured graphs (while the device runtime is still up)."""
+        self._packed_ahead = None
         if self._graphs:
             torch.cuda.synchronize(self.device)
         self._graphs.clear()
@@ -189,7 +194,41 @@ class ModelRunner:
         return self.cache.create(request_id)
 
     def end_request(self, request_id: str) -> None:
+        self._ahead.pop(request_id, None)  # its pages go with the rest
         self.cache.free(request_id)
+
+    def fits(self, plan: list[tuple[str, int]]) -> bool:
+        """The cache's `fits` for the step to come; a token that `prepare_decode` has reserved
+        already is not counted again."""
+        if not self._ahead:
+            return self.cache.fits(plan)
+        return self.cache.fits([(request_id, count - (1 if request_id in self._ahead else 0)) for request_id, count in plan])
+
+    def prepare_decode(self, request_ids: list[str]) -> bool:
+        """Does the host's share of the next step ahead of time, while the device is busy with
+        the current one: the step in which each of `request_ids` brings one token and wants its
+        logits.  Cache entries are reserved, and the index arrays packed where the step will be
+        replayed from a graph; the tokens themselves come with `step`.  A step that turns out
+        otherwise costs nothing: reservations of requests it holds are used, the others are
+        taken back.  Returns False, having done nothing, if the cache has no room."""
+        self._cancel_ahead()
+        if not request_ids or self.cache.states:
+            return False
+        plan = [(request_id, 1) for request_id in request_ids]
+        if any(request_id not in self.cache.sequences for request_id in request_ids) or not self.cache.fits(plan):
+            return False
+        reservations = [self.cache.reserve(request_id, 1, checked=True) for request_id in request_ids]
+        self._ahead = {r.request_id: r for r in reservations}
+        if self.use_graphs:
+            entries = [StepEntry(request_id, (0,), (0,)) for request_id in request_ids]
+            self._packed_ahead = (tuple(request_ids), *self._pack_decode(reservations, entries))
+        return True
+
+    def _cancel_ahead(self) -> None:
+        for reservation in self._ahead.values():
+            self.cache.cancel(reservation)
+        self._ahead.clear()
+        self._packed_ahead = None
 
     def has_request(self, request_id: str) -> bool:
         return request_id in self.cache.sequences
@@ -203,6 +242,18 @@ class ModelRunner:
         says that the caller has asked the cache's `fits` for exactly these entries."""
         if not entries:
             raise ValueError("a step needs at least one entry")
+        ahead = self._packed_ahead
+        if ahead is not None and len(entries) == len(ahead[0]) and all(
+            entry.request_id == request_id and len(entry.tokens) == 1 and tuple(entry.want) == (0,)
+            for entry, request_id in zip(entries, ahead[0])
+        ):  # the step that `prepare_decode` was told to expect: only the tokens are new
+            tokens = [entry.tokens[0] for entry in entries]
+            if min(tokens) < 0 or max(tokens) >= self.vocab_size:
+                raise ValueError("a token is outside the vocabulary")
+            reservations = [self._ahead[request_id] for request_id in ahead[0]]
+            self._ahead.clear()
+            self._packed_ahead = None
+            return self._decode_with_graph(reservations, entries, ahead[1:])
         seen = set()
         for entry in entries:
             if entry.request_id in seen:
@@ -224,14 +275,24 @@ class ModelRunner:
                     self.add_request(entry.request_id)
                     created.append(entry.request_id)
             plan = [(entry.request_id, len(entry.tokens)) for entry in entries]
-            if not fits_checked and not self.cache.fits(plan):
+            if not fits_checked and not self.fits(plan):
                 raise CacheFullError("the step's tokens do not fit the cache")
         except Exception:
             for request_id in created:
                 self.end_request(request_id)
             raise
-        reservations = [self.cache.reserve(request_id, count, checked=True) for request_id, count in plan]
+        packed_ahead, self._packed_ahead = self._packed_ahead, None
+        reservations = []
+        for request_id, count in plan:
+            ahead = self._ahead.pop(request_id, None)
+            if ahead is not None and count != 1:
+                self.cache.cancel(ahead)
+                ahead = None
+            reservations.append(ahead or self.cache.reserve(request_id, count, checked=True))
+        self._cancel_ahead()  # requests that were expected and did not come
         if self.use_graphs and not self.cache.states and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
+            if packed_ahead is not None and packed_ahead[0] == tuple(entry.request_id for entry in entries):
+                return self._decode_with_graph(reservations, entries, packed_ahead[1:])
             return self._decode_with_graph(reservations, entries)
         batch = build_step_batch(reservations, entries, self.cache, self.device)
         return self.forward(batch)
@@ -257,17 +318,26 @@ class ModelRunner:
             size *= 2
         return size
 
-    @torch.inference_mode()
-    def _decode_with_graph(self, reservations: list[Reservation], entries: list[StepEntry]) -> torch.Tensor:
-        """A step of single tokens, one per request, replayed from a HIP graph: the launches
-        of a decode step cost more on the host than the step takes on the device.  Graphs are
-        kept per (requests rounded up to a power of two, block-table width likewise); the
-        step's index arrays go into the graph's static buffer and the same kernels run."""
+    def _pack_decode(self, reservations: list[Reservation], entries: list[StepEntry]):
+        """The index arrays of a step of single tokens, padded to its graph's shape; first the graph's key."""
         requests = self._bucket(len(reservations))
         blocks = max(-(-(r.start + 1) // self.cache.page_size) for r in reservations)
         width = min(self._bucket(blocks), self._bucket(self.cache.max_blocks_per_sequence))
-        key = (requests, width)
-        packed, sizes, widths, facts = _pack_step(reservations, entries, self.cache, pad_to=requests, width=width)
+        return ((requests, width), *_pack_step(reservations, entries, self.cache, pad_to=requests, width=width))
+
+    @torch.inference_mode()
+    def _decode_with_graph(self, reservations: list[Reservation], entries: list[StepEntry], packed_ahead=None) -> torch.Tensor:
+        """A step of single tokens, one per request, replayed from a HIP graph: the launches
+        of a decode step cost more on the host than the step takes on the device.  Graphs are
+        kept per (requests rounded up to a power of two, block-table width likewise); the
+        step's index arrays go into the graph's static buffer and the same kernels run.
+        `packed_ahead` is what `_pack_decode` made of the same reservations before the tokens
+        were known: the token ids, which lead the arrays, are filled in."""
+        if packed_ahead is not None:
+            key, packed, sizes, widths, facts = packed_ahead
+            packed[: len(entries)] = [entry.tokens[0] for entry in entries]
+        else:
+            key, packed, sizes, widths, facts = self._pack_decode(reservations, entries)
         graph = self._graphs.get(key)
         if graph is None:
             graph = self._capture(key, packed, sizes, widths, facts)

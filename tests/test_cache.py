@@ -154,9 +154,18 @@ def test_random_orders_lose_nothing(config, block):
             count = rng.choice([1, 1, 1, 2, 3, 7, 16, 33])
             fits = cache.fits([(name, count)])
             if fits:
+                before = (cache.used_pages, cache.stats(200)["used_tokens"])
                 reservation = cache.reserve(name, count)
                 assert reservation.start == live[name]
-                live[name] += count
+                if rng.random() < 0.25:  # taken back unused: as if it had never been made
+                    cache.cancel(reservation)
+                    # (a page that the window has passed at this position stays given back)
+                    assert cache.used_pages <= before[0] and cache.stats(200)["used_tokens"] == before[1]
+                    assert cache.sequences[name].length == live[name]
+                    with pytest.raises(ValueError):
+                        cache.cancel(reservation)
+                else:
+                    live[name] += count
             else:
                 before = cache.used_pages
                 with pytest.raises(CacheFullError):

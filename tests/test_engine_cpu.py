@@ -244,6 +244,40 @@ def test_pages_run_out_the_largest_gives_way_and_replays(model_folders):
     assert core.runner.cache.used_pages == 0
 
 
+def test_looking_ahead_changes_no_decision(model_folders):
+    """While a decode step runs, the engine has the runner reserve and pack the next one.  With
+    requests that arrive late, stop early and give way for want of pages, every plan and every
+    token is what it is without looking ahead, and nothing stays reserved."""
+    config, weights = oracle(model_folders, "A")
+    prompts = [random_tokens(n, config.vocab_size, seed=70 + n) for n in (20, 9, 26, 3)]
+    free_run = [plain.generate(weights, config, prompt, 12) for prompt in prompts]
+    stops = [(), (free_run[1][9],), (free_run[2][2],), ()]  # two requests stop on a token of their own
+    outcomes = []
+    for look_ahead in (True, False):
+        core = core_for(model_folders, "A", num_blocks=3, batch=3, budget=12, chunk=8)
+        core.look_ahead = look_ahead
+        requests = [RequestState(f"r{i}", prompt, 12) for i, prompt in enumerate(prompts)]
+        for request, stop in zip(requests[:2], stops):
+            core.submit(request, GenerationConfig(max_new_tokens=12, stop_token_ids=stop))
+        steps = 0
+        while core.has_work or steps < 8:
+            if steps == 4:
+                core.submit(requests[2], GenerationConfig(max_new_tokens=12, stop_token_ids=stops[2]))
+            if steps == 7:
+                core.submit(requests[3], GenerationConfig(max_new_tokens=12))
+            core.step()
+            core.runner.cache.check_invariants()
+            steps += 1
+        assert not core.runner._ahead and core.runner.cache.used_pages == 0
+        assert all(request.error is None for request in requests)
+        outcomes.append((core.step_log, [r.generated_token_ids for r in requests], [r.preemptions for r in requests]))
+    assert outcomes[0] == outcomes[1]
+    assert sum(outcomes[0][2]) > 0  # pages did run out
+    for tokens, whole, stop in zip(outcomes[0][1], free_run, stops):
+        cut = whole.index(stop[0]) + 1 if stop else len(whole)
+        assert tokens == whole[:cut]
+
+
 def test_a_request_that_can_never_fit_fails_alone(model_folders):
     """reference tests/test_engine.py:261-277"""
     core = core_for(model_folders, "A", num_blocks=2, batch=2)
