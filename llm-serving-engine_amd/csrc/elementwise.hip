@@ -56,6 +56,23 @@ __global__ void add_rms_norm_kernel(float* __restrict__ hidden, const float* __r
 // The same for rows of up to 256 * 4 * VECTORS floats whose length is a multiple of 4: the row
 // stays in registers between the two passes and moves in 16-byte pieces.
 #define NORM_VECTORS 8
+template <int PARTS>
+__device__ __forceinline__ void add_parts(float4 (&v)[NORM_VECTORS], const float* from, size_t part_stride, int quads) {
+#pragma unroll
+  for (int j = 0; j < NORM_VECTORS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < quads) {
+      float4 d[PARTS];
+#pragma unroll
+      for (int p = 0; p < PARTS; ++p) d[p] = ((const float4*)(from + (size_t)p * part_stride))[i];
+#pragma unroll
+      for (int p = 0; p < PARTS; ++p) {
+        v[j].x += d[p].x; v[j].y += d[p].y; v[j].z += d[p].z; v[j].w += d[p].w;
+      }
+    }
+  }
+}
+
 template <typename TO>
 __global__ __launch_bounds__(256) void add_rms_norm_vector_kernel(float* __restrict__ hidden,
                                                                   const float* __restrict__ delta, int parts,
@@ -83,15 +100,18 @@ __global__ __launch_bounds__(256) void add_rms_norm_vector_kernel(float* __restr
     }
   }
   if (add) {
-    for (int p = 0; p < parts; ++p) {
-      const float4* part = (const float4*)(add + p * part_stride);
-#pragma unroll
-      for (int j = 0; j < NORM_VECTORS; ++j) {
-        const int i = threadIdx.x + j * 256;
-        if (i < quads) {
-          const float4 d = part[i];
-          v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
-        }
+    // the parts are added in order, up to eight at a time: their loads are all requested before the first is used
+    for (int first = 0; first < parts; first += 8) {
+      const float* from = add + (size_t)first * part_stride;
+      switch (min(parts - first, 8)) {
+        case 1: add_parts<1>(v, from, part_stride, quads); break;
+        case 2: add_parts<2>(v, from, part_stride, quads); break;
+        case 3: add_parts<3>(v, from, part_stride, quads); break;
+        case 4: add_parts<4>(v, from, part_stride, quads); break;
+        case 5: add_parts<5>(v, from, part_stride, quads); break;
+        case 6: add_parts<6>(v, from, part_stride, quads); break;
+        case 7: add_parts<7>(v, from, part_stride, quads); break;
+        default: add_parts<8>(v, from, part_stride, quads); break;
       }
     }
   }
@@ -264,8 +284,15 @@ __global__ void gather_rows_kernel(const float* __restrict__ hidden, const float
   float* dst = out + (size_t)blockIdx.x * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = hidden[src + i];
-    if (delta)
-      for (int p = 0; p < parts; ++p) v += delta[p * part_stride + src + i];
+    if (delta) {
+      for (int first = 0; first < parts; first += 8) {  // eight loads in flight, added in order
+        float d[8];
+#pragma unroll
+        for (int p = 0; p < 8; ++p) d[p] = first + p < parts ? delta[(size_t)(first + p) * part_stride + src + i] : 0.f;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) v += d[p];
+      }
+    }
     dst[i] = v;
   }
 }
