@@ -464,12 +464,197 @@ static int launch_tiled(const void* x, const void* w, const void* bias, int bias
   return LAUNCH_STATUS();
 }
 
+// ---------------------------------------------------------------------------- many rows, wide tiles
+// gemm_wide: the tiled product with a 256 x 256 tile, steps of 64 over K, and both operands brought
+// from global memory straight into LDS (global_load_lds_dwordx4: a wave's 64 lanes fill 1 KB of LDS
+// in lane order, no registers in between), two stages: the next step's 64 KB are under way while
+// the current step is multiplied.  A staged row is 128 bytes = 8 pieces of 16; piece p of row r lies
+// in slot p ^ (r & 7), so that the eight lanes that read one piece of eight consecutive rows for an
+// MFMA operand hit eight different slots (no bank conflict), while the writes stay in lane order.
+// Each of the four waves (2 x 2) owns 4 x 4 tiles of v_mfma_f32_32x32x16_bf16: 256 accumulators.
+#define WIDE_TILE 256
+#define WIDE_K 64
+
+__device__ __forceinline__ void wide_stage(const bf16_t* __restrict__ from, int rows_total, int row0, int ld, int k0,
+                                           bf16_t* staged, int wave, int lane) {
+  // 256 rows x 8 pieces = 2048 pieces of 16 bytes; wave w, instruction i fills pieces (w * 8 + i) * 64 + lane
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int piece = (wave * 8 + i) * 64 + lane;
+    const int row = piece >> 3, slot = piece & 7;
+    const int part = slot ^ (row & 7);
+    const bf16_t* src = from + (size_t)min(row0 + row, rows_total - 1) * ld + k0 + part * 8;
+    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                     (void __attribute__((address_space(3)))*)(staged + (size_t)(wave * 8 + i) * 512),
+                                     16, 0, 0);
+  }
+}
+
+template <typename TO, bool GATED>
+__global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                        const void* __restrict__ bias, int bias_is_float,
+                                                        TO* __restrict__ out, int M, int N, int K, int k_split) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t staged[];  // [2 stages][w, x][256 rows][64]
+  constexpr int OPERAND = WIDE_TILE * WIDE_K;  // elements of one staged operand
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int wave_n = wave & 1, wave_m = wave >> 1;
+  const int n0 = blockIdx.x * WIDE_TILE, m0 = blockIdx.y * WIDE_TILE;
+  const int k_first = blockIdx.z * k_split;
+  const int r32 = lane & 31, half = lane >> 5;
+
+  f32x16 acc[4][4];  // [tile of weight rows][tile of x rows]
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int steps = k_split / WIDE_K;
+  wide_stage(w, N, n0, K, k_first, staged, wave, lane);
+  wide_stage(x, M, m0, K, k_first, staged + OPERAND, wave, lane);
+  for (int step = 0; step < steps; ++step) {
+    bf16_t* now = staged + (size_t)(step & 1) * 2 * OPERAND;
+    if (step + 1 < steps) {
+      bf16_t* next = staged + (size_t)((step + 1) & 1) * 2 * OPERAND;
+      wide_stage(w, N, n0, K, k_first + (step + 1) * WIDE_K, next, wave, lane);
+      wide_stage(x, M, m0, K, k_first + (step + 1) * WIDE_K, next + OPERAND, wave, lane);
+      __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): this step's pieces have landed, the next step's 16 may be out
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    }
+    __syncthreads();
+    const bf16_t* from_w = now + (size_t)(wave_n * 128 + r32) * WIDE_K;
+    const bf16_t* from_x = now + OPERAND + (size_t)(wave_m * 128 + r32) * WIDE_K;
+    // this lane's piece of a row in sub-step kk: part kk * 2 + half, in slot part ^ (row & 7); rows r32 + 32 i
+    // keep r32 & 7.  The operands of sub-step kk + 1 are read from LDS while sub-step kk is multiplied.
+    bf16x8 a[2][4], b[2][4];
+    auto read_operands = [&](int kk, bf16x8 (&a_now)[4], bf16x8 (&b_now)[4]) {
+      const int slot = ((kk * 2 + half) ^ (r32 & 7)) * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a_now[i] = *(const bf16x8*)(from_w + (size_t)i * 32 * WIDE_K + slot);
+        b_now[i] = *(const bf16x8*)(from_x + (size_t)i * 32 * WIDE_K + slot);
+      }
+    };
+    read_operands(0, a[0], b[0]);
+#pragma unroll
+    for (int kk = 0; kk < WIDE_K / 16; ++kk) {
+      if (kk + 1 < WIDE_K / 16) read_operands(kk + 1, a[(kk + 1) & 1], b[(kk + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);  // the reads stay in front of this sub-step's products: one wave a SIMD, nobody else hides their latency
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk & 1][i], b[kk & 1][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();  // everyone has read this stage: the step after next may be written over it
+  }
+
+  // D[n][m] of a 32 x 32 tile: lane holds column m = lane % 32 and rows n = 8 * (e / 4) + 4 * (lane / 32) + e % 4,
+  // so a lane's values lie in 32 different rows of `out`.  They go through LDS (the stages are free
+  // now), 32 rows of x at a time, and leave as whole rows: 16 lanes write the 128 columns of a row.
+  const bool with_bias = bias && blockIdx.z == 0;
+  constexpr int ROW = 128 + 4;  // floats of a transposed row, padded
+  float* mine = (float*)staged + (size_t)wave * 32 * ROW;  // [32 m][128 n] of this wave
+  const int piece = lane & 15, row_in_pass = lane >> 4;    // this lane's 8 columns; 4 rows a pass
+  const int n_piece = n0 + wave_n * 128 + piece * 8;
+  float bias_here[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    bias_here[e] = with_bias && n_piece + e < N ? load_as_float(bias, bias_is_float, n_piece + e) : 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int quad = 0; quad < 4; ++quad)
+        *(f32x4*)(mine + (size_t)r32 * ROW + i * 32 + quad * 8 + half * 4) =
+            (f32x4){acc[i][j][quad * 4], acc[i][j][quad * 4 + 1], acc[i][j][quad * 4 + 2], acc[i][j][quad * 4 + 3]};
+    // (a wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order)
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+      const int row = pass * 4 + row_in_pass;
+      const int m = m0 + wave_m * 128 + j * 32 + row;
+      const f32x4 lo = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8);
+      const f32x4 hi = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8 + 4);
+      float value[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) value[e] += bias_here[e];
+      if (m >= M) continue;
+      if (GATED) {
+        TO* dst = out + (size_t)m * (N / 2) + n_piece / 2;
+        float gated[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gated[e] = value[2 * e] / (1.f + expf(-value[2 * e])) * value[2 * e + 1];
+        if (n_piece + 8 <= N && sizeof(TO) == 2 && (N / 2) % 4 == 0) {
+          bf16_t packed[4] = {(bf16_t)gated[0], (bf16_t)gated[1], (bf16_t)gated[2], (bf16_t)gated[3]};
+          *(uint2*)dst = *(const uint2*)packed;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n_piece + 2 * e + 1 < N) dst[e] = from_float<TO>(gated[e]);
+        }
+      } else {
+        TO* dst = out + ((size_t)blockIdx.z * M + m) * N + n_piece;
+        if (n_piece + 8 <= N && N % 8 == 0) {
+          if (sizeof(TO) == 2) {
+            bf16_t packed[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) packed[e] = (bf16_t)value[e];
+            *(uint4*)dst = *(const uint4*)packed;
+          } else {
+            *(f32x4*)dst = (f32x4){value[0], value[1], value[2], value[3]};
+            *(f32x4*)((float*)dst + 4) = (f32x4){value[4], value[5], value[6], value[7]};
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n_piece + e < N) dst[e] = from_float<TO>(value[e]);
+        }
+      }
+    }
+  }
+}
+
+template <typename TO, bool GATED>
+static int launch_wide(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
+                       int K, int splits, hipStream_t stream) {
+  const size_t lds = (size_t)2 * 2 * WIDE_TILE * WIDE_K * sizeof(bf16_t);  // 128 KB
+  static bool asked = false;
+  if (!asked) {
+    if (hipFuncSetAttribute((const void*)gemm_wide_kernel<TO, GATED>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      return ERR_BAD_ARGUMENT;
+    asked = true;
+  }
+  hipLaunchKernelGGL((gemm_wide_kernel<TO, GATED>),
+                     dim3((N + WIDE_TILE - 1) / WIDE_TILE, (M + WIDE_TILE - 1) / WIDE_TILE, splits), dim3(256), lds,
+                     stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K, K / splits);
+  return LAUNCH_STATUS();
+}
+
+// As llmserve_gemm_tiled, with K (and K / splits) a multiple of 64.
+extern "C" int llmserve_gemm_wide(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
+                                  int out_is_float, int gated, int M, int N, int K, int splits, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || K % WIDE_K || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
+  if (splits > 1 && (gated || !out_is_float || K % splits || (K / splits) % WIDE_K)) return ERR_BAD_ARGUMENT;
+  if (gated)
+    return out_is_float ? launch_wide<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                        : launch_wide<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+  return out_is_float ? launch_wide<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
+                      : launch_wide<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+}
+
 template <typename TO, bool GATED>
 static int pick_tiled(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
                       int splits, hipStream_t stream) {
-  // the big tile when there are enough of them for every CU (256) to get one
-  const long big_tiles = (long)((N + 255) / 256) * ((M + 255) / 256) * splits;
-  if (big_tiles >= 200) return launch_tiled<4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  // the wide tile when there are enough of them for most CUs (256) to get one
+  const long wide_tiles = (long)((N + 255) / 256) * ((M + 255) / 256) * splits;
+  if (wide_tiles >= 200 && (K / splits) % WIDE_K == 0)
+    return launch_wide<TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
   return launch_tiled<2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
 }
 

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "llmserve_gemm_skinny": "pppipiiiiiip",
     "llmserve_gemm_medium": "pppipiiiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
+    "llmserve_gemm_wide": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifip",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
     "llmserve_attention_can_fuse": "i",
