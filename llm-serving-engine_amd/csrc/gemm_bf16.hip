@@ -334,6 +334,79 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define TILE_K 32
 #define TILE_STRIDE (TILE_K + 8)  // bf16 elements per staged row: 64 bytes + 16 of padding
 
+// The end of a tiled product.  D[n][m] of a 32 x 32 tile: a lane holds column m = lane % 32 and rows
+// n = 8 * (e / 4) + 4 * (lane / 32) + e % 4, so its values lie in 32 different rows of `out`.  They go
+// through LDS (`mine`: 32 x (32 WT + 4) floats of this wave's own), 32 rows of x at a time, and leave as
+// whole rows: 4 WT lanes write the 32 WT columns of a row, eight columns (16 bytes of bfloat16) a lane.
+// n_wave, m_wave: where the wave's WT x WT tiles begin; `slice` the K split (its own copy of `out`).
+template <int WT, typename TO, bool GATED>
+__device__ __forceinline__ void store_tiles(const f32x16 (&acc)[WT][WT], float* mine, TO* __restrict__ out,
+                                            const void* __restrict__ bias, int bias_is_float, int slice, int M, int N,
+                                            int n_wave, int m_wave, int lane) {
+  constexpr int ROW = 32 * WT + 4;           // floats of a transposed row, padded
+  constexpr int LANES_A_ROW = 4 * WT, ROWS_A_PASS = 64 / LANES_A_ROW;
+  const int r32 = lane & 31, half = lane >> 5;
+  const int piece = lane % LANES_A_ROW, row_in_pass = lane / LANES_A_ROW;
+  const int n_piece = n_wave + piece * 8;
+  const bool with_bias = bias && slice == 0;
+  float bias_here[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    bias_here[e] = with_bias && n_piece + e < N ? load_as_float(bias, bias_is_float, n_piece + e) : 0.f;
+#pragma unroll
+  for (int j = 0; j < WT; ++j) {
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+      for (int quad = 0; quad < 4; ++quad)
+        *(f32x4*)(mine + (size_t)r32 * ROW + i * 32 + quad * 8 + half * 4) =
+            (f32x4){acc[i][j][quad * 4], acc[i][j][quad * 4 + 1], acc[i][j][quad * 4 + 2], acc[i][j][quad * 4 + 3]};
+    // (a wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order)
+#pragma unroll
+    for (int pass = 0; pass < 32 / ROWS_A_PASS; ++pass) {
+      const int row = pass * ROWS_A_PASS + row_in_pass;
+      const int m = m_wave + j * 32 + row;
+      const f32x4 lo = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8);
+      const f32x4 hi = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8 + 4);
+      float value[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) value[e] += bias_here[e];
+      if (m >= M) continue;
+      if (GATED) {
+        TO* dst = out + (size_t)m * (N / 2) + n_piece / 2;
+        float gated[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gated[e] = value[2 * e] / (1.f + expf(-value[2 * e])) * value[2 * e + 1];
+        if (n_piece + 8 <= N && sizeof(TO) == 2 && (N / 2) % 4 == 0) {
+          bf16_t packed[4] = {(bf16_t)gated[0], (bf16_t)gated[1], (bf16_t)gated[2], (bf16_t)gated[3]};
+          *(uint2*)dst = *(const uint2*)packed;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n_piece + 2 * e + 1 < N) dst[e] = from_float<TO>(gated[e]);
+        }
+      } else {
+        TO* dst = out + ((size_t)slice * M + m) * N + n_piece;
+        if (n_piece + 8 <= N && N % 8 == 0) {
+          if (sizeof(TO) == 2) {
+            bf16_t packed[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) packed[e] = (bf16_t)value[e];
+            *(uint4*)dst = *(const uint4*)packed;
+          } else {
+            *(f32x4*)dst = (f32x4){value[0], value[1], value[2], value[3]};
+            *(f32x4*)((float*)dst + 4) = (f32x4){value[4], value[5], value[6], value[7]};
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n_piece + e < N) dst[e] = from_float<TO>(value[e]);
+        }
+      }
+    }
+  }
+}
+
 template <int WT, typename TO, bool GATED>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                          const void* __restrict__ bias, int bias_is_float,
@@ -411,44 +484,18 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     if (step + 1 < steps) stage(buffer ^ 1);  // read last in step - 1: everyone has passed this step's barrier since
   }
 
-  // D[n][m] of a 32 x 32 tile: lane holds column m = lane % 32 and rows n = 8 * (e / 4) + 4 * (lane / 32) + e % 4
-  const bool with_bias = bias && blockIdx.z == 0;
-#pragma unroll
-  for (int j = 0; j < WT; ++j) {
-    const int m = m0 + wave_m * 32 * WT + j * 32 + r32;
-    if (m >= M) continue;
-#pragma unroll
-    for (int i = 0; i < WT; ++i) {
-#pragma unroll
-      for (int quad = 0; quad < 4; ++quad) {
-        const int n_first = n0 + wave_n * 32 * WT + i * 32 + quad * 8 + half * 4;
-        float value[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          value[e] = acc[i][j][quad * 4 + e];
-          if (with_bias && n_first + e < N) value[e] += load_as_float(bias, bias_is_float, n_first + e);
-        }
-        if (GATED) {
-          TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
-#pragma unroll
-          for (int e = 0; e < 2; ++e)
-            if (n_first + 2 * e + 1 < N) dst[e] = from_float<TO>(value[2 * e] / (1.f + expf(-value[2 * e])) * value[2 * e + 1]);
-        } else {
-          TO* dst = out + ((size_t)blockIdx.z * M + m) * N + n_first;
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n_first + e < N) dst[e] = from_float<TO>(value[e]);
-        }
-      }
-    }
-  }
+  __syncthreads();  // every wave has read the last stage: LDS is free for the way out
+  store_tiles<WT, TO, GATED>(acc, (float*)staged + (size_t)wave * 32 * (32 * WT + 4), out, bias, bias_is_float,
+                             blockIdx.z, M, N, n0 + wave_n * 32 * WT, m0 + wave_m * 32 * WT, lane);
 }
 
 template <int WT, typename TO, bool GATED>
 static int launch_tiled(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
                         int K, int splits, hipStream_t stream) {
   constexpr int TILE = 64 * WT;
-  const size_t lds = (size_t)4 * TILE * TILE_STRIDE * sizeof(bf16_t);
+  const size_t stages = (size_t)4 * TILE * TILE_STRIDE * sizeof(bf16_t);
+  const size_t way_out = (size_t)4 * 32 * (32 * WT + 4) * sizeof(float);  // store_tiles' rows of the four waves
+  const size_t lds = stages > way_out ? stages : way_out;
   if (lds > 64 * 1024) {
     static bool asked = false;
     if (!asked) {
@@ -552,70 +599,8 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict
     __syncthreads();  // everyone has read this stage: the step after next may be written over it
   }
 
-  // D[n][m] of a 32 x 32 tile: lane holds column m = lane % 32 and rows n = 8 * (e / 4) + 4 * (lane / 32) + e % 4,
-  // so a lane's values lie in 32 different rows of `out`.  They go through LDS (the stages are free
-  // now), 32 rows of x at a time, and leave as whole rows: 16 lanes write the 128 columns of a row.
-  const bool with_bias = bias && blockIdx.z == 0;
-  constexpr int ROW = 128 + 4;  // floats of a transposed row, padded
-  float* mine = (float*)staged + (size_t)wave * 32 * ROW;  // [32 m][128 n] of this wave
-  const int piece = lane & 15, row_in_pass = lane >> 4;    // this lane's 8 columns; 4 rows a pass
-  const int n_piece = n0 + wave_n * 128 + piece * 8;
-  float bias_here[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e)
-    bias_here[e] = with_bias && n_piece + e < N ? load_as_float(bias, bias_is_float, n_piece + e) : 0.f;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int quad = 0; quad < 4; ++quad)
-        *(f32x4*)(mine + (size_t)r32 * ROW + i * 32 + quad * 8 + half * 4) =
-            (f32x4){acc[i][j][quad * 4], acc[i][j][quad * 4 + 1], acc[i][j][quad * 4 + 2], acc[i][j][quad * 4 + 3]};
-    // (a wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order)
-#pragma unroll
-    for (int pass = 0; pass < 8; ++pass) {
-      const int row = pass * 4 + row_in_pass;
-      const int m = m0 + wave_m * 128 + j * 32 + row;
-      const f32x4 lo = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8);
-      const f32x4 hi = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8 + 4);
-      float value[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) value[e] += bias_here[e];
-      if (m >= M) continue;
-      if (GATED) {
-        TO* dst = out + (size_t)m * (N / 2) + n_piece / 2;
-        float gated[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) gated[e] = value[2 * e] / (1.f + expf(-value[2 * e])) * value[2 * e + 1];
-        if (n_piece + 8 <= N && sizeof(TO) == 2 && (N / 2) % 4 == 0) {
-          bf16_t packed[4] = {(bf16_t)gated[0], (bf16_t)gated[1], (bf16_t)gated[2], (bf16_t)gated[3]};
-          *(uint2*)dst = *(const uint2*)packed;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n_piece + 2 * e + 1 < N) dst[e] = from_float<TO>(gated[e]);
-        }
-      } else {
-        TO* dst = out + ((size_t)blockIdx.z * M + m) * N + n_piece;
-        if (n_piece + 8 <= N && N % 8 == 0) {
-          if (sizeof(TO) == 2) {
-            bf16_t packed[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) packed[e] = (bf16_t)value[e];
-            *(uint4*)dst = *(const uint4*)packed;
-          } else {
-            *(f32x4*)dst = (f32x4){value[0], value[1], value[2], value[3]};
-            *(f32x4*)((float*)dst + 4) = (f32x4){value[4], value[5], value[6], value[7]};
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n_piece + e < N) dst[e] = from_float<TO>(value[e]);
-        }
-      }
-    }
-  }
+  store_tiles<4, TO, GATED>(acc, (float*)staged + (size_t)wave * 32 * (32 * 4 + 4), out, bias, bias_is_float,
+                            blockIdx.z, M, N, n0 + wave_n * 128, m0 + wave_m * 128, lane);
 }
 
 template <typename TO, bool GATED>
