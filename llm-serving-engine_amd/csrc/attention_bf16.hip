@@ -82,7 +82,7 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
 };
 
 template <int COLUMN_TILES, bool FUSED, int WAVES>
-__global__ __launch_bounds__(WAVES * 64, COLUMN_TILES > 2 ? 1 : 2) void attention_tiles_kernel(
+__global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 1 : 2) void attention_tiles_kernel(
     const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
     float* __restrict__ partial_ml, bf16_t* __restrict__ keys,
     bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,

@@ -452,7 +452,8 @@ class HipKernels:
         if batch.max_query_length > per_tile:
             # four column tiles a wave halve the cache traffic of two, at one wave a SIMD instead of
             # two: that pays once the keys no longer fit the chiplets' L2
-            wide = 4 if batch.max_context_length >= 4096 else 2
+            # (heads wider than 128 leave no registers for more than one tile)
+            wide = 1 if layout.head_dim > 128 else 4 if batch.max_context_length >= 4096 else 2
             launches.append((wide, *self._attention_work(batch, wide * per_tile, per_tile, None)))
         for column_tiles, work, items in launches:
             if items == 0:

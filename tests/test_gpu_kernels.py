@@ -182,6 +182,7 @@ ATTENTION_SHAPES = [  # heads, kv_heads, dim, page
     (5, 5, 80, 24),  # a page that is no power of two
     (8, 2, 128, 16),
     (3, 1, 112, 64),
+    (4, 2, 256, 16),  # the widest head the matrix-core kernel takes: one column tile a wave
     (4, 4, 16, 1),
 ]
 
@@ -355,7 +356,7 @@ def test_sampling_edges(kernels):
 
 
 @pytest.mark.parametrize("pairing", ["adjacent", "half", "none"])
-@pytest.mark.parametrize("heads,kv_heads,dim,page", [(12, 2, 128, 16), (6, 1, 64, 8), (5, 5, 32, 4), (4, 2, 48, 16), (40, 2, 64, 16)])
+@pytest.mark.parametrize("heads,kv_heads,dim,page", [(12, 2, 128, 16), (6, 1, 64, 8), (5, 5, 32, 4), (4, 2, 48, 16), (40, 2, 64, 16), (2, 1, 256, 16)])
 def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
     """A step of single tokens: rotation, the store of the new key and value, attention and the
     merge of key splits in one kernel (or, where the sizes do not allow it, in the separate ones):
