@@ -81,6 +81,104 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
   const int* slots;           // [rows] page * page_size + offset of each token, negative: store nothing
 };
 
+// One step's operands as a lane holds them: its slices of the K rows of the two 16-row tiles and,
+// for every 16-row tile of V^T, eight consecutive keys of its row.
+struct StepLoads {
+  QkOperand k_lo[QK_STEPS], k_hi[QK_STEPS];
+  bf16x8 v[D_TILES];
+};
+
+// What a lane keeps for its column in each of its column tiles.
+template <int COLUMN_TILES>
+struct Columns {
+  int position[COLUMN_TILES], first[COLUMN_TILES];  // the keys the column sees: [first, position]
+  QkOperand query[COLUMN_TILES][QK_STEPS];
+  float running_max[COLUMN_TILES], running_sum[COLUMN_TILES];
+  f32x4 acc[COLUMN_TILES][D_TILES];
+};
+
+// First product of a step, for all column tiles: after it the K rows are no longer needed.
+template <int COLUMN_TILES>
+__device__ __forceinline__ void scores_of(const Columns<COLUMN_TILES>& columns, const StepLoads& L, f32x4* s_lo,
+                                          f32x4* s_hi) {
+#pragma unroll
+  for (int t = 0; t < COLUMN_TILES; ++t) {
+    s_lo[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    s_hi[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < QK_STEPS; ++s) {
+      s_lo[t] = mfma_qk(L.k_lo[s], columns.query[t][s], s_lo[t]);
+      s_hi[t] = mfma_qk(L.k_hi[s], columns.query[t][s], s_hi[t]);
+    }
+  }
+}
+
+// Softmax weights and second product of a step.  Scores are kept in units of log2 (scale * log2 e is
+// folded into one multiply-add, weights are exp2 of differences to the column's reference).  The
+// reference is the column's maximum at some earlier step; it moves only when a score exceeds it by
+// more than RESCALE_STEP, so weights reach 2^RESCALE_STEP at most, the accumulators are rescaled
+// rarely, and the common step needs no exchange between the four lanes of a column: each checks its
+// own eight scores.  `interior`: every column of the wave sees all 32 keys of the step (no masks).
+// `v_start`: the first of the eight keys this lane's V values were really read from; values of keys
+// after `last_key` (slots never written) are kept out of 0 * x.
+template <int COLUMN_TILES>
+__device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, StepLoads& L, const f32x4* s_lo,
+                                              const f32x4* s_hi, int key0, int q, bool interior, int last_key,
+                                              int v_start, float scale_log2) {
+  bf16x8 weights[COLUMN_TILES];
+#pragma unroll
+  for (int t = 0; t < COLUMN_TILES; ++t) {
+    // lane holds, for its column, keys key0 + 8q + i
+    const bool unset = columns.running_max[t] == -INFINITY;  // nothing seen yet by this column
+    const float reference = unset ? 0.f : columns.running_max[t];
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = fmaf(i < 4 ? s_lo[t][i] : s_hi[t][i - 4], scale_log2, -reference);
+    if (!interior) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int key = key0 + 8 * q + i;
+        if (key > columns.position[t] || key < columns.first[t]) x[i] = -INFINITY;
+      }
+    }
+    const float highest = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+    if (__any(highest > (unset ? -INFINITY : RESCALE_STEP))) {
+      float column_highest = fmaxf(highest, __shfl_xor(highest, 16, WAVE));
+      column_highest = fmaxf(column_highest, __shfl_xor(column_highest, 32, WAVE));
+      if (column_highest > (unset ? -INFINITY : RESCALE_STEP)) {  // the same answer in the four lanes of a column
+        const float correction = unset ? 0.f : __builtin_amdgcn_exp2f(-column_highest);
+        columns.running_max[t] = reference + column_highest;
+        columns.running_sum[t] *= correction;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] -= column_highest;
+#pragma unroll
+        for (int d = 0; d < D_TILES; ++d) columns.acc[t][d] *= correction;
+      }
+    }
+    float added = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p = __builtin_amdgcn_exp2f(x[i]);  // exp2(-inf) = 0 for keys the column does not see
+      added += p;
+      weights[t][i] = (bf16_t)p;
+    }
+    columns.running_sum[t] += added;
+  }
+  if (key0 + KEYS - 1 > last_key) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (v_start + i > last_key) {
+#pragma unroll
+        for (int d = 0; d < D_TILES; ++d) L.v[d][i] = (bf16_t)0.f;
+      }
+  }
+#pragma unroll
+  for (int t = 0; t < COLUMN_TILES; ++t)
+#pragma unroll
+    for (int d = 0; d < D_TILES; ++d)
+      columns.acc[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(L.v[d], weights[t], columns.acc[t][d], 0, 0, 0);
+}
+
 template <int COLUMN_TILES, bool FUSED, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 1 : 2) void attention_tiles_kernel(
     const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
@@ -106,9 +204,14 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
   const int* table = block_tables + (size_t)request * table_width;
 
   // this lane's column in each of its column tiles
-  int column_position[COLUMN_TILES], column_first[COLUMN_TILES];
+  Columns<COLUMN_TILES> columns;
   bool column_live[COLUMN_TILES];
-  QkOperand query[COLUMN_TILES][QK_STEPS];
+  auto& column_position = columns.position;
+  auto& column_first = columns.first;
+  auto& query = columns.query;
+  auto& running_max = columns.running_max;
+  auto& running_sum = columns.running_sum;
+  auto& acc = columns.acc;
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
     const int token = t * tokens_per_tile + c / heads_here;
@@ -148,8 +251,6 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
 #endif
   }
 
-  float running_max[COLUMN_TILES], running_sum[COLUMN_TILES];
-  f32x4 acc[COLUMN_TILES][D_TILES];
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
     running_max[t] = -INFINITY;
@@ -196,10 +297,6 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
   // (row d = 16 * tile + c, keys 8q .. 8q+7; a page holds a multiple of 8 keys).  Keys outside
   // [first_key, last_key] are read from a key inside it (their weights are zero), so no page is
   // touched that the request does not hold.
-  struct StepLoads {
-    QkOperand k_lo[QK_STEPS], k_hi[QK_STEPS];
-    bf16x8 v[D_TILES];
-  };
   const int row_key = 8 * (c >> 2) + (c & 3);  // this lane's K row within a step (lo tile; hi: + 4)
   const int low_limit = first_key & ~7, high_limit = last_key & ~7;
   // Where a step's rows lie: the page numbers come from the block table (a load of their own,
@@ -240,83 +337,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
     for (int d = 0; d < D_TILES; ++d) L.v[d] = *(const bf16x8*)(base + (unsigned)(d * 16 + c) * page_size);
   };
 
-  // Scores are kept in units of log2 (scale * log2 e is folded into one multiply-add, weights are
-  // exp2 of differences to the column's reference).  The reference is the column's maximum at
-  // some earlier step; it moves only when a score exceeds it by more than RESCALE_STEP, so weights
-  // reach 2^RESCALE_STEP at most, the accumulators are rescaled rarely, and the common step needs
-  // no exchange between the four lanes of a column: each checks its own eight scores.
   const float scale_log2 = scale * 1.44269504088896f;
-  // first product of a step, for all column tiles: after it the K rows are no longer needed
-  auto scores_of = [&](const StepLoads& L, f32x4* s_lo, f32x4* s_hi) {
-#pragma unroll
-    for (int t = 0; t < COLUMN_TILES; ++t) {
-      s_lo[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      s_hi[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < QK_STEPS; ++s) {
-        s_lo[t] = mfma_qk(L.k_lo[s], query[t][s], s_lo[t]);
-        s_hi[t] = mfma_qk(L.k_hi[s], query[t][s], s_hi[t]);
-      }
-    }
-  };
-  // softmax weights and second product of a step
-  auto weigh_and_add = [&](int step, StepLoads& L, const f32x4* s_lo, const f32x4* s_hi) {
-    const int key0 = step * KEYS;
-    const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
-    bf16x8 weights[COLUMN_TILES];
-#pragma unroll
-    for (int t = 0; t < COLUMN_TILES; ++t) {
-      // lane holds, for its column, keys key0 + 8q + i
-      const bool unset = running_max[t] == -INFINITY;  // nothing seen yet by this column
-      const float reference = unset ? 0.f : running_max[t];
-      float x[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) x[i] = fmaf(i < 4 ? s_lo[t][i] : s_hi[t][i - 4], scale_log2, -reference);
-      if (!interior) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int key = key0 + 8 * q + i;
-          if (key > column_position[t] || key < column_first[t]) x[i] = -INFINITY;
-        }
-      }
-      const float highest = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-      if (__any(highest > (unset ? -INFINITY : RESCALE_STEP))) {
-        float column_highest = fmaxf(highest, __shfl_xor(highest, 16, WAVE));
-        column_highest = fmaxf(column_highest, __shfl_xor(column_highest, 32, WAVE));
-        if (column_highest > (unset ? -INFINITY : RESCALE_STEP)) {  // the same answer in the four lanes of a column
-          const float correction = unset ? 0.f : __builtin_amdgcn_exp2f(-column_highest);
-          running_max[t] = reference + column_highest;
-          running_sum[t] *= correction;
-#pragma unroll
-          for (int i = 0; i < 8; ++i) x[i] -= column_highest;
-#pragma unroll
-          for (int d = 0; d < D_TILES; ++d) acc[t][d] *= correction;
-        }
-      }
-      float added = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float p = __builtin_amdgcn_exp2f(x[i]);  // exp2(-inf) = 0 for keys the column does not see
-        added += p;
-        weights[t][i] = (bf16_t)p;
-      }
-      running_sum[t] += added;
-    }
-    if (key0 + KEYS - 1 > last_key) {  // slots after the last key were never written: keep them out of 0 * x
-      const int start = min(max(key0 + 8 * q, low_limit), high_limit);  // the slots really read
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (start + i > last_key) {
-#pragma unroll
-          for (int d = 0; d < D_TILES; ++d) L.v[d][i] = (bf16_t)0.f;
-        }
-    }
-#pragma unroll
-    for (int t = 0; t < COLUMN_TILES; ++t)
-#pragma unroll
-      for (int d = 0; d < D_TILES; ++d)
-        acc[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(L.v[d], weights[t], acc[t][d], 0, 0, 0);
-  };
 
   // A wave's next step is requested into the registers of the current one as soon as they are
   // free: the K rows after the first product, the V rows after the second; the page numbers of a
@@ -331,9 +352,12 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
     for (int step = step0; step < step_end; step += WAVES) {
       const bool more = step + WAVES < step_end;
       f32x4 s_lo[COLUMN_TILES], s_hi[COLUMN_TILES];
-      scores_of(loads, s_lo, s_hi);
+      scores_of(columns, loads, s_lo, s_hi);
       if (more) fetch_keys(step + WAVES, pages, loads);
-      weigh_and_add(step, loads, s_lo, s_hi);
+      const int key0 = step * KEYS;
+      const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
+      weigh_and_add(columns, loads, s_lo, s_hi, key0, q, interior, last_key,
+                    min(max(key0 + 8 * q, low_limit), high_limit), scale_log2);
       if (more) fetch_values(step + WAVES, pages, loads);
       if (step + 2 * WAVES < step_end) pages = pages_of(step + 2 * WAVES);
     }
@@ -393,6 +417,222 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
     __syncthreads();
   }
 }
+
+// ---------------------------------------------------------------------------- prompt portions, D = 128
+// For portions of many tokens the kernel above reads every key once per few tokens; this one shares
+// each step's K and V among the four waves of a workgroup through LDS.  A workgroup takes up to
+// 4 * COLUMN_TILES * tokens_per_tile consecutive tokens of a request (16 with two tiles and six
+// query heads a kv head); every wave owns the columns of its own tokens and walks all of their keys
+// itself (no key split, nothing to merge).  A step's 32 K rows and 128 x 32 V^T block (16 KB) are
+// brought in by all 256 threads, four 16-byte pieces each: requested into registers two steps ahead,
+// written to one of two LDS stages one step ahead.  A 16-byte piece of a row lies in the slot
+// (piece ^ f(row)) of its row, f chosen so that the 16 lanes that read one piece of 16 different
+// rows for an MFMA operand hit different banks.
+// (Loads that go from global memory straight into LDS were tried for this: the compiler makes every
+// read of LDS wait for all of them, whichever array they fill, so they cannot run two steps ahead.)
+#if HEAD_DIM == 128
+constexpr int PORTION_STAGE = 2 * KEYS * D;  // bf16 elements of a stage: K rows, then V^T rows
+
+struct StagedPieces {  // a lane's share of a step on its way to LDS
+  bf16x8 k[2], v[2];
+};
+
+template <int COLUMN_TILES>
+__global__ __launch_bounds__(256, 2) void attention_portions_kernel(
+    const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, const bf16_t* __restrict__ keys,
+    const bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
+    const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
+    int page_size, int page_shift, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) bf16_t stage_0[PORTION_STAGE], stage_1[PORTION_STAGE];  // each [K: 32 x 128 | V^T: 128 x 32]
+  const int group = heads / kv_heads;
+  const int kv_head = blockIdx.y % kv_heads, head_tile = blockIdx.y / kv_heads;
+  const int heads_here = min(group - head_tile * 16, 16);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, q = lane >> 4;
+  const int* item = work + (size_t)(gridDim.x - 1 - blockIdx.x) * 4;  // late tokens walk more keys: they start first
+  const int request = __builtin_amdgcn_readfirstlane(item[0]), row_first = __builtin_amdgcn_readfirstlane(item[1]);
+  const int tokens_all = __builtin_amdgcn_readfirstlane(item[2]);
+  const int position_first = __builtin_amdgcn_readfirstlane(positions[row_first]);
+  // the workgroup's keys, and this wave's: the tokens [mine_first, mine_first + tokens) of the item
+  const int last_key_all = position_first + tokens_all - 1;
+  const int first_key_all = window > 0 ? max(0, position_first - window + 1) : 0;
+  const int mine_first = wave * COLUMN_TILES * tokens_per_tile;
+  const int tokens = min(tokens_all - mine_first, COLUMN_TILES * tokens_per_tile);  // <= 0: nothing of its own
+  const int row0 = row_first + mine_first, position0 = position_first + mine_first;
+  const int last_key = position0 + tokens - 1;
+  const int first_key = window > 0 ? max(0, position0 - window + 1) : 0;
+  const int* table = block_tables + (size_t)request * table_width;
+
+  Columns<COLUMN_TILES> columns;
+  bool column_live[COLUMN_TILES];
+#pragma unroll
+  for (int t = 0; t < COLUMN_TILES; ++t) {
+    const int token = t * tokens_per_tile + c / heads_here;
+    column_live[t] = token < tokens && c / heads_here < tokens_per_tile;
+    const int safe = max(0, min(token, tokens - 1));
+    const int head = kv_head * group + head_tile * 16 + c % heads_here;
+    columns.position[t] = column_live[t] ? position0 + safe : -1;
+    columns.first[t] = window > 0 ? columns.position[t] - window + 1 : 0;
+    const bf16_t* q_row = qkv + (size_t)(min(row0, row_first + tokens_all - 1) + safe) * row_width + (size_t)head * D;
+#pragma unroll
+    for (int s = 0; s < QK_STEPS; ++s) columns.query[t][s] = load_qk(q_row, s, q);
+    columns.running_max[t] = -INFINITY;
+    columns.running_sum[t] = 0.f;
+#pragma unroll
+    for (int d = 0; d < D_TILES; ++d) columns.acc[t][d] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int step_first_all = first_key_all / KEYS, step_last_all = last_key_all / KEYS;
+  const int step_first = first_key / KEYS, step_last = tokens > 0 ? last_key / KEYS : -1;
+  const unsigned page_stride = (unsigned)kv_heads * page_size * D;
+  const unsigned head_offset = (unsigned)kv_head * page_size * D;
+  const int low_limit = first_key_all & ~7, high_limit = last_key_all & ~7;
+  auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
+
+  // This lane's four pieces of a step: of K rows 8 wave .. 8 wave + 7 and of V^T rows 32 wave .. 32 wave + 31.
+  // The four groups of eight keys of a step each lie in one page, looked up through scalar loads.
+  auto fetch_step = [&](int step, StagedPieces& pieces) {
+    const int key0 = step * KEYS;
+    int pages[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pages[i] = table[page_index(min(max(key0 + 8 * i, first_key_all), last_key_all))];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      // K: lane l takes piece l % 16 of row 4 (2 wave + j) + l / 16: 256 bytes of a row from 16 lanes
+      const int row = 4 * (2 * wave + j) + (lane >> 4);
+      const int key = min(max(key0 + row, first_key_all), last_key_all);
+      const int offset = key - page_index(key) * page_size;
+      pieces.k[j] = *(const bf16x8*)(keys + (size_t)(unsigned)pages[wave] * page_stride +
+                                     (head_offset + (unsigned)offset * D) + (lane & 15) * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      // V^T: lane l takes piece l % 4 (the keys 8 piece .. 8 piece + 7 of the step) of row 16 (2 wave + j) + l / 4
+      const int d = 16 * (2 * wave + j) + (lane >> 2);
+      const int piece = lane & 3;
+      const int key = min(max(key0 + 8 * piece, low_limit), high_limit);
+      const int page = piece == 0 ? pages[0] : piece == 1 ? pages[1] : piece == 2 ? pages[2] : pages[3];
+      const int offset = key - page_index(key) * page_size;
+      pieces.v[j] = *(const bf16x8*)(values + (size_t)(unsigned)page * page_stride +
+                                     (head_offset + (unsigned)d * page_size + offset));
+    }
+  };
+  auto write_step = [&](const StagedPieces& pieces, bf16_t* stage) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int row = 4 * (2 * wave + j) + (lane >> 4);
+      const int slot = (lane & 15) ^ ((row & 3) | ((row >> 3) << 2));
+      *(bf16x8*)(stage + (size_t)row * D + slot * 8) = pieces.k[j];
+      const int d = 16 * (2 * wave + j) + (lane >> 2);
+      *(bf16x8*)(stage + KEYS * D + (size_t)d * KEYS + ((lane & 3) ^ ((d >> 1) & 3)) * 8) = pieces.v[j];
+    }
+  };
+
+  const float scale_log2 = scale * 1.44269504088896f;
+  const int row_lo = 8 * (c >> 2) + (c & 3);  // this lane's K row in the "lo" tile ("hi": four further)
+  const int k_swizzle = (row_lo & 3) | ((row_lo >> 3) << 2), v_swizzle = (c >> 1) & 3;
+  // One step: its operands are in `stage`.  `ahead` holds the pieces of the next step, requested two
+  // steps ago: they go to `other`, which was read last a step ago, and `ahead` is requested anew
+  // for the step after the one after next.
+  auto walk_step = [&](int step, const bf16_t* stage, bf16_t* other, StagedPieces& ahead) {
+    write_step(ahead, other);
+    fetch_step(step + 3, ahead);
+    if (step >= step_first && step <= step_last) {
+      StepLoads loads;
+#pragma unroll
+      for (int s = 0; s < QK_STEPS; ++s) {
+        const int slot = ((s * 4 + q) ^ k_swizzle) * 8;
+        loads.k_lo[s].v = *(const bf16x8*)(stage + (size_t)row_lo * D + slot);
+        loads.k_hi[s].v = *(const bf16x8*)(stage + (size_t)(row_lo + 4) * D + slot);
+      }
+#pragma unroll
+      for (int d = 0; d < D_TILES; ++d)
+        loads.v[d] = *(const bf16x8*)(stage + KEYS * D + (size_t)(d * 16 + c) * KEYS + (q ^ v_swizzle) * 8);
+      f32x4 s_lo[COLUMN_TILES], s_hi[COLUMN_TILES];
+      scores_of(columns, loads, s_lo, s_hi);
+      const int key0 = step * KEYS;
+      const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
+      weigh_and_add(columns, loads, s_lo, s_hi, key0, q, interior, last_key_all,
+                    min(max(key0 + 8 * q, low_limit), high_limit), scale_log2);
+    }
+    // what was written to `other` is there for everyone, and everyone has read `stage` (a bare barrier:
+    // the loads under way are not to be waited for)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  };
+  StagedPieces even, odd;  // the pieces of the even and of the odd steps, counted from the first
+  fetch_step(step_first_all, even);
+  fetch_step(step_first_all + 1, odd);
+  write_step(even, stage_0);
+  fetch_step(step_first_all + 2, even);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  for (int step = step_first_all; step <= step_last_all; step += 2) {  // (a step past the last one is walked empty)
+    walk_step(step, stage_0, stage_1, odd);
+    walk_step(step + 1, stage_1, stage_0, even);
+  }
+  // (the last barrier of the walk has passed: LDS is free)
+
+  // each wave's columns leave through its own half of a stage (16 columns x 128 floats) as whole rows of `out`
+  constexpr int STRIDE = D;
+  float* mine = (float*)(wave < 2 ? stage_0 : stage_1) + (size_t)(wave & 1) * 16 * STRIDE;
+#pragma unroll
+  for (int t = 0; t < COLUMN_TILES; ++t) {
+    float sum = columns.running_sum[t];
+    sum += __shfl_xor(sum, 16, WAVE);
+    sum += __shfl_xor(sum, 32, WAVE);
+    const float inverse = sum > 0.f ? 1.f / sum : 0.f;
+#pragma unroll
+    for (int d = 0; d < D_TILES; ++d)
+      *(f32x4*)(mine + (size_t)c * STRIDE + d * 16 + 4 * q) = columns.acc[t][d] * inverse;
+    // lane (column l / 4, quarter l % 4) writes 32 values of the column's row
+    const int column = lane >> 2, quarter = lane & 3;
+    const int token = t * tokens_per_tile + column / heads_here;
+    if (token < tokens && column / heads_here < tokens_per_tile) {
+      const int head = kv_head * group + head_tile * 16 + column % heads_here;
+      bf16_t* dst = out + ((size_t)(row0 + token) * heads + head) * D + quarter * 32;
+#pragma unroll
+      for (int piece = 0; piece < 4; ++piece) {
+        const f32x4 lo = *(const f32x4*)(mine + (size_t)column * STRIDE + quarter * 32 + piece * 8);
+        const f32x4 hi = *(const f32x4*)(mine + (size_t)column * STRIDE + quarter * 32 + piece * 8 + 4);
+        bf16_t packed[8] = {(bf16_t)lo[0], (bf16_t)lo[1], (bf16_t)lo[2], (bf16_t)lo[3],
+                            (bf16_t)hi[0], (bf16_t)hi[1], (bf16_t)hi[2], (bf16_t)hi[3]};
+        *(uint4*)(dst + piece * 8) = *(const uint4*)packed;
+      }
+    }
+  }
+}
+
+// `work` holds `items` entries {request index in the step, first token row, tokens, unused}; an item
+// covers at most 4 * column_tiles * tokens_per_tile tokens (column_tiles 1 or 2), tokens_per_tile = max(1, 16 / (heads /
+// kv_heads)).  page_size a multiple of 8.
+extern "C" int llmserve_attention_portions(const void* qkv, int row_width, void* out, const void* keys,
+                                           const void* values, const int* block_tables, int table_width,
+                                           const int* positions, const int* work, int items, int column_tiles,
+                                           int heads, int kv_heads, int page_size, float scale, int window,
+                                           hipStream_t stream) {
+  if (items <= 0) return 0;
+  if (heads % kv_heads || page_size % 8 || (column_tiles != 1 && column_tiles != 2)) return ERR_BAD_ARGUMENT;
+  if ((long)kv_heads * page_size * D >= (1L << 31)) return ERR_BAD_ARGUMENT;
+  const int group = heads / kv_heads;
+  const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+  const dim3 grid(items, kv_heads * ((group + 15) / 16));
+  if (column_tiles == 1)
+    hipLaunchKernelGGL(attention_portions_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)qkv, row_width,
+                       (bf16_t*)out, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width, positions,
+                       work, heads, kv_heads, tokens_per_tile, page_size, page_shift, scale, window);
+  else
+    hipLaunchKernelGGL(attention_portions_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)qkv, row_width,
+                       (bf16_t*)out, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width, positions,
+                       work, heads, kv_heads, tokens_per_tile, page_size, page_shift, scale, window);
+  return LAUNCH_STATUS();
+}
+#else
+extern "C" int llmserve_attention_portions(const void*, int, void*, const void*, const void*, const int*, int,
+                                           const int*, const int*, int, int, int, int, int, float, int, hipStream_t) {
+  return ERR_BAD_ARGUMENT;  // built for head size 128 only
+}
+#endif
 
 // Merges the key splits of one (token, head): out = sum_s acc_s * 2^(m_s - m) / sum_s l_s *
 // 2^(m_s - m), in split order (the maxima are kept in units of log2).  A second kernel rather than "the last workgroup merges": a

@@ -57,6 +57,7 @@ _SIGNATURES = {
     "llmserve_gemm_wide": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifip",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
+    "llmserve_attention_portions": "pippppippiiiiifip",
     "llmserve_attention_can_fuse": "i",
     "llmserve_argmax": "ppppiip",
     "llmserve_sample": "ppppppiip",
@@ -108,8 +109,12 @@ class GatedLinearWeights:
 
 class HipKernels:
     def __init__(
-        self, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0", *, library_products: bool = True
+        self, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0", *, library_products: bool = True,
+        shared_portions: str = "auto",
     ) -> None:
+        """`library_products=False` keeps every product on the hand-written kernels.  `shared_portions`:
+        whether prompt portions at head size 128 go to the attention kernel whose waves share K and V
+        through LDS: "auto" (when the step has 512 workgroups of it or more), "always", "never"."""
         if dtype not in (torch.bfloat16, torch.float32):
             raise KernelError(f"run dtype must be bfloat16 or float32, not {dtype}")
         if not torch.cuda.is_available():
@@ -117,6 +122,7 @@ class HipKernels:
         self.dtype = dtype
         self.device = torch.device(device)
         self.library_products = library_products
+        self.shared_portions = shared_portions
         name = torch.cuda.get_device_properties(self.device).gcnArchName
         if not name.startswith("gfx950"):
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
@@ -449,7 +455,21 @@ class HipKernels:
         head_tiles = -(-(heads // kv_heads) // 16)
         tokens = qkv.shape[0]
         launches = [(1, *self._attention_work(batch, per_tile, 0, per_tile))]
-        if batch.max_query_length > per_tile:
+        shared = False
+        if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never":
+            # Prompt portions at this head size may go to the kernel whose waves share each step's K and V
+            # through LDS (a quarter of the cache traffic).  Its workgroups walk all their keys step after
+            # step, so it needs several workgroups a CU to be ahead: long prompts, or many of them.
+            work, items = self._attention_work(batch, 8 * per_tile, per_tile, None)
+            shared = self.shared_portions == "always" or items * kv_heads * head_tiles >= 512
+        if shared:
+            status = library.llmserve_attention_portions(
+                _pointer(qkv), layout.width, _pointer(out), _pointer(cell.keys), _pointer(cell.values),
+                _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items,
+                2, heads, kv_heads, group.page_size, scale, window, self._stream,
+            )
+            _check(status, "paged_attention")
+        elif batch.max_query_length > per_tile:
             # four column tiles a wave halve the cache traffic of two, at one wave a SIMD instead of
             # two: that pays once the keys no longer fit the chiplets' L2
             # (heads wider than 128 leave no registers for more than one tile)

@@ -256,6 +256,32 @@ def test_paged_attention_finds_a_far_key_among_hundreds(kernels, dtype):
         torch.testing.assert_close(out[0], rounded(v, dtype)[far, 0], atol=5e-2, rtol=0)
 
 
+@pytest.mark.parametrize("window", [None, 21, 64])
+@pytest.mark.parametrize("heads,kv_heads,page", [(12, 2, 16), (28, 4, 8), (40, 2, 16), (5, 5, 24), (3, 1, 32)])
+def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, window):
+    """At head size 128 prompt portions may go to the kernel whose four waves share each step's K and V
+    through LDS: portions that fill its workgroups, that leave waves empty, that end inside a step of 32
+    keys and that begin long after the sequence's start, with and without a window."""
+    from llmserve_amd.kernels import HipKernels
+
+    dim, dtype = 128, torch.bfloat16
+    shared = HipKernels(dtype, shared_portions="always")
+    apart = HipKernels(dtype, shared_portions="never")
+    lengths = [130, 97, 33, 300, 64, 5]
+    counts = [130, 40, 33, 70, 17, 3]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=heads)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    scale = 0.11
+    out = shared.paged_attention(qkv, layout, batch, cell, scale, window).cpu().double()
+    expected = []
+    for (q, k, v), count in zip(per_request, counts):
+        full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), scale, window)
+        expected.append(full[-count:].flatten(1))
+    torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
+    other = apart.paged_attention(qkv, layout, batch, cell, scale, window).cpu().double()
+    torch.testing.assert_close(out, other, **TOLERANCE[dtype])
+
+
 @pytest.mark.parametrize("window", [None, 1500])
 def test_paged_attention_portion_of_a_long_context(kernels, window):
     """Beyond 4,096 keys the bfloat16 kernel carries four column tiles a wave: a portion at the end of
