@@ -67,7 +67,7 @@ __device__ __forceinline__ f32x4 mfma_qk(const QkOperand& a, const QkOperand& b,
 #endif
 }
 
-// work[tile] = {request index in the step, first token row, tokens in the tile, unused}
+// work[tile] = {request index in the step, first token row, first head, columns}: see ColumnMap
 // pairing: 0 none, 1 adjacent pairs (2j, 2j+1), 2 half pairs (j, j + D/2)
 __device__ __forceinline__ void rotate_pair(float& a, float& b, float2 cos_sin) {
   const float x = a * cos_sin.x - b * cos_sin.y, y = b * cos_sin.x + a * cos_sin.y;
@@ -86,6 +86,28 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
 struct StepLoads {
   QkOperand k_lo[QK_STEPS], k_hi[QK_STEPS];
   bf16x8 v[D_TILES];
+};
+
+// Which (token, query head) a column of a work item is.  With up to 16 query heads a kv head the
+// columns run through the item's tokens head by head, beginning at `first_head` of its first token,
+// so that every column tile is full whatever the number of heads; with more than 16 a workgroup
+// takes 16 heads (or what is left) and a column tile is one token.
+struct ColumnMap {
+  int heads_here, first_head, columns;
+  bool packed;
+  __device__ __forceinline__ void of(int tile, int c, int& token, int& head, bool& live) const {
+    if (packed) {
+      const int flat = first_head + tile * 16 + c;
+      token = flat / heads_here;
+      head = flat - token * heads_here;
+      live = tile * 16 + c < columns;
+    } else {
+      token = tile;
+      head = min(c, heads_here - 1);
+      live = tile < columns && c < heads_here;
+    }
+  }
+  __device__ __forceinline__ int tokens() const { return packed ? (first_head + columns - 1) / heads_here + 1 : columns; }
 };
 
 // What a lane keeps for its column in each of its column tiles.
@@ -197,7 +219,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
   // (when FUSED every request brings one token: tile i is request i and row i, nothing to look up)
   const int* item = work + (size_t)(gridDim.x - 1 - blockIdx.x) * 4;
   const int request = FUSED ? (int)blockIdx.x : item[0], row0 = FUSED ? (int)blockIdx.x : item[1];
-  const int tokens = FUSED ? 1 : item[2];
+  const ColumnMap map = {heads_here, FUSED ? 0 : item[2], FUSED ? (group <= 16 ? heads_here : 1) : item[3], group <= 16};
+  const int tokens = map.tokens();
   const int position0 = positions[row0];
   const int last_key = position0 + tokens - 1;
   const int first_key = window > 0 ? max(0, position0 - window + 1) : 0;
@@ -214,10 +237,10 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
   auto& acc = columns.acc;
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
-    const int token = t * tokens_per_tile + c / heads_here;
-    column_live[t] = token < tokens && c / heads_here < tokens_per_tile;
+    int token, head_here;
+    map.of(t, c, token, head_here, column_live[t]);
     const int safe = min(token, tokens - 1);
-    const int head = kv_head * group + head_tile * 16 + c % heads_here;
+    const int head = kv_head * group + head_tile * 16 + head_here;
     column_position[t] = column_live[t] ? position0 + safe : -1;
     column_first[t] = window > 0 ? column_position[t] - window + 1 : 0;
     const bf16_t* q_row = qkv + (size_t)(row0 + safe) * row_width + (size_t)head * D;
@@ -383,8 +406,10 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
     __syncthreads();
     for (int index = threadIdx.x; index < 16 * (D / 4); index += WAVES * 64) {
       const int column = index / (D / 4), d4 = (index % (D / 4)) * 4;
-      const int token = t * tokens_per_tile + column / heads_here;
-      if (token >= tokens || column / heads_here >= tokens_per_tile) continue;
+      int token, head_here;
+      bool live;
+      map.of(t, column, token, head_here, live);
+      if (!live) continue;
       float best = -INFINITY;
       for (int w = 0; w < WAVES; ++w) best = fmaxf(best, lds[((size_t)w * 16 + column) * STRIDE + D]);
       float total = 0.f;
@@ -396,7 +421,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
 #pragma unroll
         for (int i = 0; i < 4; ++i) merged[i] += theirs[d4 + i] * factor;
       }
-      const int head = kv_head * group + head_tile * 16 + column % heads_here;
+      const int head = kv_head * group + head_tile * 16 + head_here;
       const size_t row = (size_t)row0 + token;
       if (splits == 1) {
         bf16_t* dst = out + (row * heads + head) * D + d4;
@@ -421,8 +446,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
 // ---------------------------------------------------------------------------- prompt portions, D = 128
 // For portions of many tokens the kernel above reads every key once per few tokens; this one shares
 // each step's K and V among the four waves of a workgroup through LDS.  A workgroup takes up to
-// 4 * COLUMN_TILES * tokens_per_tile consecutive tokens of a request (16 with two tiles and six
-// query heads a kv head); every wave owns the columns of its own tokens and walks all of their keys
+// 4 * COLUMN_TILES column tiles of a request (128 (token, head) pairs with two tiles: 21 tokens at six
+// query heads a kv head); every wave owns its own column tiles and walks all of their keys
 // itself (no key split, nothing to merge).  A step's 32 K rows and 128 x 32 V^T block (16 KB) are
 // brought in by all 256 threads, four 16-byte pieces each: requested into registers two steps ahead,
 // written to one of two LDS stages one step ahead.  A 16-byte piece of a row lies in the slot
@@ -452,13 +477,18 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   const int c = lane & 15, q = lane >> 4;
   const int* item = work + (size_t)(gridDim.x - 1 - blockIdx.x) * 4;  // late tokens walk more keys: they start first
   const int request = __builtin_amdgcn_readfirstlane(item[0]), row_first = __builtin_amdgcn_readfirstlane(item[1]);
-  const int tokens_all = __builtin_amdgcn_readfirstlane(item[2]);
+  const ColumnMap all = {heads_here, __builtin_amdgcn_readfirstlane(item[2]), __builtin_amdgcn_readfirstlane(item[3]),
+                         group <= 16};
+  const int tokens_all = all.tokens();
   const int position_first = __builtin_amdgcn_readfirstlane(positions[row_first]);
-  // the workgroup's keys, and this wave's: the tokens [mine_first, mine_first + tokens) of the item
+  // the workgroup's keys, and this wave's: its COLUMN_TILES column tiles of the item's columns
   const int last_key_all = position_first + tokens_all - 1;
   const int first_key_all = window > 0 ? max(0, position_first - window + 1) : 0;
-  const int mine_first = wave * COLUMN_TILES * tokens_per_tile;
-  const int tokens = min(tokens_all - mine_first, COLUMN_TILES * tokens_per_tile);  // <= 0: nothing of its own
+  const int skipped = wave * COLUMN_TILES * (all.packed ? 16 : 1);  // columns (packed) or tokens before this wave's
+  const int mine_first = all.packed ? (all.first_head + skipped) / heads_here : skipped;  // its first token, within the item
+  const ColumnMap map = {heads_here, all.packed ? (all.first_head + skipped) % heads_here : 0,
+                         max(0, min(all.columns - skipped, COLUMN_TILES * (all.packed ? 16 : 1))), all.packed};
+  const int tokens = map.columns > 0 ? map.tokens() : 0;  // 0: nothing of its own
   const int row0 = row_first + mine_first, position0 = position_first + mine_first;
   const int last_key = position0 + tokens - 1;
   const int first_key = window > 0 ? max(0, position0 - window + 1) : 0;
@@ -468,10 +498,10 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   bool column_live[COLUMN_TILES];
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
-    const int token = t * tokens_per_tile + c / heads_here;
-    column_live[t] = token < tokens && c / heads_here < tokens_per_tile;
+    int token, head_here;
+    map.of(t, c, token, head_here, column_live[t]);
     const int safe = max(0, min(token, tokens - 1));
-    const int head = kv_head * group + head_tile * 16 + c % heads_here;
+    const int head = kv_head * group + head_tile * 16 + head_here;
     columns.position[t] = column_live[t] ? position0 + safe : -1;
     columns.first[t] = window > 0 ? columns.position[t] - window + 1 : 0;
     const bf16_t* q_row = qkv + (size_t)(min(row0, row_first + tokens_all - 1) + safe) * row_width + (size_t)head * D;
@@ -586,9 +616,11 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
       *(f32x4*)(mine + (size_t)c * STRIDE + d * 16 + 4 * q) = columns.acc[t][d] * inverse;
     // lane (column l / 4, quarter l % 4) writes 32 values of the column's row
     const int column = lane >> 2, quarter = lane & 3;
-    const int token = t * tokens_per_tile + column / heads_here;
-    if (token < tokens && column / heads_here < tokens_per_tile) {
-      const int head = kv_head * group + head_tile * 16 + column % heads_here;
+    int token, head_here;
+    bool live;
+    map.of(t, column, token, head_here, live);
+    if (live) {
+      const int head = kv_head * group + head_tile * 16 + head_here;
       bf16_t* dst = out + ((size_t)(row0 + token) * heads + head) * D + quarter * 32;
 #pragma unroll
       for (int piece = 0; piece < 4; ++piece) {
@@ -602,8 +634,8 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   }
 }
 
-// `work` holds `items` entries {request index in the step, first token row, tokens, unused}; an item
-// covers at most 4 * column_tiles * tokens_per_tile tokens (column_tiles 1 or 2), tokens_per_tile = max(1, 16 / (heads /
+// `work` holds `items` entries as for llmserve_attention_tiles; an item covers at most 4 * column_tiles
+// column tiles (column_tiles 1 or 2), tokens_per_tile = max(1, 16 / (heads /
 // kv_heads)).  page_size a multiple of 8.
 extern "C" int llmserve_attention_portions(const void* qkv, int row_width, void* out, const void* keys,
                                            const void* values, const int* block_tables, int table_width,
@@ -691,9 +723,10 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
   return pairing == 1 || (pairing == 2 && D % 64 == 0);
 }
 
-// `work` holds `tiles` items of four ints; a tile covers `column_tiles * tokens_per_tile`
-// tokens at most, where tokens_per_tile = max(1, 16 / (heads / kv_heads)).  page_size must
-// be a multiple of 8.  With splits > 1, partial_acc is float32 [rows * heads * splits * D],
+// `work` holds `tiles` items of four ints {request index in the step, first token row, first head,
+// columns}: with up to 16 query heads a kv head a run of at most `column_tiles` * 16 (token, head)
+// pairs of the request, beginning at `first head` of the first token; with more, at most
+// `column_tiles` tokens ("columns" counts tokens).  page_size must be a multiple of 8.  With splits > 1, partial_acc is float32 [rows * heads * splits * D],
 // partial_ml [rows * heads * splits * 2] (rows being the step's token count), and every row
 // of the step must lie in one of the tiles: a second kernel merges the splits of all rows.
 // With `fuse` tile i is row i, the one token of request i (`work` is not read), qkv is as the projection left it, and the kernel

@@ -114,7 +114,7 @@ class HipKernels:
     ) -> None:
         """`library_products=False` keeps every product on the hand-written kernels.  `shared_portions`:
         whether prompt portions at head size 128 go to the attention kernel whose waves share K and V
-        through LDS: "auto" (when the step has 512 workgroups of it or more), "always", "never"."""
+        through LDS: "auto" (when the step's walks, taken together, are long beside the longest), "always", "never"."""
         if dtype not in (torch.bfloat16, torch.float32):
             raise KernelError(f"run dtype must be bfloat16 or float32, not {dtype}")
         if not torch.cuda.is_available():
@@ -402,11 +402,13 @@ class HipKernels:
             self._attention_bf16[head_dim] = _declared(load_module("attention_bf16", {"HEAD_DIM": head_dim}))
         return self._attention_bf16[head_dim]
 
-    def _attention_work(self, batch, tokens_per_item: int, longer_than: int, up_to: int | None):
-        """Work items (request, first row, tokens, 0) for the requests of the step whose token
-        count lies in (longer_than, up_to], cut into items of `tokens_per_item` tokens.  Built
-        once per step and kept on the batch."""
-        key = ("attention_work", tokens_per_item, longer_than, up_to)
+    def _attention_work(self, batch, group: int, column_tiles: int, longer_than: int, up_to: int | None):
+        """Work items (request, first row, first head, columns) for the requests of the step whose
+        token count lies in (longer_than, up_to].  With up to 16 query heads a kv head (`group`) an
+        item is a run of `column_tiles` * 16 (token, head) pairs of a request, token by token and
+        head by head, wherever in a token it begins; with more, `column_tiles` tokens (and
+        "columns" counts tokens).  Built once per step and kept on the batch."""
+        key = ("attention_work", group, column_tiles, longer_than, up_to)
         if key not in batch.scratch:
             import numpy as np
 
@@ -416,13 +418,20 @@ class HipKernels:
             if up_to is not None:
                 chosen &= counts <= up_to
             which = np.nonzero(chosen)[0]
-            items = -(-counts[which] // tokens_per_item)
+            packed = group <= 16
+            per_token = group if packed else 1
+            per_item = column_tiles * (16 if packed else 1)
+            totals = counts[which] * per_token
+            items = -(-totals // per_item)
             request = np.repeat(which, items)
             inside = np.arange(int(items.sum())) - np.repeat(np.cumsum(items) - items, items)
-            first = inside * tokens_per_item
-            tokens = np.minimum(tokens_per_item, counts[request] - first)
-            work = np.stack([request, starts[request] + first, tokens, np.zeros_like(first)], axis=1).astype(np.int32)
-            batch.scratch[key] = (self.to_device(torch.from_numpy(work)) if len(work) else None, len(work))
+            first = inside * per_item
+            columns = np.minimum(per_item, np.repeat(totals, items) - first)
+            work = np.stack([request, starts[request] + first // per_token, first % per_token, columns], axis=1).astype(np.int32)
+            # about how many 32-key steps the items walk, all together
+            begins = np.array([chunk.start for chunk in batch.chunks], dtype=np.int64)[which]
+            steps = int((items * ((begins + counts[which] / 2) / 32 + 1)).sum())
+            batch.scratch[key] = (self.to_device(torch.from_numpy(work)) if len(work) else None, len(work), steps)
         return batch.scratch[key]
 
     def paged_attention(self, qkv, layout, batch, cell, scale: float, window: int | None) -> torch.Tensor:
@@ -454,14 +463,21 @@ class HipKernels:
         per_tile = max(1, 16 // (heads // kv_heads))
         head_tiles = -(-(heads // kv_heads) // 16)
         tokens = qkv.shape[0]
-        launches = [(1, *self._attention_work(batch, per_tile, 0, per_tile))]
+        group_size = heads // kv_heads
+        launches = [(1, *self._attention_work(batch, group_size, 1, 0, per_tile)[:2])]
         shared = False
         if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never":
             # Prompt portions at this head size may go to the kernel whose waves share each step's K and V
             # through LDS (a quarter of the cache traffic).  Its workgroups walk all their keys step after
             # step, so it needs several workgroups a CU to be ahead: long prompts, or many of them.
-            work, items = self._attention_work(batch, 8 * per_tile, per_tile, None)
-            shared = self.shared_portions == "always" or items * kv_heads * head_tiles >= 512
+            work, items, steps = self._attention_work(batch, group_size, 8, per_tile, None)
+            workgroups = items * kv_heads * head_tiles
+            # measured at 6 and 7 query heads a kv head: it takes 1.2 us for every step of its longest walk
+            # and 0.4 ns for every step of all walks, the other kernel 4 to 6 ns for every step of all walks
+            longest = batch.max_context_length / 32
+            shared = self.shared_portions == "always" or (
+                workgroups >= 256 and steps * kv_heads * head_tiles > 200 * longest
+            )
         if shared:
             status = library.llmserve_attention_portions(
                 _pointer(qkv), layout.width, _pointer(out), _pointer(cell.keys), _pointer(cell.values),
@@ -474,7 +490,7 @@ class HipKernels:
             # two: that pays once the keys no longer fit the chiplets' L2
             # (heads wider than 128 leave no registers for more than one tile)
             wide = 1 if layout.head_dim > 128 else 4 if batch.max_context_length >= 4096 else 2
-            launches.append((wide, *self._attention_work(batch, wide * per_tile, per_tile, None)))
+            launches.append((wide, *self._attention_work(batch, group_size, wide, per_tile, None)[:2]))
         for column_tiles, work, items in launches:
             if items == 0:
                 continue
