@@ -9,7 +9,7 @@ import torch
 
 from tests.gpu_helpers import TraceBuilder, replay
 from tests.plain import qwen2_plain as plain
-from tests.tiny import CONFIGS, random_tokens
+from tests.tiny import CONFIGS, PAGE_WIDE, WIDE, random_tokens, write_wide_folder
 
 pytestmark = pytest.mark.gpu
 
@@ -19,7 +19,7 @@ TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=3e-2, 
 LENGTHS = {"A": [1, 5, 17, 33, 70, 100], "B": [2, 9, 23, 40, 64, 100], "C": [3, 48, 65]}
 
 
-def build_trace(prompts: dict[str, list[int]], page: int):
+def build_trace(prompts: dict[str, list[int]], page: int, budget: int = 4 * 64):
     trace = TraceBuilder()
     # 1. each request alone and whole
     for name, tokens in prompts.items():
@@ -46,7 +46,7 @@ def build_trace(prompts: dict[str, list[int]], page: int):
     rng = torch.Generator().manual_seed(9)
     done = {name: 0 for name in names}
     waiting, live = list(names) + [], []
-    budget = 4 * 64  # tokens the pool holds; each live request counts rounded up to 64
+    # `budget`: tokens the pool holds; each live request counts rounded up to 64
     while waiting or live:
         while waiting and len(live) < 4 and sum(-(-len(prompts[n]) // 64) * 64 for n in live + [waiting[0]]) <= budget:
             live.append(waiting.pop(0))
@@ -99,3 +99,34 @@ def test_float32_cuts_agree_with_each_other_to_rounding(model_folders, tmp_path)
         whole = rows[("whole-p90", position)]
         for mode in ("cut", "mix"):
             torch.testing.assert_close(rows[(f"{mode}-p90", position)], whole, atol=3e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_at_benchmark_layer_sizes(tmp_path_factory, tmp_path, dtype):
+    """Two layers of the 1.5B benchmark widths (head size 128, six query heads a kv head): the same four
+    ways of cutting, with prompts that cross many pages and a pool that the three do not fit into together."""
+    folder = write_wide_folder(tmp_path_factory.mktemp("wide"))
+    plain_config, weights = plain.PlainConfig.from_folder(folder), plain.read_weights(folder)
+    prompts = {f"p{n}": random_tokens(n, WIDE.vocab_size, seed=300 + n) for n in (3, 130, 290)}
+    expected = {key: plain.forward(weights, plain_config, tokens) for key, tokens in prompts.items()}
+    trace = build_trace(prompts, PAGE_WIDE, budget=512)
+    results = replay(folder, dtype, trace.steps, tmp_path / "out", max_tokens=512, block_size=PAGE_WIDE,
+                     vocab=WIDE.vocab_size)
+    # These logits spread five times wider than the tiny models' (std 0.78: the width is 1536), so the bfloat16
+    # bound is stated in units of that spread: each of the ten or so roundings of an activation between kernels
+    # adds about 2^-9 of it, 0.6 % together; the largest of 1.7 million elements lies near five times that.
+    spread = float(torch.cat(list(expected.values())).std())
+    bound = TOLERANCE[dtype] if dtype == "float32" else dict(atol=0.06 * spread, rtol=3e-2)
+    total, count = 0.0, 0
+    for (request, position), logits in trace.collect(results).items():
+        mode, key = request.split("-", 1)
+        torch.testing.assert_close(
+            logits.double(), expected[key][position], **bound,
+            msg=lambda m: f"{mode} {key} position {position}: {m}",
+        )
+        total += float((logits.double() - expected[key][position]).abs().sum())
+        count += logits.numel()
+    print(f"{dtype}: mean error {total / count:.3e}, spread {spread:.3f}")
+    # a systematic fault that stays under the bound for the largest element still moves the mean
+    # (32-bit: sums over 8,960 terms in another order differ by about sqrt(8960) * 2^-24 of the spread)
+    assert total / count < (1e-5 if dtype == "float32" else 0.01) * spread

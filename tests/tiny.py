@@ -72,6 +72,31 @@ TINY_C = Qwen2Config(
 PAGE_C = 32
 
 
+# W: the layer sizes of the 1.5B benchmark configuration (head size 128, G = 6, widths 1536 and 8960)
+# with two layers and a small vocabulary that is no power of two: the kernels that serving picks at
+# real widths, inside a whole model.
+WIDE = Qwen2Config(
+    vocab_size=1031,
+    hidden_size=1536,
+    intermediate_size=8960,
+    num_layers=2,
+    num_attention_heads=12,
+    num_key_value_heads=2,
+    head_dim=128,
+    max_position_embeddings=4096,
+    rope_theta=1e6,
+    rms_norm_eps=1e-6,
+    attention_bias=True,
+    tie_word_embeddings=True,
+    rope_pairing="half",
+)
+PAGE_WIDE = 16
+
+
+def write_wide_folder(root: Path) -> Path:
+    return write_model_folder(root / "W", WIDE, seed=31, norm_std=0.1)
+
+
 def write_tiny_folders(root: Path) -> dict[str, Path]:
     return {
         # norm weights 1.0 as the reference initialises them, biases drawn
