@@ -202,13 +202,16 @@ __device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, St
 }
 
 template <int COLUMN_TILES, bool FUSED, int WAVES>
-__global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 1 : 2) void attention_tiles_kernel(
+__global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || WAVES > 4) ? 1 : 2) void attention_tiles_kernel(
     const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
     float* __restrict__ partial_ml, bf16_t* __restrict__ keys,
     bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
     int page_size, int page_shift, float scale, int window, int splits, FusedDecode fused) {
   extern __shared__ float lds[];  // [WAVES][16 columns][D + 2]
+  if (FUSED)  // a short kernel: fetch all arguments in one go rather than each before its first use
+    asm volatile("" ::"s"(row_width), "s"(table_width), "s"(heads), "s"(kv_heads), "s"(page_size), "s"(page_shift),
+                 "s"(scale), "s"(window), "s"(splits), "s"(fused.pairing));
   const int group = heads / kv_heads;
   const int kv_head = blockIdx.y % kv_heads, head_tile = blockIdx.y / kv_heads;
   const int heads_here = min(group - head_tile * 16, 16);
@@ -222,9 +225,44 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
   const ColumnMap map = {heads_here, FUSED ? 0 : item[2], FUSED ? (group <= 16 ? heads_here : 1) : item[3], group <= 16};
   const int tokens = map.tokens();
   const int position0 = positions[row0];
+  const int* table = block_tables + (size_t)request * table_width;
+  // FUSED: a step of single tokens is short, and what it takes is mostly the time its loads need to come
+  // back.  So everything the start of the kernel needs is asked for here at once, before anything is
+  // used: the pieces of the token's key and value row (one wave will store them; which one depends on the
+  // position, so all ask), the angles, and the pages of this wave's first step, looked up as if that
+  // step lay wholly inside the context (if it does not, they are looked up again below).
+  constexpr int PAIR_PIECES = (D / 2 + WAVE - 1) / WAVE, VALUE_PIECES = (D + WAVE - 1) / WAVE;
+  [[maybe_unused]] bf16_t new_a[PAIR_PIECES], new_b[PAIR_PIECES], new_v[VALUE_PIECES];
+  [[maybe_unused]] float2 new_angle[PAIR_PIECES];
+  [[maybe_unused]] int new_slot = -1;
+  [[maybe_unused]] int early_k = -1, early_k_hi = -1, early_v = -1;
+  const bool early_pages = FUSED && window <= 0 && splits == 1 && (wave * KEYS + KEYS - 1) / page_size < table_width;
+  if (FUSED) {
+    const bf16_t* k_row = qkv + (size_t)row0 * row_width + (size_t)(heads + kv_head) * D;
+    const bf16_t* v_row = k_row + (size_t)kv_heads * D;
+    // (the slot is the same for all lanes; asked for as if it were not, or the compiler waits for it right
+    // here to move it into a scalar register)
+    int no_offset;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(no_offset));
+    new_slot = fused.slots[row0 + no_offset];
+#pragma unroll
+    for (int i = 0; i < PAIR_PIECES; ++i) {
+      const int j = min(lane + i * WAVE, D / 2 - 1);
+      new_a[i] = k_row[fused.pairing == 2 ? j : 2 * j];
+      new_b[i] = k_row[fused.pairing == 2 ? j + D / 2 : 2 * j + 1];
+      if (fused.pairing != 0) new_angle[i] = fused.table[(size_t)row0 * (D / 2) + j];
+    }
+#pragma unroll
+    for (int i = 0; i < VALUE_PIECES; ++i) new_v[i] = v_row[min(lane + i * WAVE, D - 1)];
+    if (early_pages) {
+      const int key = wave * KEYS + 8 * (c >> 2) + (c & 3);
+      early_k = table[key / page_size];
+      early_k_hi = table[(key + 4) / page_size];
+      early_v = table[(wave * KEYS + 8 * q) / page_size];
+    }
+  }
   const int last_key = position0 + tokens - 1;
   const int first_key = window > 0 ? max(0, position0 - window + 1) : 0;
-  const int* table = block_tables + (size_t)request * table_width;
 
   // this lane's column in each of its column tiles
   Columns<COLUMN_TILES> columns;
@@ -249,13 +287,23 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
 #if HEAD_DIM % 32 == 0
     if (FUSED && fused.pairing != 0) {  // the queries come unrotated: rotate them here, in float32
       const float2* angles = fused.table + (size_t)(row0 + safe) * (D / 2);
-      if (fused.pairing == 1) {
+      // All angles are asked for before the first is used, and without a branch on the pairing (the
+      // compiler would otherwise wait for the queries before it asks).  Adjacent pairs: lane q rotates
+      // pairs 4q .. 4q+3 of every 16; halves: elements 8q .. 8q+7 of every 32 with their partners D/2 on.
+      float2 angle[QK_STEPS * 4];
+      const bool adjacent = fused.pairing == 1;
+#pragma unroll
+      for (int n = 0; n < QK_STEPS * 4; ++n)
+        angle[n] = angles[adjacent ? (n / 4) * 16 + q * 4 + n % 4 : (n / 8) * 32 + q * 8 + n % 8];
+      // the position is wanted in a scalar register from here on: ask now, not at its first use
+      asm volatile("" ::"s"(position0));
+      if (adjacent) {
 #pragma unroll
         for (int s = 0; s < QK_STEPS; ++s)
 #pragma unroll
           for (int pair = 0; pair < 4; ++pair) {
             float a = (float)query[t][s].v[2 * pair], b = (float)query[t][s].v[2 * pair + 1];
-            rotate_pair(a, b, angles[(s * 32 + q * 8) / 2 + pair]);
+            rotate_pair(a, b, angle[s * 4 + pair]);
             query[t][s].v[2 * pair] = (bf16_t)a;
             query[t][s].v[2 * pair + 1] = (bf16_t)b;
           }
@@ -265,7 +313,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             float a = (float)query[t][s].v[i], b = (float)query[t][s + QK_STEPS / 2].v[i];
-            rotate_pair(a, b, angles[s * 32 + q * 8 + i]);
+            rotate_pair(a, b, angle[s * 8 + i]);
             query[t][s].v[i] = (bf16_t)a;
             query[t][s + QK_STEPS / 2].v[i] = (bf16_t)b;
           }
@@ -289,27 +337,34 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
   const unsigned page_stride = (unsigned)kv_heads * page_size * D;  // elements of one page: checked to fit by the host
   const unsigned head_offset = (unsigned)kv_head * page_size * D;
 
-  if (FUSED && step_last >= step_begin && step_last < step_end) {
-    // this workgroup reads the newest key: it stores it first (one token per tile when FUSED; with
-    // more than 16 query heads per kv head several workgroups store the same values)
-    const int slot = fused.slots[row0];
-    if (slot >= 0 && wave == 0) {
-      const bf16_t* k_row = qkv + (size_t)row0 * row_width + (size_t)(heads + kv_head) * D;
-      const bf16_t* v_row = k_row + (size_t)kv_heads * D;
-      bf16_t* k_page = keys + (size_t)(slot / page_size) * page_stride + head_offset + (size_t)(slot % page_size) * D;
-      bf16_t* v_page = values + (size_t)(slot / page_size) * page_stride + head_offset + slot % page_size;
-      const float2* angles = fused.table + (size_t)row0 * (D / 2);
-      for (int j = lane; j < D / 2; j += WAVE) {
-        const int ia = fused.pairing == 2 ? j : 2 * j, ib = fused.pairing == 2 ? j + D / 2 : 2 * j + 1;
-        float a = (float)k_row[ia], b = (float)k_row[ib];
-        if (fused.pairing != 0) rotate_pair(a, b, angles[j]);
-        k_page[ia] = (bf16_t)a;
-        k_page[ib] = (bf16_t)b;
+  // FUSED: the wave that will read the newest key stores it (and the value) first; no other wave of the
+  // workgroup reads it
+  // (one token per tile when FUSED; with more than 16 query heads per kv head several workgroups store
+  // the same values)
+  const bool stores_token = FUSED && step_last >= step_begin && step_last < step_end &&
+                            wave == (step_last - step_begin) % WAVES;
+  if (stores_token && new_slot >= 0) {
+    bf16_t* k_page = keys + (size_t)(new_slot / page_size) * page_stride + head_offset + (size_t)(new_slot % page_size) * D;
+    bf16_t* v_page = values + (size_t)(new_slot / page_size) * page_stride + head_offset + new_slot % page_size;
+#pragma unroll
+    for (int i = 0; i < PAIR_PIECES; ++i) {
+      const int j = lane + i * WAVE;
+      if (j < D / 2) {
+        float a = (float)new_a[i], b = (float)new_b[i];
+        if (fused.pairing != 0) rotate_pair(a, b, new_angle[i]);
+        k_page[fused.pairing == 2 ? j : 2 * j] = (bf16_t)a;
+        k_page[fused.pairing == 2 ? j + D / 2 : 2 * j + 1] = (bf16_t)b;
       }
-      for (int d = lane; d < D; d += WAVE) v_page[(size_t)d * page_size] = v_row[d];
-      __threadfence_block();  // read again below by this workgroup only
     }
-    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < VALUE_PIECES; ++i) {
+      const int d = lane + i * WAVE;
+      if (d < D) v_page[(size_t)d * page_size] = new_v[i];
+    }
+    // Other lanes of this wave read these bytes back below.  A wave's accesses to memory are carried
+    // out in the order it issues them, so nothing has to be waited for; the fence keeps the compiler
+    // from moving the loads up.
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
   }
 
   // One step's loads.  The 32 keys of a step are dealt to the two 16-row tiles of the first product
@@ -368,7 +423,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192) ? 
   if (step_begin + wave < step_end) {
     const int step0 = step_begin + wave;
     StepLoads loads;
-    StepPages pages = pages_of(step0);
+    StepPages pages = early_pages && step0 < step_last ? StepPages{early_k, early_k_hi, early_v} : pages_of(step0);
     fetch_keys(step0, pages, loads);
     fetch_values(step0, pages, loads);
     if (step0 + WAVES < step_end) pages = pages_of(step0 + WAVES);
@@ -687,6 +742,10 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial_acc, co
   }
 }
 
+// waves of a workgroup of the fused decode form: eight walk a tile's keys where the registers allow it
+#ifndef FUSED_WAVES
+#define FUSED_WAVES (HEAD_DIM > 128 ? 4 : 8)
+#endif
 template <int COLUMN_TILES, bool FUSED, int WAVES>
 static int launch_tiles(const void* qkv, int row_width, void* out, float* partial_acc, float* partial_ml,
                         void* keys, void* values, const int* block_tables, int table_width,
@@ -749,7 +808,7 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   if (fuse) {
     if (column_tiles != 1 || tiles != rows || !slots || !llmserve_attention_can_fuse(pairing) || (pairing != 0 && !table))
       return ERR_BAD_ARGUMENT;
-    status = launch_tiles<1, true, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
+    status = launch_tiles<1, true, FUSED_WAVES>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
                                         table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile,
                                         page_size, scale, window, splits, fused, stream);
   } else if (column_tiles == 1) {

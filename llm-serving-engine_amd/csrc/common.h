@@ -47,13 +47,9 @@ __device__ __forceinline__ float block_sum(float v, float* shared /* >= 17 float
   __syncthreads();
   if (lane == 0) shared[wave] = v;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    float total = 0.f;
-    for (int i = 0; i < waves; ++i) total += shared[i];
-    shared[16] = total;
-  }
-  __syncthreads();
-  return shared[16];
+  float total = 0.f;  // every thread adds the waves' sums itself, in the same order
+  for (int i = 0; i < waves; ++i) total += shared[i];
+  return total;
 }
 
 __device__ __forceinline__ float block_max(float v, float* shared /* >= 17 floats */) {

@@ -53,71 +53,85 @@ __global__ void add_rms_norm_kernel(float* __restrict__ hidden, const float* __r
     dst[i] = from_float<TO>(row[i] * scale * load_as_float(weight, weight_is_float, i));
 }
 
-// The same for rows of up to 256 * 4 * VECTORS floats whose length is a multiple of 4: the row
-// stays in registers between the two passes and moves in 16-byte pieces.
-#define NORM_VECTORS 8
-template <int PARTS>
-__device__ __forceinline__ void add_parts(float4 (&v)[NORM_VECTORS], const float* from, size_t part_stride, int quads) {
+// The same for rows whose length is a multiple of 4, up to 16,384 floats: the row stays in
+// registers between the two passes and moves in 16-byte pieces.  The block has a thread for every
+// piece of a row of up to 4,096 floats (PIECES = 1; 2 or 4 pieces a thread beyond), so that all of
+// a thread's loads (its piece of the row, of the weight and of every partial sum) are on their way
+// before the first is used: on a short row the kernel takes as long as its loads need to come
+// back, and a second piece per thread would be a second trip.  Piece j of a thread is quad
+// min(threadIdx.x + j * blockDim.x, quads - 1): threads past the end read the last quad again and
+// store nothing, so the loads need no branch.
+template <int PARTS, int PIECES>
+__device__ __forceinline__ void add_parts(float4 (&v)[PIECES], const float* from, size_t part_stride, int quads) {
 #pragma unroll
-  for (int j = 0; j < NORM_VECTORS; ++j) {
-    const int i = threadIdx.x + j * 256;
-    if (i < quads) {
-      float4 d[PARTS];
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = min((int)(threadIdx.x + j * blockDim.x), quads - 1);
+    float4 d[PARTS];
 #pragma unroll
-      for (int p = 0; p < PARTS; ++p) d[p] = ((const float4*)(from + (size_t)p * part_stride))[i];
+    for (int p = 0; p < PARTS; ++p) d[p] = ((const float4*)(from + (size_t)p * part_stride))[i];
 #pragma unroll
-      for (int p = 0; p < PARTS; ++p) {
-        v[j].x += d[p].x; v[j].y += d[p].y; v[j].z += d[p].z; v[j].w += d[p].w;
-      }
+    for (int p = 0; p < PARTS; ++p) {
+      v[j].x += d[p].x; v[j].y += d[p].y; v[j].z += d[p].z; v[j].w += d[p].w;
     }
   }
 }
 
-template <typename TO>
-__global__ __launch_bounds__(256) void add_rms_norm_vector_kernel(float* __restrict__ hidden,
-                                                                  const float* __restrict__ delta, int parts,
-                                                                  size_t part_stride,
-                                                                  const void* __restrict__ weight,
-                                                                  int weight_is_float, TO* __restrict__ out,
-                                                                  int width, float eps) {
+template <int PIECES>
+__device__ __forceinline__ void add_some_parts(float4 (&v)[PIECES], const float* from, int count, size_t part_stride,
+                                               int quads) {
+  switch (count) {
+    case 1: add_parts<1, PIECES>(v, from, part_stride, quads); break;
+    case 2: add_parts<2, PIECES>(v, from, part_stride, quads); break;
+    case 3: add_parts<3, PIECES>(v, from, part_stride, quads); break;
+    case 4: add_parts<4, PIECES>(v, from, part_stride, quads); break;
+    case 5: add_parts<5, PIECES>(v, from, part_stride, quads); break;
+    case 6: add_parts<6, PIECES>(v, from, part_stride, quads); break;
+    case 7: add_parts<7, PIECES>(v, from, part_stride, quads); break;
+    default: add_parts<8, PIECES>(v, from, part_stride, quads); break;
+  }
+}
+
+__device__ __forceinline__ void store_four(float* dst, float a, float b, float c, float d) {
+  *(float4*)dst = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void store_four(bf16_t* dst, float a, float b, float c, float d) {
+  typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
+  *(bf16x4*)dst = (bf16x4){(bf16_t)a, (bf16_t)b, (bf16_t)c, (bf16_t)d};
+}
+
+template <typename TO, int PIECES>
+__global__ __launch_bounds__(1024) void add_rms_norm_vector_kernel(float* __restrict__ hidden,
+                                                                   const float* __restrict__ delta, int parts,
+                                                                   size_t part_stride,
+                                                                   const void* __restrict__ weight,
+                                                                   int weight_is_float, TO* __restrict__ out,
+                                                                   int width, float eps) {
   __shared__ float shared[17];
   const int quads = width / 4;
   float4* row = (float4*)(hidden + (size_t)blockIdx.x * width);
   const float* add = delta ? delta + (size_t)blockIdx.x * width : nullptr;
-  float4 v[NORM_VECTORS], w[NORM_VECTORS];
-  float squares = 0.f;
+  float4 v[PIECES], wide[PIECES];
+  uint2 narrow[PIECES];  // four bfloat16 weights as they lie in memory: converted after the loads
 #pragma unroll
-  for (int j = 0; j < NORM_VECTORS; ++j) {
-    const int i = threadIdx.x + j * 256;
-    if (i < quads) {
-      v[j] = row[i];
-      if (weight_is_float) {
-        w[j] = ((const float4*)weight)[i];
-      } else {
-        const bf16_t* wb = (const bf16_t*)weight + 4 * i;
-        w[j] = make_float4((float)wb[0], (float)wb[1], (float)wb[2], (float)wb[3]);
-      }
-    }
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = min((int)(threadIdx.x + j * blockDim.x), quads - 1);
+    v[j] = row[i];
+    if (weight_is_float)
+      wide[j] = ((const float4*)weight)[i];
+    else
+      narrow[j] = ((const uint2*)weight)[i];
   }
   if (add) {
-    // the parts are added in order, up to eight at a time: their loads are all requested before the first is used
-    for (int first = 0; first < parts; first += 8) {
-      const float* from = add + (size_t)first * part_stride;
-      switch (min(parts - first, 8)) {
-        case 1: add_parts<1>(v, from, part_stride, quads); break;
-        case 2: add_parts<2>(v, from, part_stride, quads); break;
-        case 3: add_parts<3>(v, from, part_stride, quads); break;
-        case 4: add_parts<4>(v, from, part_stride, quads); break;
-        case 5: add_parts<5>(v, from, part_stride, quads); break;
-        case 6: add_parts<6>(v, from, part_stride, quads); break;
-        case 7: add_parts<7>(v, from, part_stride, quads); break;
-        default: add_parts<8>(v, from, part_stride, quads); break;
-      }
-    }
+    // the parts are added in order, up to eight at a time: their loads are all requested before the
+    // first is used (the first eight outside the loop, so that they need not wait for the row's piece)
+    add_some_parts<PIECES>(v, add, min(parts, 8), part_stride, quads);
+    for (int first = 8; first < parts; first += 8)
+      add_some_parts<PIECES>(v, add + (size_t)first * part_stride, min(parts - first, 8), part_stride, quads);
   }
+  float squares = 0.f;
 #pragma unroll
-  for (int j = 0; j < NORM_VECTORS; ++j) {
-    const int i = threadIdx.x + j * 256;
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
     if (i < quads) {
       if (add) row[i] = v[j];
       squares += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
@@ -127,15 +141,35 @@ __global__ __launch_bounds__(256) void add_rms_norm_vector_kernel(float* __restr
   const float scale = rsqrtf(total / (float)width + eps);
   TO* dst = out + (size_t)blockIdx.x * width;
 #pragma unroll
-  for (int j = 0; j < NORM_VECTORS; ++j) {
-    const int i = threadIdx.x + j * 256;
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
     if (i < quads) {
-      dst[4 * i + 0] = from_float<TO>(v[j].x * scale * w[j].x);
-      dst[4 * i + 1] = from_float<TO>(v[j].y * scale * w[j].y);
-      dst[4 * i + 2] = from_float<TO>(v[j].z * scale * w[j].z);
-      dst[4 * i + 3] = from_float<TO>(v[j].w * scale * w[j].w);
+      float4 w = wide[j];
+      if (!weight_is_float)  // a bfloat16 is the upper half of the float32 of the same value
+        w = make_float4(__uint_as_float(narrow[j].x << 16), __uint_as_float(narrow[j].x & 0xffff0000u),
+                        __uint_as_float(narrow[j].y << 16), __uint_as_float(narrow[j].y & 0xffff0000u));
+      store_four(dst + 4 * i, v[j].x * scale * w.x, v[j].y * scale * w.y, v[j].z * scale * w.z, v[j].w * scale * w.w);
     }
   }
+}
+
+template <typename TO>
+static void launch_add_rms_norm_vector(float* hidden, const float* delta, int parts, size_t part_stride,
+                                       const void* weight, int weight_is_float, TO* out, int rows, int width,
+                                       float eps, hipStream_t stream) {
+  // a thread for every four floats of the row, in whole waves: the block size depends on the width alone
+  const int quads = width / 4;
+  const int pieces = quads <= 1024 ? 1 : quads <= 2048 ? 2 : 4;
+  const int threads = ((quads + pieces - 1) / pieces + WAVE - 1) / WAVE * WAVE;
+  if (pieces == 1)
+    hipLaunchKernelGGL((add_rms_norm_vector_kernel<TO, 1>), dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, weight_is_float, out, width, eps);
+  else if (pieces == 2)
+    hipLaunchKernelGGL((add_rms_norm_vector_kernel<TO, 2>), dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, weight_is_float, out, width, eps);
+  else
+    hipLaunchKernelGGL((add_rms_norm_vector_kernel<TO, 4>), dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, weight_is_float, out, width, eps);
 }
 
 extern "C" int llmserve_add_rms_norm(float* hidden, const float* delta, int parts, const void* weight,
@@ -144,13 +178,13 @@ extern "C" int llmserve_add_rms_norm(float* hidden, const float* delta, int part
   if (rows <= 0) return 0;
   if (delta && parts < 1) return ERR_BAD_ARGUMENT;
   const size_t part_stride = (size_t)rows * width;
-  if (width % 4 == 0 && width <= 256 * 4 * NORM_VECTORS) {
+  if (width % 4 == 0 && width <= 1024 * 4 * 4) {
     if (out_is_float)
-      hipLaunchKernelGGL(add_rms_norm_vector_kernel<float>, dim3(rows), dim3(256), 0, stream, hidden, delta, parts,
-                         part_stride, weight, weight_is_float, (float*)out, width, eps);
+      launch_add_rms_norm_vector<float>(hidden, delta, parts, part_stride, weight, weight_is_float, (float*)out, rows,
+                                        width, eps, stream);
     else
-      hipLaunchKernelGGL(add_rms_norm_vector_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, hidden, delta, parts,
-                         part_stride, weight, weight_is_float, (bf16_t*)out, width, eps);
+      launch_add_rms_norm_vector<bf16_t>(hidden, delta, parts, part_stride, weight, weight_is_float, (bf16_t*)out,
+                                         rows, width, eps, stream);
     return LAUNCH_STATUS();
   }
   const int threads = width >= 2048 ? 512 : 256;
