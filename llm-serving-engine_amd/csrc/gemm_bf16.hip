@@ -52,6 +52,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // the bias of this lane's four outputs is asked for now and used at the end
+  const bool with_bias = bias && blockIdx.y == 0;
+  // (as 16-bit halves, so that both types of bias take the same loads: a float32 is two of them, a
+  // bfloat16 the upper one alone)
+  // (without a branch: where there is no bias the same loads read the start of the weights and
+  // their result is dropped; loads inside a branch would be waited for at its end)
+  unsigned short bias_low[4], bias_high[4];
+  {
+    const unsigned short* source = with_bias ? (const unsigned short*)bias : (const unsigned short*)w;
+    const int halves = with_bias && bias_is_float ? 2 : 1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int at = min((int)blockIdx.x * 16 + g * 4 + i, N - 1) * halves;
+      bias_low[i] = source[at];
+      bias_high[i] = source[at + halves - 1];
+    }
+  }
 
   const int groups = k_split / (STEP * GROUP);
   bf16x8 a[GROUP], a_next[GROUP];
@@ -99,10 +116,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   const int m = t * 16 + r;
   const int n_first = blockIdx.x * 16 + g * 4;
   if (m >= M) return;
-  if (bias && blockIdx.y == 0) {
+  if (with_bias) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (n_first + i < N) total[i] += load_as_float(bias, bias_is_float, n_first + i);
+      total[i] += __uint_as_float((unsigned)bias_high[i] << 16 | (bias_is_float ? (unsigned)bias_low[i] : 0u));
   }
   if (GATED) {
     TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
