@@ -33,6 +33,14 @@ class TokenEvent:
     token: int
 
 
+@dataclass
+class _StepInFlight:
+    """A decode step that was queued before the tokens it consumes had reached the host."""
+
+    requests: list[RequestState]  # row i of `logits` is requests[i]
+    logits: torch.Tensor
+
+
 class EngineCore:
     """One iteration at a time over a `ModelRunner`."""
 
@@ -45,6 +53,7 @@ class EngineCore:
         prefill_chunk_size: int = 16,
         collect_iteration_metrics: bool = False,
         look_ahead: bool = True,
+        run_ahead: bool = True,
     ) -> None:
         scheduler_config = scheduler_config or SchedulerConfig()
         if prefill_chunk_size <= 0:
@@ -61,6 +70,11 @@ class EngineCore:
         self.collect_iteration_metrics = collect_iteration_metrics
         self.look_ahead = look_ahead  # prepare the next decode step on the host while the device runs this one
         self._expected: list[RequestState] | None = None  # the requests of the step that is prepared
+        # Queue the next decode step behind the sampling of this one, its tokens passed on the device:
+        # the device then never waits for the host between two steps.  A request that turns out to have
+        # ended (a stop token) has a row in that step that nobody reads.
+        self.run_ahead = run_ahead and look_ahead
+        self._in_flight: _StepInFlight | None = None
         self.generation_configs: dict[str, GenerationConfig] = {}
         self.finished: list[RequestState] = []
         self._cpu_ms = {"prefill": 0.0, "decode": 0.0, "mixed": 0.0}
@@ -139,42 +153,65 @@ class EngineCore:
                     self._events[phase].append(events)
 
     def _run_iteration(self, active: list[RequestState]) -> list[TokenEvent]:
-        expected, self._expected = self._expected, None
-        if expected is not None and len(expected) == len(active) and all(a is b for a, b in zip(expected, active)):
-            # the step that was prepared while the last one ran: every request brings the token it
-            # has just been given, and the runner holds the cache entries already
-            planned = [(request, 1) for request in active]
+        in_flight, self._in_flight = self._in_flight, None
+        if in_flight is not None and any(not request.finished for request in in_flight.requests):
+            # this iteration's step runs already: its requests each brought the token they had just been given
+            rows = in_flight.requests
+            logits = in_flight.logits
+            planned = [(request, 1) for request in rows if not request.finished]
+            if self.step_log is not None:
+                self.step_log.append([(request.request_id, 1) for request, _ in planned])
         else:
-            planned = self._plan(active)
-            if planned is None:
-                return []
-        if self.step_log is not None:
-            self.step_log.append([(request.request_id, count) for request, count in planned])
+            expected, self._expected = self._expected, None
+            if expected is not None and len(expected) == len(active) and all(a is b for a, b in zip(expected, active)):
+                # the step that was prepared while the last one ran: every request brings the token it
+                # has just been given, and the runner holds the cache entries already
+                planned = [(request, 1) for request in active]
+            else:
+                planned = self._plan(active)
+                if planned is None:
+                    return []
+            if self.step_log is not None:
+                self.step_log.append([(request.request_id, count) for request, count in planned])
 
-        entries, sampled = [], []
-        for request, count in planned:
-            tokens = request.tokens_between(request.processed_tokens, request.processed_tokens + count)
-            last = request.processed_tokens + count == len(request.prompt_token_ids) + len(request.generated_token_ids)
-            entries.append(StepEntry(request.request_id, tokens, (count - 1,) if last else ()))
-            if last:  # otherwise: a portion of a prompt, or a replay after preemption
-                sampled.append(request)
-        logits = self.runner.step(entries, fits_checked=True)
+            entries, rows = [], []
+            for request, count in planned:
+                tokens = request.tokens_between(request.processed_tokens, request.processed_tokens + count)
+                last = request.processed_tokens + count == len(request.prompt_token_ids) + len(request.generated_token_ids)
+                entries.append(StepEntry(request.request_id, tokens, (count - 1,) if last else ()))
+                if last:  # otherwise: a portion of a prompt, or a replay after preemption
+                    rows.append(request)
+            logits = self.runner.step(entries, fits_checked=True)
         for request, count in planned:
             request.processed_tokens += count
+        sampled = [request for request in rows if not request.finished]
         if not sampled:
             return []
-        configs = [self.generation_configs[request.request_id] for request in sampled]
-        steps = [len(request.generated_token_ids) for request in sampled]
-        if self.look_ahead and len(sampled) == len(planned) == len(active) and not self.scheduler.waiting:
+        greedy = GenerationConfig()
+        configs = [self.generation_configs.get(request.request_id, greedy) for request in rows]
+        steps = [len(request.generated_token_ids) for request in rows]
+        tokens = None
+        if self.look_ahead and len(sampled) == len(rows) == len(planned) == len(active) and not self.scheduler.waiting:
             # Every running request has just decoded and nothing waits: unless a stop token comes,
             # the next step is these requests again, less those at their last token.  The runner does
             # its host work for that step now, while the device is still busy with this one.
             staying = [r for r in sampled if len(r.generated_token_ids) + 1 < r.max_new_tokens]
             if self.runner.prepare_decode([r.request_id for r in staying]):
-                self._expected = staying
-        tokens = self.sampler.sample(logits, configs, steps)
+                if self.run_ahead and len(staying) == len(rows):
+                    # and queues it: the tokens go from the sampler to the step on the device
+                    chosen = self.sampler.sample_on_device(logits, configs, steps)
+                    fetch = self.runner.fetch_later(chosen)
+                    next_logits = self.runner.step_from_device([r.request_id for r in staying], chosen)
+                    self._in_flight = _StepInFlight(staying, next_logits)
+                    tokens = fetch()
+                else:
+                    self._expected = staying
+        if tokens is None:
+            tokens = self.sampler.sample(logits, configs, steps)
         produced = []
-        for request, config, token in zip(sampled, configs, tokens):
+        for request, config, token in zip(rows, configs, tokens):
+            if request.finished:  # a row of a step queued before its request's end was known
+                continue
             request.generated_token_ids.append(token)
             produced.append(TokenEvent(request, token))
             if len(request.generated_token_ids) >= request.max_new_tokens or token in config.stop_token_ids:

@@ -224,6 +224,39 @@ class ModelRunner:
             self._packed_ahead = (tuple(request_ids), *self._pack_decode(reservations, entries))
         return True
 
+    def step_from_device(self, request_ids: list[str], tokens: torch.Tensor) -> torch.Tensor:
+        """The step that `prepare_decode(request_ids)` has just prepared, with request i's token taken
+        from `tokens[i]`, an integer tensor on the device (the sampler's output for the step before):
+        the step is queued behind the work that produces the tokens, and the host never waits for
+        them.  Returns what `step` returns."""
+        if set(self._ahead) != set(request_ids) or len(tokens) != len(request_ids):
+            raise RuntimeError("step_from_device follows prepare_decode for the same requests")
+        ahead = self._packed_ahead
+        if ahead is None:  # no graphs here (a host run): the tokens are read after all
+            entries = [StepEntry(request_id, (int(token),), (0,)) for request_id, token in zip(request_ids, tokens.tolist())]
+            return self.step(entries, fits_checked=True)
+        reservations = [self._ahead[request_id] for request_id in ahead[0]]
+        self._ahead.clear()
+        self._packed_ahead = None
+        return self._decode_with_graph(reservations, None, ahead[1:], device_tokens=tokens)
+
+    def fetch_later(self, values: torch.Tensor):
+        """Queues a copy of a small integer tensor to the host behind the work queued so far; returns a
+        function that waits for that copy, and not for what is queued after this call, and gives the
+        values as a list."""
+        if self.device.type != "cuda":
+            return values.tolist
+        host = torch.empty(values.shape, dtype=values.dtype, pin_memory=True)
+        host.copy_(values, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+
+        def result() -> list[int]:
+            done.synchronize()
+            return host.tolist()
+
+        return result
+
     def _cancel_ahead(self) -> None:
         for reservation in self._ahead.values():
             self.cache.cancel(reservation)
@@ -326,16 +359,20 @@ class ModelRunner:
         return ((requests, width), *_pack_step(reservations, entries, self.cache, pad_to=requests, width=width))
 
     @torch.inference_mode()
-    def _decode_with_graph(self, reservations: list[Reservation], entries: list[StepEntry], packed_ahead=None) -> torch.Tensor:
+    def _decode_with_graph(
+        self, reservations: list[Reservation], entries: list[StepEntry] | None, packed_ahead=None, device_tokens=None
+    ) -> torch.Tensor:
         """A step of single tokens, one per request, replayed from a HIP graph: the launches
         of a decode step cost more on the host than the step takes on the device.  Graphs are
         kept per (requests rounded up to a power of two, block-table width likewise); the
         step's index arrays go into the graph's static buffer and the same kernels run.
         `packed_ahead` is what `_pack_decode` made of the same reservations before the tokens
-        were known: the token ids, which lead the arrays, are filled in."""
+        were known: the token ids, which lead the arrays, are filled in, from `entries` or, on the
+        device, from `device_tokens`."""
         if packed_ahead is not None:
             key, packed, sizes, widths, facts = packed_ahead
-            packed[: len(entries)] = [entry.tokens[0] for entry in entries]
+            if entries is not None:
+                packed[: len(entries)] = [entry.tokens[0] for entry in entries]
         else:
             key, packed, sizes, widths, facts = self._pack_decode(reservations, entries)
         graph = self._graphs.get(key)
@@ -350,6 +387,8 @@ class ModelRunner:
         event = torch.cuda.Event()
         event.record()
         graph.copied[turn] = event
+        if device_tokens is not None:
+            graph.static[: len(reservations)].copy_(device_tokens)
         graph.graph.replay()
         return graph.logits[: len(reservations)]
 

@@ -48,10 +48,14 @@ class Sampler:
     def sample(self, logits: torch.Tensor, configs: list[GenerationConfig], steps: list[int]) -> list[int]:
         """`steps[i]` is the number of tokens row i's request has sampled before.
         One device-to-host copy for the whole batch (`engine.py:44-72`)."""
+        return self.sample_on_device(logits, configs, steps).cpu().tolist()
+
+    def sample_on_device(self, logits: torch.Tensor, configs: list[GenerationConfig], steps: list[int]) -> torch.Tensor:
+        """The same, left on the device as an integer tensor [rows]: nothing waits for the result."""
         if logits.ndim != 2 or logits.shape[0] != len(configs) or len(configs) != len(steps):
             raise ValueError("batched sampling inputs must have matching rows")
         if all(config.temperature <= 0 for config in configs):
-            return self.kernels.argmax(logits).cpu().tolist()
+            return self.kernels.argmax(logits)
         values = torch.tensor(
             [
                 [config.temperature for config in configs],
@@ -61,4 +65,4 @@ class Sampler:
             dtype=torch.float32,
         )
         values = self.kernels.to_device(values)
-        return self.kernels.sample(logits, values[0], values[1], values[2]).cpu().tolist()
+        return self.kernels.sample(logits, values[0], values[1], values[2])

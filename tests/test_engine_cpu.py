@@ -245,17 +245,27 @@ def test_pages_run_out_the_largest_gives_way_and_replays(model_folders):
 
 
 def test_looking_ahead_changes_no_decision(model_folders):
-    """While a decode step runs, the engine has the runner reserve and pack the next one.  With
-    requests that arrive late, stop early and give way for want of pages, every plan and every
-    token is what it is without looking ahead, and nothing stays reserved."""
+    """While a decode step runs, the engine has the runner reserve and pack the next one, and queues
+    it before this one's tokens have reached the host.  With requests that arrive late, stop early
+    (a stop token is seen only after the next step was queued) and give way for want of pages,
+    every plan and every token is what it is without either, and nothing stays reserved."""
     config, weights = oracle(model_folders, "A")
     prompts = [random_tokens(n, config.vocab_size, seed=70 + n) for n in (20, 9, 26, 3)]
     free_run = [plain.generate(weights, config, prompt, 12) for prompt in prompts]
     stops = [(), (free_run[1][9],), (free_run[2][2],), ()]  # two requests stop on a token of their own
-    outcomes = []
-    for look_ahead in (True, False):
+    outcomes, queued_ahead = [], []
+    # (prepare the next step while this one runs, and queue it before this one's tokens are read)
+    for look_ahead, run_ahead in ((True, True), (True, False), (False, False)):
         core = core_for(model_folders, "A", num_blocks=3, batch=3, budget=12, chunk=8)
-        core.look_ahead = look_ahead
+        core.look_ahead, core.run_ahead = look_ahead, run_ahead
+        queued_ahead.append(0)
+        from_device = core.runner.step_from_device
+
+        def counted(*args, _inner=from_device, **kwargs):
+            queued_ahead[-1] += 1
+            return _inner(*args, **kwargs)
+
+        core.runner.step_from_device = counted
         requests = [RequestState(f"r{i}", prompt, 12) for i, prompt in enumerate(prompts)]
         for request, stop in zip(requests[:2], stops):
             core.submit(request, GenerationConfig(max_new_tokens=12, stop_token_ids=stop))
@@ -271,7 +281,8 @@ def test_looking_ahead_changes_no_decision(model_folders):
         assert not core.runner._ahead and core.runner.cache.used_pages == 0
         assert all(request.error is None for request in requests)
         outcomes.append((core.step_log, [r.generated_token_ids for r in requests], [r.preemptions for r in requests]))
-    assert outcomes[0] == outcomes[1]
+    assert outcomes[0] == outcomes[1] == outcomes[2]
+    assert queued_ahead[0] > 5 and queued_ahead[1:] == [0, 0]
     assert sum(outcomes[0][2]) > 0  # pages did run out
     for tokens, whole, stop in zip(outcomes[0][1], free_run, stops):
         cut = whole.index(stop[0]) + 1 if stop else len(whole)
