@@ -262,11 +262,79 @@ __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const float2* __res
   }
 }
 
+// The same for bfloat16 heads whose size is a multiple of 16, in 16-byte pieces: a thread takes 16
+// elements of a q or k head (two pieces that hold eight pairs: with adjacent pairs elements 16p ..
+// 16p + 15, with half pairs 8p .. 8p + 7 and their partners dim/2 on), rotates them, writes them
+// back, and, for a k head, writes them to the page as well; further threads take eight elements of
+// a v head each.  Threads are dealt to (token, piece) pairs without regard to blocks.
+__global__ __launch_bounds__(256) void rotate_and_store_vector_kernel(
+    bf16_t* __restrict__ qkv, const float2* __restrict__ table, int pairing, int heads, int kv_heads, int dim,
+    bf16_t* __restrict__ keys, bf16_t* __restrict__ values, const int* __restrict__ slots, int page_size, int tokens) {
+  typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+  const int per_head = dim / 16, half = dim / 2;
+  const int rotated = (heads + kv_heads) * per_head, pieces = rotated + kv_heads * (dim / 8);
+  const size_t id = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int token = (int)(id / pieces), piece = (int)(id % pieces);
+  if (token >= tokens) return;
+  bf16_t* row = qkv + (size_t)token * (heads + 2 * kv_heads) * dim;
+  const int slot = slots ? slots[token] : -1;
+  if (piece < rotated) {
+    const int head = piece / per_head, p = piece % per_head;
+    bf16_t* h = row + head * dim;
+    const int ia = pairing == 2 ? 8 * p : 16 * p, ib = pairing == 2 ? 8 * p + half : 16 * p + 8;
+    bf16x8 a = *(const bf16x8*)(h + ia), b = *(const bf16x8*)(h + ib);
+    if (pairing != 0) {
+      float2 cs[8];
+      const float2* angles = table + (size_t)token * half + 8 * p;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) cs[i] = angles[i];
+      if (pairing == 2) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float x = (float)a[i], y = (float)b[i];
+          a[i] = (bf16_t)(x * cs[i].x - y * cs[i].y);
+          b[i] = (bf16_t)(y * cs[i].x + x * cs[i].y);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float x = (float)a[2 * i], y = (float)a[2 * i + 1];
+          a[2 * i] = (bf16_t)(x * cs[i].x - y * cs[i].y);
+          a[2 * i + 1] = (bf16_t)(y * cs[i].x + x * cs[i].y);
+          const float u = (float)b[2 * i], v = (float)b[2 * i + 1];
+          b[2 * i] = (bf16_t)(u * cs[4 + i].x - v * cs[4 + i].y);
+          b[2 * i + 1] = (bf16_t)(v * cs[4 + i].x + u * cs[4 + i].y);
+        }
+      }
+      *(bf16x8*)(h + ia) = a;
+      *(bf16x8*)(h + ib) = b;
+    }
+    if (head >= heads && slot >= 0) {
+      bf16_t* k_row = keys + (((size_t)(slot / page_size) * kv_heads + (head - heads)) * page_size + slot % page_size) * dim;
+      *(bf16x8*)(k_row + ia) = a;
+      *(bf16x8*)(k_row + ib) = b;
+    }
+  } else if (slot >= 0) {
+    const int at = piece - rotated, head = at / (dim / 8), d0 = (at % (dim / 8)) * 8;
+    const bf16x8 v = *(const bf16x8*)(row + (size_t)(heads + kv_heads + head) * dim + d0);
+    bf16_t* v_page = values + ((size_t)(slot / page_size) * kv_heads + head) * page_size * dim + slot % page_size;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v_page[(size_t)(d0 + e) * page_size] = v[e];
+  }
+}
+
 extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const float* table, int pairing, int tokens,
                                          int heads, int kv_heads, int dim, void* keys, void* values,
                                          const int* slots, int page_size, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (dim % 2 || (pairing != 0 && table == nullptr) || pairing < 0 || pairing > 2) return ERR_BAD_ARGUMENT;
+  if (!is_float && dim % 16 == 0) {
+    const size_t threads = (size_t)tokens * ((heads + kv_heads) * (dim / 16) + kv_heads * (dim / 8));
+    hipLaunchKernelGGL(rotate_and_store_vector_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                       (bf16_t*)qkv, (const float2*)table, pairing, heads, kv_heads, dim, (bf16_t*)keys,
+                       (bf16_t*)values, slots, page_size, tokens);
+    return LAUNCH_STATUS();
+  }
   if (is_float)
     hipLaunchKernelGGL(rotate_and_store_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float*)qkv,
                        (const float2*)table, pairing, heads, kv_heads, dim, (float*)keys, (float*)values, slots,
@@ -292,9 +360,34 @@ __global__ void silu_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out,
   }
 }
 
+// The same for bfloat16 rows whose width is a multiple of 8: a thread takes eight outputs, 32 bytes in
+// (two 16-byte loads, both on their way before the first is used) and 16 bytes out.
+__global__ __launch_bounds__(256) void silu_mul_vector_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out,
+                                                              size_t octets) {
+  typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+  const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (at >= octets) return;
+  const bf16x8 first = ((const bf16x8*)in)[2 * at], second = ((const bf16x8*)in)[2 * at + 1];
+  bf16x8 result;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float gate = (float)first[2 * i], up = (float)first[2 * i + 1];
+    result[i] = (bf16_t)(gate / (1.f + expf(-gate)) * up);
+    const float gate2 = (float)second[2 * i], up2 = (float)second[2 * i + 1];
+    result[4 + i] = (bf16_t)(gate2 / (1.f + expf(-gate2)) * up2);
+  }
+  ((bf16x8*)out)[at] = result;
+}
+
 extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
                                  hipStream_t stream) {
   if (rows <= 0) return 0;
+  if (!in_is_float && !out_is_float && width % 8 == 0) {  // rows are contiguous: the whole is one run of octets
+    const size_t octets = (size_t)rows * (width / 8);
+    hipLaunchKernelGGL(silu_mul_vector_kernel, dim3((unsigned)((octets + 255) / 256)), dim3(256), 0, stream,
+                       (const bf16_t*)in, (bf16_t*)out, octets);
+    return LAUNCH_STATUS();
+  }
   // a row is cut over several blocks when the rows alone would not fill the chip
   const int pieces = rows >= 1024 ? 1 : max(1, min((width + 255) / 256, 1024 / rows));
   const dim3 grid(rows, pieces), block(256);
