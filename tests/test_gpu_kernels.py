@@ -338,6 +338,27 @@ def test_rotate_and_store(kernels, dtype, pairing, heads, kv_heads, dim, page):
     torch.testing.assert_close(again, qkv)
 
 
+@pytest.mark.parametrize("width,parts", [(64, 1), (1536, 3), (4096, 8), (5120, 11), (12292, 2), (16384, 17), (4102, 9)])
+def test_add_rms_norm_of_partial_sums(kernels, width, parts):
+    """What a product cut over K leaves: [parts, rows, width] partial sums, added in order.  Widths
+    with one, two and four pieces a thread, the widest the register-resident kernel takes, and one
+    that is no multiple of four (the plain kernel)."""
+    rows = 5
+    hidden, delta = torch.randn(rows, width), 0.3 * torch.randn(parts, rows, width)
+    weight = 1 + 0.2 * torch.randn(width)
+    k = kernels[torch.bfloat16]
+    device_hidden = on_gpu(hidden.clone())
+    out = k.add_rms_norm(device_hidden, on_gpu(delta), on_gpu(weight, torch.bfloat16), 1e-6)
+    summed = hidden.double() + delta.double().sum(0)
+    torch.testing.assert_close(device_hidden.cpu().double(), summed, atol=2e-6, rtol=1e-6)
+    expected = plain.rms_norm(summed, rounded(weight, torch.bfloat16), 1e-6)
+    torch.testing.assert_close(out.cpu().double(), expected, **TOLERANCE[torch.bfloat16])
+    # a row's result does not depend on how many rows there are
+    one = on_gpu(hidden[2:3].clone())
+    alone = k.add_rms_norm(one, on_gpu(delta[:, 2:3].contiguous()), on_gpu(weight, torch.bfloat16), 1e-6)
+    assert torch.equal(alone[0], out[2]) and torch.equal(one[0], device_hidden[2])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gather_rows(kernels, dtype):
     hidden, delta = torch.randn(9, 100), torch.randn(9, 100)
