@@ -13,6 +13,7 @@
 // With `gated`, weight rows alternate gate_j, up_j and the epilogue writes
 // silu(gate) * up (reference model.py:188) to out[M, N / 2].
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -352,76 +353,106 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define TILE_STRIDE (TILE_K + 8)  // bf16 elements per staged row: 64 bytes + 16 of padding
 
 // The end of a tiled product.  D[n][m] of a 32 x 32 tile: a lane holds column m = lane % 32 and rows
-// n = 8 * (e / 4) + 4 * (lane / 32) + e % 4, so its values lie in 32 different rows of `out`.  They go
-// through LDS (`mine`: 32 x (32 WT + 4) floats of this wave's own), 32 rows of x at a time, and leave as
-// whole rows: 4 WT lanes write the 32 WT columns of a row, eight columns (16 bytes of bfloat16) a lane.
-// n_wave, m_wave: where the wave's WT x WT tiles begin; `slice` the K split (its own copy of `out`).
+// n = 8 * (e / 4) + 4 * (lane / 32) + e % 4, four consecutive n at a time.  Lanes l and l + 32 hold the two
+// halves of eight consecutive n of the same m, for e / 4 = 0, 1 (and 2, 3): one exchange between the upper
+// and the lower half of the wave (v_permlane32_swap) per value leaves eight consecutive n in one lane,
+// which it writes as one piece (16 bytes of bfloat16) straight from its registers.  A row of `out` gets
+// 32 bytes from each such store and the next ones fill the line; nothing goes through LDS and nothing
+// is waited for.  n_wave, m_wave: where the wave's WT x WT tiles begin; `slice` the K split (its own
+// copy of `out`).
+__device__ __forceinline__ void swap_halves(float& upper_of_this, float& lower_of_that) {
+  // lanes 32..63 of the first change places with lanes 0..31 of the second
+  const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(upper_of_this), __float_as_uint(lower_of_that), false, false);
+  upper_of_this = __uint_as_float(both[0]);
+  lower_of_that = __uint_as_float(both[1]);
+}
+
 template <int WT, typename TO, bool GATED>
-__device__ __forceinline__ void store_tiles(const f32x16 (&acc)[WT][WT], float* mine, TO* __restrict__ out,
+__device__ __forceinline__ void store_tiles(f32x16 (&acc)[WT][WT], TO* __restrict__ out,
                                             const void* __restrict__ bias, int bias_is_float, int slice, int M, int N,
                                             int n_wave, int m_wave, int lane) {
-  constexpr int ROW = 32 * WT + 4;           // floats of a transposed row, padded
-  constexpr int LANES_A_ROW = 4 * WT, ROWS_A_PASS = 64 / LANES_A_ROW;
   const int r32 = lane & 31, half = lane >> 5;
-  const int piece = lane % LANES_A_ROW, row_in_pass = lane / LANES_A_ROW;
-  const int n_piece = n_wave + piece * 8;
   const bool with_bias = bias && slice == 0;
-  float bias_here[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e)
-    bias_here[e] = with_bias && n_piece + e < N ? load_as_float(bias, bias_is_float, n_piece + e) : 0.f;
 #pragma unroll
   for (int j = 0; j < WT; ++j) {
+    const int m = m_wave + j * 32 + r32;
 #pragma unroll
-    for (int i = 0; i < WT; ++i)
+    for (int i = 0; i < WT; ++i) {
 #pragma unroll
-      for (int quad = 0; quad < 4; ++quad)
-        *(f32x4*)(mine + (size_t)r32 * ROW + i * 32 + quad * 8 + half * 4) =
-            (f32x4){acc[i][j][quad * 4], acc[i][j][quad * 4 + 1], acc[i][j][quad * 4 + 2], acc[i][j][quad * 4 + 3]};
-    // (a wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order)
+      for (int pair = 0; pair < 2; ++pair) {
+        float value[8];
 #pragma unroll
-    for (int pass = 0; pass < 32 / ROWS_A_PASS; ++pass) {
-      const int row = pass * ROWS_A_PASS + row_in_pass;
-      const int m = m_wave + j * 32 + row;
-      const f32x4 lo = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8);
-      const f32x4 hi = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8 + 4);
-      float value[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) value[e] += bias_here[e];
-      if (m >= M) continue;
-      if (GATED) {
-        TO* dst = out + (size_t)m * (N / 2) + n_piece / 2;
-        float gated[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) gated[e] = value[2 * e] / (1.f + expf(-value[2 * e])) * value[2 * e + 1];
-        if (n_piece + 8 <= N && sizeof(TO) == 2 && (N / 2) % 4 == 0) {
-          bf16_t packed[4] = {(bf16_t)gated[0], (bf16_t)gated[1], (bf16_t)gated[2], (bf16_t)gated[3]};
-          *(uint2*)dst = *(const uint2*)packed;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n_piece + 2 * e + 1 < N) dst[e] = from_float<TO>(gated[e]);
+        for (int e = 0; e < 4; ++e) {
+          float first = acc[i][j][pair * 8 + e], second = acc[i][j][pair * 8 + 4 + e];
+          swap_halves(first, second);
+          value[e] = first;
+          value[4 + e] = second;
         }
-      } else {
-        TO* dst = out + ((size_t)slice * M + m) * N + n_piece;
-        if (n_piece + 8 <= N && N % 8 == 0) {
-          if (sizeof(TO) == 2) {
-            bf16_t packed[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) packed[e] = (bf16_t)value[e];
-            *(uint4*)dst = *(const uint4*)packed;
-          } else {
-            *(f32x4*)dst = (f32x4){value[0], value[1], value[2], value[3]};
-            *(f32x4*)((float*)dst + 4) = (f32x4){value[4], value[5], value[6], value[7]};
-          }
-        } else {
+        const int n_piece = n_wave + i * 32 + pair * 16 + half * 8;
+        if (with_bias) {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (n_piece + e < N) dst[e] = from_float<TO>(value[e]);
+            if (n_piece + e < N) value[e] += load_as_float(bias, bias_is_float, n_piece + e);
+        }
+        if (m >= M) continue;
+        if (GATED) {
+          TO* dst = out + (size_t)m * (N / 2) + n_piece / 2;
+          float gated[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            // a bfloat16 result takes the hardware's 2^x and 1/x (a tile has 128 of these a lane; the
+            // library routines are some forty instructions each)
+            const float gate = value[2 * e], up = value[2 * e + 1];
+            gated[e] = sizeof(TO) == 2 ? gate * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(gate * -1.44269504088896f)) * up
+                                       : gate / (1.f + expf(-gate)) * up;
+          }
+          if (n_piece + 8 <= N && sizeof(TO) == 2 && (N / 2) % 4 == 0) {
+            bf16_t packed[4] = {(bf16_t)gated[0], (bf16_t)gated[1], (bf16_t)gated[2], (bf16_t)gated[3]};
+            *(uint2*)dst = *(const uint2*)packed;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n_piece + 2 * e + 1 < N) dst[e] = from_float<TO>(gated[e]);
+          }
+        } else {
+          TO* dst = out + ((size_t)slice * M + m) * N + n_piece;
+          if (n_piece + 8 <= N && N % 8 == 0) {
+            if (sizeof(TO) == 2) {
+              bf16_t packed[8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) packed[e] = (bf16_t)value[e];
+              *(uint4*)dst = *(const uint4*)packed;
+            } else {
+              *(f32x4*)dst = (f32x4){value[0], value[1], value[2], value[3]};
+              *(f32x4*)((float*)dst + 4) = (f32x4){value[4], value[5], value[6], value[7]};
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (n_piece + e < N) dst[e] = from_float<TO>(value[e]);
+          }
         }
       }
     }
   }
+}
+
+// Which tile a workgroup takes.  The chip hands workgroups to its eight chiplets (XCDs) in turn,
+// workgroup i to chiplet i % 8, and every chiplet has an L2 of its own: tiles dealt out in launch
+// order would make every chiplet read all of both operands.  So chiplet c takes a contiguous run
+// of the tiles instead, counted through bands of eight tile rows of x, down the band first, then
+// along the weight rows: what runs on a chiplet at one time is a few columns of one band, whose
+// operand rows it fetches once and shares through its L2.
+#define CHIPLETS 8
+#define BAND 8
+__device__ __forceinline__ void tile_of_workgroup(int index, int tiles_n, int tiles_m, int& tile_n, int& tile_m) {
+  const int tiles = tiles_n * tiles_m;
+  const int chiplet = index % CHIPLETS, turn = index / CHIPLETS;
+  const int place = chiplet * (tiles / CHIPLETS) + min(chiplet, tiles % CHIPLETS) + turn;
+  const int band = place / (BAND * tiles_n), within = place % (BAND * tiles_n);
+  const int rows = min(BAND, tiles_m - band * BAND);
+  tile_m = band * BAND + within % rows;
+  tile_n = within / rows;
 }
 
 template <int WT, typename TO, bool GATED>
@@ -435,7 +466,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   auto staged_x = [&](int buffer) { return staged + (size_t)(buffer * 2 + 1) * TILE * TILE_STRIDE; };
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wave_n = wave & 1, wave_m = wave >> 1;
-  const int n0 = blockIdx.x * TILE, m0 = blockIdx.y * TILE;
+  int tile_n, tile_m;
+  tile_of_workgroup(blockIdx.x, (N + TILE - 1) / TILE, (M + TILE - 1) / TILE, tile_n, tile_m);
+  const int n0 = tile_n * TILE, m0 = tile_m * TILE;
   const int k_first = blockIdx.z * k_split;
   const int r32 = lane & 31, half = lane >> 5;
 
@@ -501,9 +534,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     if (step + 1 < steps) stage(buffer ^ 1);  // read last in step - 1: everyone has passed this step's barrier since
   }
 
-  __syncthreads();  // every wave has read the last stage: LDS is free for the way out
-  store_tiles<WT, TO, GATED>(acc, (float*)staged + (size_t)wave * 32 * (32 * WT + 4), out, bias, bias_is_float,
-                             blockIdx.z, M, N, n0 + wave_n * 32 * WT, m0 + wave_m * 32 * WT, lane);
+  store_tiles<WT, TO, GATED>(acc, out, bias, bias_is_float, blockIdx.z, M, N, n0 + wave_n * 32 * WT,
+                             m0 + wave_m * 32 * WT, lane);
 }
 
 template <int WT, typename TO, bool GATED>
@@ -511,8 +543,7 @@ static int launch_tiled(const void* x, const void* w, const void* bias, int bias
                         int K, int splits, hipStream_t stream) {
   constexpr int TILE = 64 * WT;
   const size_t stages = (size_t)4 * TILE * TILE_STRIDE * sizeof(bf16_t);
-  const size_t way_out = (size_t)4 * 32 * (32 * WT + 4) * sizeof(float);  // store_tiles' rows of the four waves
-  const size_t lds = stages > way_out ? stages : way_out;
+  const size_t lds = stages;
   if (lds > 64 * 1024) {
     static bool asked = false;
     if (!asked) {
@@ -522,49 +553,111 @@ static int launch_tiled(const void* x, const void* w, const void* bias, int bias
       asked = true;
     }
   }
-  hipLaunchKernelGGL((gemm_tiled_kernel<WT, TO, GATED>), dim3((N + TILE - 1) / TILE, (M + TILE - 1) / TILE, splits),
+  hipLaunchKernelGGL((gemm_tiled_kernel<WT, TO, GATED>), dim3(((N + TILE - 1) / TILE) * ((M + TILE - 1) / TILE), 1, splits),
                      dim3(256), lds, stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K,
                      K / splits);
   return LAUNCH_STATUS();
 }
 
 // ---------------------------------------------------------------------------- many rows, wide tiles
-// gemm_wide: the tiled product with a 256 x 256 tile, steps of 64 over K, and both operands brought
-// from global memory straight into LDS (global_load_lds_dwordx4: a wave's 64 lanes fill 1 KB of LDS
-// in lane order, no registers in between), two stages: the next step's 64 KB are under way while
-// the current step is multiplied.  A staged row is 128 bytes = 8 pieces of 16; piece p of row r lies
-// in slot p ^ (r & 7), so that the eight lanes that read one piece of eight consecutive rows for an
-// MFMA operand hit eight different slots (no bank conflict), while the writes stay in lane order.
+// gemm_wide: the tiled product with a 256 x 256 tile and both operands brought from global memory
+// straight into LDS (global_load_lds_dwordx4: a wave's 64 lanes fill 1 KB of LDS in lane order, no
+// registers in between).  K goes in steps of 32 through four stages of 32 KB, so the loads of three
+// steps are under way while one is multiplied: a load takes longer to come back than a step's
+// products take, and with one wave a SIMD nobody else hides it.
+// A staged row is 64 bytes = 4 pieces of 16; piece p of row r lies in slot p ^ f(r), f mixing bits
+// 1 to 3 of r, so that the lanes that read one piece of consecutive rows for an MFMA operand hit
+// different banks, while the writes stay in lane order.
 // Each of the four waves (2 x 2) owns 4 x 4 tiles of v_mfma_f32_32x32x16_bf16: 256 accumulators.
+// The reads of LDS are written as instructions, with their waits: left to the compiler, every read
+// of LDS waits for all loads into LDS that are under way, whichever stage they fill.
+// One barrier a step, between its two halves: after it the next step's stage has landed for all
+// waves, and all waves have read the previous one, which the step after next may be written over.
 #define WIDE_TILE 256
-#define WIDE_K 64
+#define WIDE_K 32
+#define WIDE_STAGES 4
+#define WIDE_OPERAND_BYTES (WIDE_TILE * WIDE_K * 2)     // one staged operand: 16 KB
+#define WIDE_STAGE_BYTES (2 * WIDE_OPERAND_BYTES)        // w, then x
 
-__device__ __forceinline__ void wide_stage(const bf16_t* __restrict__ from, int rows_total, int row0, int ld, int k0,
-                                           bf16_t* staged, int wave, int lane) {
-  // 256 rows x 8 pieces = 2048 pieces of 16 bytes; wave w, instruction i fills pieces (w * 8 + i) * 64 + lane
+__device__ __forceinline__ int wide_swizzle(int row) { return (((row >> 1) ^ (row >> 3)) & 1) | (((row >> 2) & 1) << 1); }
+
+// The wave's share of one operand's step: pieces (wave * 4 + i) * 64 + lane of 1024, four instructions.
+__device__ __forceinline__ void wide_stage(const bf16_t* const (&src)[4], int k_offset, bf16_t* staged_operand, int wave) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int piece = (wave * 8 + i) * 64 + lane;
-    const int row = piece >> 3, slot = piece & 7;
-    const int part = slot ^ (row & 7);
-    const bf16_t* src = from + (size_t)min(row0 + row, rows_total - 1) * ld + k0 + part * 8;
-    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
-                                     (void __attribute__((address_space(3)))*)(staged + (size_t)(wave * 8 + i) * 512),
+  for (int i = 0; i < 4; ++i)
+    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(src[i] + k_offset),
+                                     (void __attribute__((address_space(3)))*)(staged_operand + (size_t)(wave * 4 + i) * 512),
                                      16, 0, 0);
-  }
 }
+
+// Loads into LDS that may still be under way: `stages` of them (8 instructions each), no more.
+__device__ __forceinline__ void wide_wait_loads(int stages) {
+  if (stages >= 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else if (stages == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// One 16-byte read of LDS for an MFMA operand: row tile I of the wave's four (32 rows = 2048 bytes
+// apart) at `at`.  The eight reads of a half step (w and x tiles in turn) are dealt out between its
+// products rather than put in front of them: a read that finds LDS busy holds up the wave, which
+// is the only one on its SIMD, and should do so while a product runs.
+template <int I>
+__device__ __forceinline__ void wide_read(bf16x8& operand, unsigned at) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(operand) : "v"(at), "n"(I * 2048) : "memory");
+}
+// The reads come back in the order they were asked for.  The operands pass through the statement
+// so that nothing that uses them is moved in front of it.
+#define WIDE_ARRIVED(a, b)                                                                                     \
+  asm volatile("s_waitcnt lgkmcnt(0)"                                                                          \
+               : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) \
+               :: "memory")
+// Two products of the current half step (tiles 2 P and 2 P + 1 of the sixteen, w tile = P / 2),
+// then one read for the half step after it.
+#define WIDE_PAIR(P, a_now, b_now, a_then, b_then, at_w, at_x)                                                      \
+  acc[(P) / 2][((P) % 2) * 2] =                                                                                     \
+      __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_now[(P) / 2], b_now[((P) % 2) * 2], acc[(P) / 2][((P) % 2) * 2], 0, 0, 0); \
+  acc[(P) / 2][((P) % 2) * 2 + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                                        \
+      a_now[(P) / 2], b_now[((P) % 2) * 2 + 1], acc[(P) / 2][((P) % 2) * 2 + 1], 0, 0, 0);                           \
+  __builtin_amdgcn_sched_barrier(0);                                                                                \
+  if ((P) % 2 == 0) wide_read<(P) / 2>(a_then[(P) / 2], at_w);                                                      \
+  else wide_read<(P) / 2>(b_then[(P) / 2], at_x);                                                                   \
+  __builtin_amdgcn_sched_barrier(0)
 
 template <typename TO, bool GATED>
 __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                         const void* __restrict__ bias, int bias_is_float,
                                                         TO* __restrict__ out, int M, int N, int K, int k_split) {
-  extern __shared__ __attribute__((aligned(16))) bf16_t staged[];  // [2 stages][w, x][256 rows][64]
-  constexpr int OPERAND = WIDE_TILE * WIDE_K;  // elements of one staged operand
+  extern __shared__ __attribute__((aligned(16))) bf16_t staged[];  // [4 stages][w, x][256 rows][32]
+  constexpr int STAGE = WIDE_STAGE_BYTES / 2, OPERAND = WIDE_OPERAND_BYTES / 2;  // in elements
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int wave_n = wave & 1, wave_m = wave >> 1;
-  const int n0 = blockIdx.x * WIDE_TILE, m0 = blockIdx.y * WIDE_TILE;
+  int tile_n, tile_m;
+  tile_of_workgroup(blockIdx.x, (N + WIDE_TILE - 1) / WIDE_TILE, (M + WIDE_TILE - 1) / WIDE_TILE, tile_n, tile_m);
+  const int n0 = tile_n * WIDE_TILE, m0 = tile_m * WIDE_TILE;
   const int k_first = blockIdx.z * k_split;
   const int r32 = lane & 31, half = lane >> 5;
+
+  // where this lane's pieces of a step come from: piece -> (row, slot), the slot holds part slot ^ f(row)
+  const bf16_t* w_src[4];
+  const bf16_t* x_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int piece = (wave * 4 + i) * 64 + lane;
+    const int row = piece >> 2, part = (piece & 3) ^ wide_swizzle(row);
+    w_src[i] = w + (size_t)min(n0 + row, N - 1) * K + k_first + part * 8;
+    x_src[i] = x + (size_t)min(m0 + row, M - 1) * K + k_first + part * 8;
+  }
+  auto load_stage = [&](int step) {
+    bf16_t* to = staged + (size_t)(step % WIDE_STAGES) * STAGE;
+    wide_stage(w_src, step * WIDE_K, to, wave);
+    wide_stage(x_src, step * WIDE_K, to + OPERAND, wave);
+  };
+  // where this lane reads its operands: rows r32 + 32 i of the wave's 128, part 2 * kk + half
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) bf16_t*)staged;
+  const int swizzle = wide_swizzle(r32);
+  const unsigned row_w = lds_base + (unsigned)(wave_n * 128 + r32) * (WIDE_K * 2);
+  const unsigned row_x = lds_base + WIDE_OPERAND_BYTES + (unsigned)(wave_m * 128 + r32) * (WIDE_K * 2);
+  const unsigned slot0 = (unsigned)((half ^ swizzle) * 16), slot1 = (unsigned)(((2 + half) ^ swizzle) * 16);
 
   f32x16 acc[4][4];  // [tile of weight rows][tile of x rows]
 #pragma unroll
@@ -575,55 +668,78 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   const int steps = k_split / WIDE_K;
-  wide_stage(w, N, n0, K, k_first, staged, wave, lane);
-  wide_stage(x, M, m0, K, k_first, staged + OPERAND, wave, lane);
-  for (int step = 0; step < steps; ++step) {
-    bf16_t* now = staged + (size_t)(step & 1) * 2 * OPERAND;
-    if (step + 1 < steps) {
-      bf16_t* next = staged + (size_t)((step + 1) & 1) * 2 * OPERAND;
-      wide_stage(w, N, n0, K, k_first + (step + 1) * WIDE_K, next, wave, lane);
-      wide_stage(x, M, m0, K, k_first + (step + 1) * WIDE_K, next + OPERAND, wave, lane);
-      __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): this step's pieces have landed, the next step's 16 may be out
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    }
-    __syncthreads();
-    const bf16_t* from_w = now + (size_t)(wave_n * 128 + r32) * WIDE_K;
-    const bf16_t* from_x = now + OPERAND + (size_t)(wave_m * 128 + r32) * WIDE_K;
-    // this lane's piece of a row in sub-step kk: part kk * 2 + half, in slot part ^ (row & 7); rows r32 + 32 i
-    // keep r32 & 7.  The operands of sub-step kk + 1 are read from LDS while sub-step kk is multiplied.
-    bf16x8 a[2][4], b[2][4];
-    auto read_operands = [&](int kk, bf16x8 (&a_now)[4], bf16x8 (&b_now)[4]) {
-      const int slot = ((kk * 2 + half) ^ (r32 & 7)) * 8;
+  const int last = steps - 1;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        a_now[i] = *(const bf16x8*)(from_w + (size_t)i * 32 * WIDE_K + slot);
-        b_now[i] = *(const bf16x8*)(from_x + (size_t)i * 32 * WIDE_K + slot);
-      }
-    };
-    read_operands(0, a[0], b[0]);
-#pragma unroll
-    for (int kk = 0; kk < WIDE_K / 16; ++kk) {
-      if (kk + 1 < WIDE_K / 16) read_operands(kk + 1, a[(kk + 1) & 1], b[(kk + 1) & 1]);
-      __builtin_amdgcn_sched_barrier(0);  // the reads stay in front of this sub-step's products: one wave a SIMD, nobody else hides their latency
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk & 1][i], b[kk & 1][j], acc[i][j], 0, 0, 0);
+  for (int step = 0; step < WIDE_STAGES - 1; ++step)
+    if (step < steps) load_stage(step);
+  wide_wait_loads(min(last, WIDE_STAGES - 2));  // stage 0 has landed
+  __builtin_amdgcn_s_barrier();
+  bf16x8 a0[4], b0[4], a1[4], b1[4];
+  wide_read<0>(a0[0], row_w + slot0);
+  wide_read<0>(b0[0], row_x + slot0);
+  wide_read<1>(a0[1], row_w + slot0);
+  wide_read<1>(b0[1], row_x + slot0);
+  wide_read<2>(a0[2], row_w + slot0);
+  wide_read<2>(b0[2], row_x + slot0);
+  wide_read<3>(a0[3], row_w + slot0);
+  wide_read<3>(b0[3], row_x + slot0);
+  // A step with the loads of the step three ahead dealt out between its products (LOADS), or, for
+  // the last three steps, without: two bodies, so that neither has a branch inside.
+  auto one_step = [&](int step, auto with_loads) {
+    constexpr bool LOADS = decltype(with_loads)::value;
+    const unsigned stage_now = (unsigned)(step % WIDE_STAGES) * WIDE_STAGE_BYTES;
+    const unsigned stage_next = (unsigned)((step + 1) % WIDE_STAGES) * WIDE_STAGE_BYTES;
+    // the stage read in step - 1 is free: every wave finished with it before the barrier of that step
+    bf16_t* to = staged + (size_t)((step + WIDE_STAGES - 1) % WIDE_STAGES) * STAGE;
+    const int k_then = (step + WIDE_STAGES - 1) * WIDE_K;
+    auto load_piece = [&](int i) {  // one of the wave's eight loads of the step three ahead
+      if (!LOADS) return;
+      const bf16_t* from = i < 4 ? w_src[i] : x_src[i - 4];
+      __builtin_amdgcn_global_load_lds(
+          (const void __attribute__((address_space(1)))*)(from + k_then),
+          (void __attribute__((address_space(3)))*)(to + (i < 4 ? 0 : OPERAND) + (size_t)(wave * 4 + i % 4) * 512), 16,
+          0, 0);
       __builtin_amdgcn_sched_barrier(0);
-    }
-    __syncthreads();  // everyone has read this stage: the step after next may be written over it
-  }
-
-  store_tiles<4, TO, GATED>(acc, (float*)staged + (size_t)wave * 32 * (32 * 4 + 4), out, bias, bias_is_float,
-                            blockIdx.z, M, N, n0 + wave_n * 128, m0 + wave_m * 128, lane);
+    };
+    const unsigned at_w1 = row_w + stage_now + slot1, at_x1 = row_x + stage_now + slot1;
+    WIDE_ARRIVED(a0, b0);
+    WIDE_PAIR(0, a0, b0, a1, b1, at_w1, at_x1); load_piece(0);
+    WIDE_PAIR(1, a0, b0, a1, b1, at_w1, at_x1); load_piece(1);
+    WIDE_PAIR(2, a0, b0, a1, b1, at_w1, at_x1); load_piece(2);
+    WIDE_PAIR(3, a0, b0, a1, b1, at_w1, at_x1); load_piece(3);
+    WIDE_PAIR(4, a0, b0, a1, b1, at_w1, at_x1); load_piece(4);
+    WIDE_PAIR(5, a0, b0, a1, b1, at_w1, at_x1); load_piece(5);
+    WIDE_PAIR(6, a0, b0, a1, b1, at_w1, at_x1); load_piece(6);
+    WIDE_PAIR(7, a0, b0, a1, b1, at_w1, at_x1); load_piece(7);
+    WIDE_ARRIVED(a1, b1);  // and this wave no longer reads the current stage
+    // stages up to min(step + 3, last) are on their way; step + 1 must have landed
+    if (LOADS) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else wide_wait_loads(last - (step + 1));
+    __builtin_amdgcn_s_barrier();
+    const unsigned at_w0 = row_w + stage_next + slot0, at_x0 = row_x + stage_next + slot0;
+    WIDE_PAIR(0, a1, b1, a0, b0, at_w0, at_x0);
+    WIDE_PAIR(1, a1, b1, a0, b0, at_w0, at_x0);
+    WIDE_PAIR(2, a1, b1, a0, b0, at_w0, at_x0);
+    WIDE_PAIR(3, a1, b1, a0, b0, at_w0, at_x0);
+    WIDE_PAIR(4, a1, b1, a0, b0, at_w0, at_x0);
+    WIDE_PAIR(5, a1, b1, a0, b0, at_w0, at_x0);
+    WIDE_PAIR(6, a1, b1, a0, b0, at_w0, at_x0);
+    WIDE_PAIR(7, a1, b1, a0, b0, at_w0, at_x0);
+  };
+  // (after the last step the reads "for the next step" fetch a stage that holds nothing new: they
+  // stay inside LDS and nobody uses them)
+  int step = 0;
+  for (; step + WIDE_STAGES - 1 < steps; ++step) one_step(step, std::true_type{});
+  for (; step < steps; ++step) one_step(step, std::false_type{});
+  WIDE_ARRIVED(a0, b0);
+  store_tiles<4, TO, GATED>(acc, out, bias, bias_is_float, blockIdx.z, M, N, n0 + wave_n * 128, m0 + wave_m * 128,
+                            lane);
 }
 
 template <typename TO, bool GATED>
 static int launch_wide(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
                        int K, int splits, hipStream_t stream) {
-  const size_t lds = (size_t)2 * 2 * WIDE_TILE * WIDE_K * sizeof(bf16_t);  // 128 KB
+  const size_t lds = (size_t)WIDE_STAGES * WIDE_STAGE_BYTES;  // 128 KB
   static bool asked = false;
   if (!asked) {
     if (hipFuncSetAttribute((const void*)gemm_wide_kernel<TO, GATED>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -632,12 +748,12 @@ static int launch_wide(const void* x, const void* w, const void* bias, int bias_
     asked = true;
   }
   hipLaunchKernelGGL((gemm_wide_kernel<TO, GATED>),
-                     dim3((N + WIDE_TILE - 1) / WIDE_TILE, (M + WIDE_TILE - 1) / WIDE_TILE, splits), dim3(256), lds,
+                     dim3(((N + WIDE_TILE - 1) / WIDE_TILE) * ((M + WIDE_TILE - 1) / WIDE_TILE), 1, splits), dim3(256), lds,
                      stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K, K / splits);
   return LAUNCH_STATUS();
 }
 
-// As llmserve_gemm_tiled, with K (and K / splits) a multiple of 64.
+// As llmserve_gemm_tiled, with K (and K / splits) a multiple of 32.
 extern "C" int llmserve_gemm_wide(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
                                   int out_is_float, int gated, int M, int N, int K, int splits, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
