@@ -353,84 +353,78 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define TILE_STRIDE (TILE_K + 8)  // bf16 elements per staged row: 64 bytes + 16 of padding
 
 // The end of a tiled product.  D[n][m] of a 32 x 32 tile: a lane holds column m = lane % 32 and rows
-// n = 8 * (e / 4) + 4 * (lane / 32) + e % 4, four consecutive n at a time.  Lanes l and l + 32 hold the two
-// halves of eight consecutive n of the same m, for e / 4 = 0, 1 (and 2, 3): one exchange between the upper
-// and the lower half of the wave (v_permlane32_swap) per value leaves eight consecutive n in one lane,
-// which it writes as one piece (16 bytes of bfloat16) straight from its registers.  A row of `out` gets
-// 32 bytes from each such store and the next ones fill the line; nothing goes through LDS and nothing
-// is waited for.  n_wave, m_wave: where the wave's WT x WT tiles begin; `slice` the K split (its own
-// copy of `out`).
-__device__ __forceinline__ void swap_halves(float& upper_of_this, float& lower_of_that) {
-  // lanes 32..63 of the first change places with lanes 0..31 of the second
-  const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(upper_of_this), __float_as_uint(lower_of_that), false, false);
-  upper_of_this = __uint_as_float(both[0]);
-  lower_of_that = __uint_as_float(both[1]);
-}
-
+// n = 8 * (e / 4) + 4 * (lane / 32) + e % 4, so its values lie in 32 different rows of `out`.  They go
+// through LDS (`mine`: 32 x (32 WT + 4) floats of this wave's own), 32 rows of x at a time, and leave as
+// whole rows: 4 WT lanes write the 32 WT columns of a row, eight columns (16 bytes of bfloat16) a lane.
+// n_wave, m_wave: where the wave's WT x WT tiles begin; `slice` the K split (its own copy of `out`).
 template <int WT, typename TO, bool GATED>
-__device__ __forceinline__ void store_tiles(f32x16 (&acc)[WT][WT], TO* __restrict__ out,
+__device__ __forceinline__ void store_tiles(const f32x16 (&acc)[WT][WT], float* mine, TO* __restrict__ out,
                                             const void* __restrict__ bias, int bias_is_float, int slice, int M, int N,
                                             int n_wave, int m_wave, int lane) {
+  constexpr int ROW = 32 * WT + 4;           // floats of a transposed row, padded
+  constexpr int LANES_A_ROW = 4 * WT, ROWS_A_PASS = 64 / LANES_A_ROW;
   const int r32 = lane & 31, half = lane >> 5;
+  const int piece = lane % LANES_A_ROW, row_in_pass = lane / LANES_A_ROW;
+  const int n_piece = n_wave + piece * 8;
   const bool with_bias = bias && slice == 0;
+  float bias_here[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    bias_here[e] = with_bias && n_piece + e < N ? load_as_float(bias, bias_is_float, n_piece + e) : 0.f;
 #pragma unroll
   for (int j = 0; j < WT; ++j) {
-    const int m = m_wave + j * 32 + r32;
 #pragma unroll
-    for (int i = 0; i < WT; ++i) {
+    for (int i = 0; i < WT; ++i)
 #pragma unroll
-      for (int pair = 0; pair < 2; ++pair) {
-        float value[8];
+      for (int quad = 0; quad < 4; ++quad)
+        *(f32x4*)(mine + (size_t)r32 * ROW + i * 32 + quad * 8 + half * 4) =
+            (f32x4){acc[i][j][quad * 4], acc[i][j][quad * 4 + 1], acc[i][j][quad * 4 + 2], acc[i][j][quad * 4 + 3]};
+    // (a wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order)
+#pragma unroll
+    for (int pass = 0; pass < 32 / ROWS_A_PASS; ++pass) {
+      const int row = pass * ROWS_A_PASS + row_in_pass;
+      const int m = m_wave + j * 32 + row;
+      const f32x4 lo = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8);
+      const f32x4 hi = *(const f32x4*)(mine + (size_t)row * ROW + piece * 8 + 4);
+      float value[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) value[e] += bias_here[e];
+      if (m >= M) continue;
+      if (GATED) {
+        TO* dst = out + (size_t)m * (N / 2) + n_piece / 2;
+        float gated[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float first = acc[i][j][pair * 8 + e], second = acc[i][j][pair * 8 + 4 + e];
-          swap_halves(first, second);
-          value[e] = first;
-          value[4 + e] = second;
+          // a bfloat16 result takes the hardware's 2^x and 1/x (a tile has 128 of these a lane; the
+          // library routines are some forty instructions each and took most of a tile's way out)
+          const float gate = value[2 * e], up = value[2 * e + 1];
+          gated[e] = sizeof(TO) == 2 ? gate * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(gate * -1.44269504088896f)) * up
+                                     : gate / (1.f + expf(-gate)) * up;
         }
-        const int n_piece = n_wave + i * 32 + pair * 16 + half * 8;
-        if (with_bias) {
+        if (n_piece + 8 <= N && sizeof(TO) == 2 && (N / 2) % 4 == 0) {
+          bf16_t packed[4] = {(bf16_t)gated[0], (bf16_t)gated[1], (bf16_t)gated[2], (bf16_t)gated[3]};
+          *(uint2*)dst = *(const uint2*)packed;
+        } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n_piece + e < N) value[e] += load_as_float(bias, bias_is_float, n_piece + e);
+          for (int e = 0; e < 4; ++e)
+            if (n_piece + 2 * e + 1 < N) dst[e] = from_float<TO>(gated[e]);
         }
-        if (m >= M) continue;
-        if (GATED) {
-          TO* dst = out + (size_t)m * (N / 2) + n_piece / 2;
-          float gated[4];
+      } else {
+        TO* dst = out + ((size_t)slice * M + m) * N + n_piece;
+        if (n_piece + 8 <= N && N % 8 == 0) {
+          if (sizeof(TO) == 2) {
+            bf16_t packed[8];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            // a bfloat16 result takes the hardware's 2^x and 1/x (a tile has 128 of these a lane; the
-            // library routines are some forty instructions each)
-            const float gate = value[2 * e], up = value[2 * e + 1];
-            gated[e] = sizeof(TO) == 2 ? gate * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(gate * -1.44269504088896f)) * up
-                                       : gate / (1.f + expf(-gate)) * up;
-          }
-          if (n_piece + 8 <= N && sizeof(TO) == 2 && (N / 2) % 4 == 0) {
-            bf16_t packed[4] = {(bf16_t)gated[0], (bf16_t)gated[1], (bf16_t)gated[2], (bf16_t)gated[3]};
-            *(uint2*)dst = *(const uint2*)packed;
+            for (int e = 0; e < 8; ++e) packed[e] = (bf16_t)value[e];
+            *(uint4*)dst = *(const uint4*)packed;
           } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n_piece + 2 * e + 1 < N) dst[e] = from_float<TO>(gated[e]);
+            *(f32x4*)dst = (f32x4){value[0], value[1], value[2], value[3]};
+            *(f32x4*)((float*)dst + 4) = (f32x4){value[4], value[5], value[6], value[7]};
           }
         } else {
-          TO* dst = out + ((size_t)slice * M + m) * N + n_piece;
-          if (n_piece + 8 <= N && N % 8 == 0) {
-            if (sizeof(TO) == 2) {
-              bf16_t packed[8];
 #pragma unroll
-              for (int e = 0; e < 8; ++e) packed[e] = (bf16_t)value[e];
-              *(uint4*)dst = *(const uint4*)packed;
-            } else {
-              *(f32x4*)dst = (f32x4){value[0], value[1], value[2], value[3]};
-              *(f32x4*)((float*)dst + 4) = (f32x4){value[4], value[5], value[6], value[7]};
-            }
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (n_piece + e < N) dst[e] = from_float<TO>(value[e]);
-          }
+          for (int e = 0; e < 8; ++e)
+            if (n_piece + e < N) dst[e] = from_float<TO>(value[e]);
         }
       }
     }
@@ -534,8 +528,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     if (step + 1 < steps) stage(buffer ^ 1);  // read last in step - 1: everyone has passed this step's barrier since
   }
 
-  store_tiles<WT, TO, GATED>(acc, out, bias, bias_is_float, blockIdx.z, M, N, n0 + wave_n * 32 * WT,
-                             m0 + wave_m * 32 * WT, lane);
+  __syncthreads();  // every wave has read the last stage: LDS is free for the way out
+  store_tiles<WT, TO, GATED>(acc, (float*)staged + (size_t)wave * 32 * (32 * WT + 4), out, bias, bias_is_float,
+                             blockIdx.z, M, N, n0 + wave_n * 32 * WT, m0 + wave_m * 32 * WT, lane);
 }
 
 template <int WT, typename TO, bool GATED>
@@ -543,7 +538,8 @@ static int launch_tiled(const void* x, const void* w, const void* bias, int bias
                         int K, int splits, hipStream_t stream) {
   constexpr int TILE = 64 * WT;
   const size_t stages = (size_t)4 * TILE * TILE_STRIDE * sizeof(bf16_t);
-  const size_t lds = stages;
+  const size_t way_out = (size_t)4 * 32 * (32 * WT + 4) * sizeof(float);  // store_tiles' rows of the four waves
+  const size_t lds = stages > way_out ? stages : way_out;
   if (lds > 64 * 1024) {
     static bool asked = false;
     if (!asked) {
@@ -732,8 +728,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict
   for (; step + WIDE_STAGES - 1 < steps; ++step) one_step(step, std::true_type{});
   for (; step < steps; ++step) one_step(step, std::false_type{});
   WIDE_ARRIVED(a0, b0);
-  store_tiles<4, TO, GATED>(acc, out, bias, bias_is_float, blockIdx.z, M, N, n0 + wave_n * 128, m0 + wave_m * 128,
-                            lane);
+  __syncthreads();  // every wave has read the last stage: LDS is free for the way out
+  store_tiles<4, TO, GATED>(acc, (float*)staged + (size_t)wave * 32 * (32 * 4 + 4), out, bias, bias_is_float,
+                            blockIdx.z, M, N, n0 + wave_n * 128, m0 + wave_m * 128, lane);
 }
 
 template <typename TO, bool GATED>

@@ -110,9 +110,17 @@ class GatedLinearWeights:
 class HipKernels:
     def __init__(
         self, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0", *, library_products: bool = True,
-        shared_portions: str = "auto",
+        shared_portions: str = "auto", wide_products: str = "never",
     ) -> None:
-        """`library_products=False` keeps every product on the hand-written kernels.  `shared_portions`:
+        """`library_products=False` keeps every product on the hand-written kernels.  `wide_products`:
+        which products of more than 64 rows leave the library for the hand-written 256 x 256 tile
+        although `library_products` is set: "never" (the default: inside a step neither is ahead, see
+        below), "partial" (float32 results that may stay partial sums over K, the down projection),
+        "gated" (those and gate/up with its fused SiLU * up).  Alone, the down projection of 2,048 rows
+        at the 1.5B sizes takes 60 us against the library's 67, but its five partial sums cost the
+        norm that adds them more than that; gate/up takes 150 us against the library's 120 + 18 for
+        SiLU * up.
+        `shared_portions`:
         whether prompt portions at head size 128 go to the attention kernel whose waves share K and V
         through LDS: "auto" (when the step's walks, taken together, are long beside the longest), "always", "never"."""
         if dtype not in (torch.bfloat16, torch.float32):
@@ -123,6 +131,7 @@ class HipKernels:
         self.device = torch.device(device)
         self.library_products = library_products
         self.shared_portions = shared_portions
+        self.wide_products = wide_products
         name = torch.cuda.get_device_properties(self.device).gcnArchName
         if not name.startswith("gfx950"):
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
@@ -297,6 +306,12 @@ class HipKernels:
                 best = splits
         return best
 
+    def _wide_applies(self, rows: int, out_features: int, in_features: int, splits: int) -> bool:
+        """Whether the tiled product would run its 256 x 256 tile: enough tiles for the chip, and
+        K a multiple of 32 of at least three steps."""
+        tiles = -(-rows // 256) * -(-out_features // 256) * splits
+        return tiles >= 200 and in_features % (32 * splits) == 0 and in_features // splits >= 96
+
     @staticmethod
     def _tiled_splits(rows: int, out_features: int, in_features: int) -> int:
         """Into how many parts of K the tiled product is cut when its float32 result may stay in
@@ -332,6 +347,16 @@ class HipKernels:
             # a long K over few weight rows (the down projection): cut over K into partial sums, the
             # hand-written kernel is ahead of the library (16 against 25 us at 64 rows of the 1.5B sizes)
             streaming = "medium"
+        if (
+            streaming is None
+            and partial
+            and out_dtype == torch.float32
+            and self.wide_products != "never"
+            and self._library(x, weights)
+            and rows > 64
+            and self._wide_applies(rows, weights.out_features, inner, self._tiled_splits(rows, weights.out_features, inner))
+        ):
+            streaming = "tiled"
         if streaming is None and self._library(x, weights):
             if (out_dtype or self.dtype) == torch.float32:  # float32 straight from the accumulators
                 out = torch.mm(x, weights.weight.t(), out_dtype=torch.float32)
@@ -373,6 +398,14 @@ class HipKernels:
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
         out = self._empty((x.shape[0], weights.width), self.dtype)
         streaming = self._streaming(x, weights.both)
+        if (
+            streaming is None
+            and self.wide_products == "gated"
+            and self._library(x, weights.both)
+            and x.shape[0] > 64
+            and self._wide_applies(x.shape[0], 2 * weights.width, x.shape[1], 1)
+        ):
+            streaming = "tiled"
         if streaming is not None:
             if streaming == "tiled":
                 status = self._gemm_bf16.llmserve_gemm_tiled(

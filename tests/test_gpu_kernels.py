@@ -102,12 +102,12 @@ def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
 @pytest.mark.parametrize("rows,inner,outer", [(17, 128, 64), (32, 256, 100), (33, 1536, 272), (64, 1280, 130), (64, 8960, 48),
                                               (40, 96, 77), (64, 160, 2048), (100, 256, 40), (65, 32, 128), (130, 1536, 272),
                                               (300, 96, 1000), (2048, 512, 384), (129, 129, 50), (2000, 64, 6500), (2048, 2048, 1500),
-                                              (1100, 2048, 700)])
+                                              (1100, 2048, 700), (2048, 416, 6400), (1000, 160, 12900), (2040, 96, 6401)])
 def test_products_without_the_library(own_kernels, rows, inner, outer):
     """17 to 64 rows: the kernel that shares x through LDS (K a multiple of 128), else the
     weight-streaming one with several tiles of x; more rows: the tiled one (K a multiple of 32; its
-    256 x 256 tiles where there are 200 of them, K cut into partial sums where a float32 result
-    may stay in parts); else the generic one."""
+    256 x 256 tiles where there are 200 of them, with K steps that are and are not a multiple of its
+    four stages, K cut into partial sums where a float32 result may stay in parts); else the generic one."""
     k, dtype = own_kernels, torch.bfloat16
     x, w, b = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer)
     expected = rounded(x, dtype) @ rounded(w, dtype).T + rounded(b, dtype)
