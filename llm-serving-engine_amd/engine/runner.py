@@ -177,6 +177,7 @@ class ModelRunner:
         self.cells = self.cache.cells()
         self.vocab_size = loaded.spec.vocab_size
         self.use_graphs = self.device.type == "cuda" if use_graphs is None else use_graphs
+        self.use_graphs = self.use_graphs and self.model.replayable  # a part that looks at values on the host is not replayed
         self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
         # What `prepare_decode` has done for the step to come: each request's reservation of one
         # token, and, where decode steps replay a graph, the step's index arrays already packed.

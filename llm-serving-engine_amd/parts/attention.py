@@ -63,6 +63,9 @@ class Attention(Mixer):
             found["v_proj.bias"] = TensorSpec((kv_size,), role="bias")
         if spec.out_bias:
             found["o_proj.bias"] = TensorSpec((spec.hidden_size,), role="bias")
+        # a position encoding with tensors of its own (a learned table) keeps them below "position."
+        for name, tensor in POSITIONS.tensors(spec.position).items():
+            found["position." + name] = tensor
         return found
 
     @classmethod
@@ -78,7 +81,9 @@ class Attention(Mixer):
         self.out = kernels.prepare_linear(
             [tensors["o_proj.weight"]], [tensors["o_proj.bias"]] if spec.out_bias else None
         )
-        self.position = POSITIONS.build(spec.position, {}, kernels)
+        own = {name[len("position."):]: tensor for name, tensor in tensors.items() if name.startswith("position.")}
+        self.position = POSITIONS.build(spec.position, own, kernels)
+        self.replayable = self.position.replayable
 
     def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
         qkv = self.kernels.linear(x, self.qkv)

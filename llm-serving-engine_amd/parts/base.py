@@ -57,6 +57,10 @@ class Part:
     """Base of norms, position encodings, mixers, feed-forwards and blocks."""
 
     kind: ClassVar[str] = ""
+    # Whether a step through the part is the same sequence of kernel launches whatever the data:
+    # then a step of single tokens may be captured into a graph once and replayed.  A part that
+    # looks at values on the host (routing that gathers rows, a loop over a request's tokens) says False.
+    replayable: ClassVar[bool] = True
 
     @classmethod
     def tensors(cls, spec: Any) -> dict[str, TensorSpec]:

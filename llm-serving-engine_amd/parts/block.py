@@ -67,6 +67,7 @@ class PreNormBlock(Block):
             for name, registry, member in self._members(spec)
         ]
         self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward = built
+        self.replayable = all(part.replayable for part in built)
 
     def forward(self, hidden, delta, batch, cell) -> torch.Tensor:
         normed = self.mixer_norm.forward(hidden, delta)

@@ -82,6 +82,7 @@ class DecoderModel:
         self.final_norm = NORMS.build(spec.final_norm, under(tensors, spec.final_norm_name), kernels)
         head = self.embedding if spec.tie_embeddings else tensors[spec.head_name]
         self.head = kernels.prepare_linear([head], None)
+        self.replayable = all(layer.replayable for layer in self.layers) and self.final_norm.replayable
 
     def _run_layers(self, batch, cells: list):
         hidden = self.kernels.embedding(self.embedding, batch.token_ids)

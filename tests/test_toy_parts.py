@@ -31,6 +31,9 @@ def test_toy_architecture_steps_like_its_plain_forward(toy_folder):
     # one group), the last run owns nothing and reads run 1's pages
     assert [type(cell.need) for cell in runner.cells] == [FixedState, PagedKeyValue, PagedKeyValue, FixedState, PagedKeyValue]
     assert len(cache.states) == 2 and len(cache.groups) == 1 and cache.groups[0].cells == [1, 2]
+    # the routed feed-forward and the decaying mixer look at values on the host: no step of this model is replayed from a graph
+    assert not runner.model.replayable and not runner.use_graphs
+    assert "layers.0.mlp.router.weight" in loaded.tensors and "layers.2.mixer.position.table" in loaded.tensors
     assert runner.cells[4].keys.data_ptr() == runner.cells[1].keys.data_ptr() and not runner.cells[4].writable
 
     prompts = {name: random_tokens(n, toy.TOY.vocab_size, seed=n) for name, n in (("a", 37), ("b", 9), ("c", 22))}

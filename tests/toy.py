@@ -3,6 +3,8 @@ architectures are added by registering them, without a change to the framework's
 
 - a mixer with state of its own (a decaying sum per request, a fixed-size state slot),
 - beside attention layers, chosen layer by layer,
+- a feed-forward with routing (a few small experts, the best two per token) in one layer,
+- a position encoding with a tensor of its own (a learned table added to queries and keys) in another,
 - a run order that names one layer twice, and a run that reads another run's cache.
 
 It is never a model of anyone's: it exists to exercise the interfaces."""
@@ -19,8 +21,8 @@ import torch
 
 from llmserve_amd.config.model import ArchitectureConfig, KeyReader
 from llmserve_amd.parts import (
-    MIXERS, AttentionSpec, FixedState, GatedMLPSpec, LayerDefinition, LayerRun, Mixer, ModelSpec, NoPositionSpec,
-    PreNormBlockSpec, RMSNormSpec, RotarySpec, TensorSpec,
+    FEED_FORWARDS, MIXERS, POSITIONS, AttentionSpec, FeedForward, FixedState, GatedMLPSpec, LayerDefinition, LayerRun,
+    Mixer, ModelSpec, NoPositionSpec, PositionEncoding, PreNormBlockSpec, RMSNormSpec, RotarySpec, TensorSpec,
 )
 from llmserve_amd.registry import register_architecture, unregister_architecture
 
@@ -36,6 +38,8 @@ class DecaySpec:
 class DecayMixer(Mixer):
     """state <- decay * state + x W_in;  out = state W_out, token after token in order.
     The state of a request lives in its slot of the cell, across steps."""
+
+    replayable = False  # a loop on the host over each request's tokens
 
     @classmethod
     def tensors(cls, spec: DecaySpec) -> dict[str, TensorSpec]:
@@ -69,6 +73,80 @@ class DecayMixer(Mixer):
 
 
 @dataclass(frozen=True)
+class RoutedSpec:
+    hidden_size: int
+    expert_size: int
+    experts: int
+    chosen: int
+    kind: str = "toy_routed"
+
+
+class RoutedFeedForward(FeedForward):
+    """Router logits in float32; the `chosen` best experts of a token, weighted by the softmax
+    over their logits alone; every expert a small gated MLP run through the kernel library on the
+    rows that chose it."""
+
+    replayable = False  # which rows go to which expert is looked up on the host
+
+    @classmethod
+    def tensors(cls, spec: RoutedSpec) -> dict[str, TensorSpec]:
+        found = {"router.weight": TensorSpec((spec.experts, spec.hidden_size))}
+        for expert in range(spec.experts):
+            found[f"experts.{expert}.gate_proj.weight"] = TensorSpec((spec.expert_size, spec.hidden_size))
+            found[f"experts.{expert}.up_proj.weight"] = TensorSpec((spec.expert_size, spec.hidden_size))
+            found[f"experts.{expert}.down_proj.weight"] = TensorSpec((spec.hidden_size, spec.expert_size))
+        return found
+
+    def __init__(self, spec: RoutedSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.router = tensors["router.weight"].float()
+        self.gate_up = [
+            kernels.prepare_gated_linear(tensors[f"experts.{e}.gate_proj.weight"], tensors[f"experts.{e}.up_proj.weight"])
+            for e in range(spec.experts)
+        ]
+        self.down = [kernels.prepare_linear([tensors[f"experts.{e}.down_proj.weight"]], None) for e in range(spec.experts)]
+
+    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        logits = x.float() @ self.router.T
+        best, which = torch.topk(logits, self.spec.chosen, dim=-1)
+        weights = torch.softmax(best, dim=-1)
+        out = torch.zeros(x.shape[0], self.spec.hidden_size, dtype=torch.float32, device=x.device)
+        for expert in range(self.spec.experts):
+            rows, place = torch.nonzero(which == expert, as_tuple=True)
+            if rows.numel() == 0:
+                continue
+            hidden = self.kernels.gated_linear(x[rows].contiguous(), self.gate_up[expert])
+            result = self.kernels.linear(hidden, self.down[expert], out_dtype=torch.float32)
+            out.index_add_(0, rows, result * weights[rows, place].unsqueeze(-1))
+        return out
+
+
+@dataclass(frozen=True)
+class LearnedPositionSpec:
+    head_dim: int
+    max_length: int
+    kind: str = "toy_learned"
+
+
+class LearnedPosition(PositionEncoding):
+    """Adds row `position` of a learned table to every query and key head; then stores."""
+
+    @classmethod
+    def tensors(cls, spec: LearnedPositionSpec) -> dict[str, TensorSpec]:
+        return {"table": TensorSpec((spec.max_length, spec.head_dim))}
+
+    def __init__(self, spec: LearnedPositionSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.table = tensors["table"]
+
+    def encode_and_store(self, qkv, layout, batch, cell) -> None:
+        rotated = layout.num_heads + layout.num_kv_heads
+        heads = qkv.view(qkv.shape[0], -1, layout.head_dim)
+        heads[:, :rotated] += self.table[batch.positions.long()].to(qkv.dtype).unsqueeze(1)
+        self.kernels.rotate_and_store(qkv, layout, batch, cell, None, "none")
+
+
+@dataclass(frozen=True)
 class ToyConfig(ArchitectureConfig):
     architecture: ClassVar[str] = "ToyStateForCausalLM"
     vocab_size: int = 0
@@ -80,6 +158,9 @@ class ToyConfig(ArchitectureConfig):
     ffn_size: int = 0
     eps: float = 0.0
     max_length: int = 0
+    experts: int = 0
+    experts_chosen: int = 0
+    expert_size: int = 0
 
     @classmethod
     def from_dict(cls, values: dict[str, Any]) -> "ToyConfig":
@@ -89,6 +170,8 @@ class ToyConfig(ArchitectureConfig):
             state_size=reader.integer("state_size"), decay=reader.number("decay"),
             num_heads=reader.integer("num_heads"), head_dim=reader.integer("head_dim"),
             ffn_size=reader.integer("ffn_size"), eps=reader.number("eps"), max_length=reader.integer("max_length"),
+            experts=reader.integer("experts"), experts_chosen=reader.integer("experts_chosen"),
+            expert_size=reader.integer("expert_size"),
         )
 
     @property
@@ -109,10 +192,11 @@ def toy_spec(config: ToyConfig) -> ModelSpec:
     )
     unrotated = AttentionSpec(
         config.hidden_size, config.num_heads, config.num_heads, config.head_dim, 1.0 / math.sqrt(config.head_dim),
-        NoPositionSpec(), qkv_bias=False,
+        LearnedPositionSpec(config.head_dim, config.max_length), qkv_bias=False,
     )
+    routed = RoutedSpec(config.hidden_size, config.expert_size, config.experts, config.experts_chosen)
     layers = (
-        LayerDefinition("layers.0.", PreNormBlockSpec(norm, decay, norm, ffn, mixer_name="mixer.")),
+        LayerDefinition("layers.0.", PreNormBlockSpec(norm, decay, norm, routed, mixer_name="mixer.")),
         LayerDefinition("layers.1.", PreNormBlockSpec(norm, attention, norm, ffn, mixer_name="mixer.")),
         LayerDefinition("layers.2.", PreNormBlockSpec(norm, unrotated, norm, ffn, mixer_name="mixer.")),
     )
@@ -125,16 +209,20 @@ def toy_spec(config: ToyConfig) -> ModelSpec:
 
 
 TOY = ToyConfig(vocab_size=97, hidden_size=48, state_size=20, decay=0.8, num_heads=3, head_dim=16, ffn_size=64,
-                eps=1e-5, max_length=256)
+                eps=1e-5, max_length=256, experts=5, experts_chosen=2, expert_size=24)
 
 
 def register_toy() -> None:
     MIXERS.register("toy_decay")(DecayMixer)
+    FEED_FORWARDS.register("toy_routed")(RoutedFeedForward)
+    POSITIONS.register("toy_learned")(LearnedPosition)
     register_architecture("ToyStateForCausalLM", ToyConfig, toy_spec)
 
 
 def unregister_toy() -> None:
     MIXERS.unregister("toy_decay")
+    FEED_FORWARDS.unregister("toy_routed")
+    POSITIONS.unregister("toy_learned")
     unregister_architecture("ToyStateForCausalLM")
 
 
@@ -162,6 +250,18 @@ def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
     def ffn(x, prefix):
         return plain.swiglu(x, w[prefix + "mlp.gate_proj.weight"], w[prefix + "mlp.up_proj.weight"], w[prefix + "mlp.down_proj.weight"])
 
+    def routed(x, prefix):
+        logits = x @ w[prefix + "mlp.router.weight"].T
+        out = torch.zeros_like(x)
+        for t in range(length):
+            order = sorted(range(config["experts"]), key=lambda e: (-logits[t, e].item(), e))[: config["experts_chosen"]]
+            weights = torch.softmax(logits[t, order], dim=0)
+            for weight, e in zip(weights, order):
+                name = f"{prefix}mlp.experts.{e}."
+                out[t] += weight * plain.swiglu(x[t : t + 1], w[name + "gate_proj.weight"], w[name + "up_proj.weight"],
+                                                w[name + "down_proj.weight"])[0]
+        return out
+
     def decay_layer(h, prefix):
         x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
         state = torch.zeros(config["state_size"], dtype=torch.float64)
@@ -170,7 +270,7 @@ def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
             state = config["decay"] * state + w[prefix + "mixer.in_proj.weight"] @ x[t]
             out.append(w[prefix + "mixer.out_proj.weight"] @ state)
         h = h + torch.stack(out)
-        return h + ffn(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
+        return h + routed(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
 
     def attention_layer(h, prefix, rotate, shared=None):
         x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
@@ -180,6 +280,9 @@ def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
         if rotate:
             angles = plain.rope_angles(dim, 100.0, torch.arange(length))
             q, k = plain.rope_half(q, angles), plain.rope_half(k, angles)
+        else:  # the learned table's row of each position, added to every query and key head
+            table = w[prefix + "mixer.position.table"][:length].unsqueeze(1)
+            q, k = q + table, k + table
         if shared is not None:
             k, v = shared  # the run reads the keys and values another run stored
         mixed = plain.causal_attention(q, k, v, 1.0 / math.sqrt(dim)).reshape(length, -1)
