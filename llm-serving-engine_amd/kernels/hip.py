@@ -140,6 +140,14 @@ class HipKernels:
         self._attention_generic = _declared(load_module("attention_generic"))
         self._gemm_bf16 = _declared(load_module("gemm_bf16")) if dtype == torch.bfloat16 else None
         self._pinned_stream: int | None = None
+        if self._gemm_bf16 is not None and library_products:
+            # The BLAS library sets itself up at its first product, which it cannot do while a stream is
+            # being captured; a step of 17 to 64 rows meets the library only inside a capture.
+            with torch.cuda.device(self.device):
+                one = torch.ones((32, 32), dtype=torch.bfloat16, device=self.device)
+                torch.nn.functional.linear(one, one, one[0])
+                torch.mm(one, one.t(), out_dtype=torch.float32)
+                torch.cuda.synchronize(self.device)
         self._attention_bf16: dict[int, ctypes.CDLL] = {}  # by head size, compiled when a model needs it
         self._sampling = None
 

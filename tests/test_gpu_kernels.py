@@ -440,3 +440,30 @@ def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
     want_v = torch.stack([rounded(p[2][-1], dtype) for p in per_request])
     torch.testing.assert_close(stored_k, want_k, **TOLERANCE[dtype])
     torch.testing.assert_close(stored_v, want_v, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("requests", [3, 12])
+def test_fused_decode_attention_over_long_contexts(kernels, requests):
+    """Single tokens against thousands of keys: the one-kernel decode step cuts the keys over several
+    workgroups and merges them.  Every request has one far key made to dominate two of its heads (the
+    value stored there must come out), at a place that differs from request to request, first and
+    last keys and the edges of the cuts among them; the other heads are compared with plain attention."""
+    dtype, heads, kv_heads, dim, page = torch.bfloat16, 12, 2, 128, 16
+    lengths = [4100, 2049, 3333] + [1500 + 37 * i for i in range(requests - 3)]
+    counts = [1] * len(lengths)
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=requests)
+    places = [0, 2048, 3332] + [(211 * i) % 1500 for i in range(requests - 3)]
+    for (q, k, v), far in zip(per_request, places):
+        k[far] = 3.0 * q[-1, ::6]  # kv head g takes the query of its first head: heads 0 and 6 find this key
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    slots = batch.groups[0].slot_mapping.cpu().long()
+    cell.keys[slots // page, :, slots % page] = float("nan")  # the step itself stores the newest key and value
+    cell.values[slots // page, :, :, slots % page] = float("nan")
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None, "none", 1.0, None).cpu().double()
+    for index, ((q, k, v), far) in enumerate(zip(per_request, places)):
+        full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), 1.0)[-1]
+        got = out[index].view(heads, dim)
+        torch.testing.assert_close(got, full, **TOLERANCE[dtype])
+        for head in (0, 6):
+            torch.testing.assert_close(got[head], rounded(v, dtype)[far, head // 6], atol=0.05, rtol=0.05)

@@ -219,3 +219,25 @@ def test_command_line_generates(model_folders, tmp_path):
     assert done.returncode == 0, done.stderr[-2000:]
     summary = json.loads(output.read_text())["summary"]
     assert summary["successful_requests"] == 6 and summary["throughput_tokens_per_s"] > 0
+
+
+def test_first_step_of_a_process_may_be_a_captured_one_of_many_rows(model_folders):
+    """A fresh process whose prompts are short: no step before the first decode step has more than 16
+    rows, so that step, captured into a graph, is the first to meet the BLAS library (which takes the
+    products of 17 to 64 rows inside a capture).  The library must be set up by then."""
+    script = f"""
+import sys
+sys.path.insert(0, {str(ROOT)!r})
+from llmserve_amd import CacheConfig, EngineCore, GenerationConfig, ModelRunner, SchedulerConfig
+from llmserve_amd.kernels import HipKernels
+from llmserve_amd.weights import load_model_folder
+loaded = load_model_folder({str(model_folders["B"])!r}, "bfloat16")
+runner = ModelRunner(loaded, HipKernels(loaded.dtype, "cuda:0"), CacheConfig(8, 256, 32))
+core = EngineCore(runner, SchedulerConfig(24, 64), prefill_chunk_size=16)
+produced = core.generate([[7 + i, 3] for i in range(20)], GenerationConfig(max_new_tokens=4))
+assert len(produced) == 20 and all(len(tokens) == 4 for tokens in produced), produced
+runner.close()
+print("ok")
+"""
+    done = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0 and done.stdout.strip().endswith("ok"), done.stderr[-2000:]
