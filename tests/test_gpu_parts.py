@@ -241,3 +241,48 @@ print("ok")
 """
     done = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0 and done.stdout.strip().endswith("ok"), done.stderr[-2000:]
+
+
+def test_everything_at_once_matches_the_plain_decoder(model_folders):
+    """Twelve requests through the engine on the GPU in float32 with all it has switched on (captured
+    decode steps, the next step prepared and queued ahead): greedy and sampled requests side by side,
+    some with stop tokens, late arrivals, and so few pages that requests give way and replay.  Every
+    request's tokens are the plain decoder's."""
+    from llmserve_amd.engine import RequestState
+    from llmserve_amd.kernels import HipKernels
+
+    config, page = CONFIGS["B"]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders["B"]), plain.read_weights(model_folders["B"])
+    lengths = [3, 30, 17, 1, 44, 9, 25, 2, 38, 12, 21, 5]
+    prompts = [random_tokens(n, config.vocab_size, seed=100 + n) for n in lengths]
+    settings = []
+    for index in range(len(prompts)):
+        sampled = index % 3 == 1
+        # stop tokens: a tenth of the vocabulary, so that some requests stop early
+        stops = tuple(range(index, config.vocab_size, 10)) if index % 4 == 0 else ()
+        settings.append(GenerationConfig(10 + index, 0.9 if sampled else 0.0, 0.85 if index % 2 else 1.0, seed=index, stop_token_ids=stops))
+    expected = [
+        plain.generate(weights, plain_config, p, s.max_new_tokens, s.temperature, s.top_p, s.seed, s.stop_token_ids)
+        for p, s in zip(prompts, settings)
+    ]
+    loaded = load_model_folder(model_folders["B"], "float32")
+    runner = ModelRunner(loaded, HipKernels(torch.float32), CacheConfig(page, 14, 6))  # 14 pages of 8: 112 tokens
+    core = EngineCore(runner, SchedulerConfig(5, 48), prefill_chunk_size=16)
+    requests = [RequestState(f"r{index}", prompt, s.max_new_tokens) for index, (prompt, s) in enumerate(zip(prompts, settings))]
+    waiting = list(zip(requests, settings))
+    for request, setting in waiting[:5]:
+        core.submit(request, setting)
+    waiting = waiting[5:]
+    turn = 0
+    while core.has_work or waiting:
+        if waiting and turn % 3 == 0:  # the others arrive one by one while the engine runs
+            core.submit(*waiting.pop(0))
+        core.step()
+        turn += 1
+        assert turn < 2000
+    runner.cache.check_invariants()
+    assert runner.cache.used_pages == 0
+    assert sum(r.preemptions for r in requests) > 0, "the pool was meant to be too small"
+    assert any(len(r.generated_token_ids) < s.max_new_tokens for r, s in zip(requests, settings)), "nobody stopped early"
+    assert [r.generated_token_ids for r in requests] == expected
+    runner.close()
