@@ -265,7 +265,7 @@ class HipKernels:
         both = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
         return GatedLinearWeights(LinearWeights(both, None), gate.shape[0])
 
-    def _streaming(self, x: torch.Tensor, weights: LinearWeights) -> str | None:
+    def _streaming(self, x: torch.Tensor, weights: LinearWeights, gated: bool = False) -> str | None:
         """Which MFMA kernel takes this product: "skinny" (up to 16 rows of x, weights streamed),
         "medium" (up to 64, x shared through LDS), "tiled" (any number, both operands through LDS),
         or None (the BLAS library, or the generic kernel)."""
@@ -278,6 +278,10 @@ class HipKernels:
             # On the device the library is ahead of "medium" as it stands, so a captured step (which
             # costs the host nothing per launch) takes the library; a step launched kernel by kernel
             # is bound by the host, where a torch call costs four times one of ours.
+            # Except a small weight at up to 32 rows: there the library's fixed cost shows (qkv and o of
+            # the 1.5B sizes in a captured chain: 7.1 us each, against 5.9 and 4.8 at 17 rows, 6.8 and 5.5 at 32).
+            if not gated and rows <= 32 and inner % 32 == 0 and weights.out_features * inner <= (1 << 22):
+                return "skinny"
             return None
         if 16 < rows <= 64 and inner % 128 == 0:
             return "medium"
@@ -405,7 +409,7 @@ class HipKernels:
 
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
         out = self._empty((x.shape[0], weights.width), self.dtype)
-        streaming = self._streaming(x, weights.both)
+        streaming = self._streaming(x, weights.both, gated=True)
         if (
             streaming is None
             and self.wide_products == "gated"

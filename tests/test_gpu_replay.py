@@ -130,3 +130,41 @@ def test_replay_at_benchmark_layer_sizes(tmp_path_factory, tmp_path, dtype):
     # a systematic fault that stays under the bound for the largest element still moves the mean
     # (32-bit: sums over 8,960 terms in another order differ by about sqrt(8960) * 2^-24 of the spread)
     assert total / count < (1e-5 if dtype == "float32" else 0.01) * spread
+
+
+@pytest.mark.parametrize("requests", [20, 40])
+def test_captured_steps_of_many_rows_at_benchmark_layer_sizes(tmp_path_factory, requests):
+    """Decode steps of 17 to 64 rows are replayed from a graph in which the products go other ways than
+    in every other step (the BLAS library for the wide ones, the weight-streaming kernel for small
+    weights at up to 32 rows).
+    Twenty and forty requests decode side by side through the step function; every step's logits are
+    compared with the plain forward over each request's whole sequence."""
+    from llmserve_amd import CacheConfig, ModelRunner, StepEntry
+    from llmserve_amd.kernels import HipKernels
+    from llmserve_amd.weights import load_model_folder
+
+    folder = write_wide_folder(tmp_path_factory.mktemp("wide"))
+    plain_config, weights = plain.PlainConfig.from_folder(folder), plain.read_weights(folder)
+    decoded = 5
+    sequences = [random_tokens(3 + (7 * index) % 40 + decoded, WIDE.vocab_size, seed=500 + index) for index in range(requests)]
+    loaded = load_model_folder(folder, "bfloat16")
+    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(PAGE_WIDE, 4 * requests + 8, requests))
+    # prompts first, a few requests a step; then `decoded` steps of one token per request
+    for first in range(0, requests, 8):
+        group = range(first, min(first + 8, requests))
+        runner.step([StepEntry(f"r{index}", sequences[index][:-decoded], []) for index in group], create_missing=True)
+    rows = []
+    for step in range(decoded):
+        at = [len(tokens) - decoded + step for tokens in sequences]
+        logits = runner.step([StepEntry(f"r{index}", [sequences[index][at[index]]], [0]) for index in range(requests)])
+        rows.append((at, logits.clone()))
+    assert runner._graphs, "these steps were meant to be replayed from a graph"
+    expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
+    spread = float(torch.cat(expected).std())
+    for at, logits in rows:
+        for index in range(requests):
+            torch.testing.assert_close(
+                logits[index].cpu().double(), expected[index][at[index]], atol=0.06 * spread, rtol=3e-2,
+                msg=lambda m: f"request {index} position {at[index]}: {m}",
+            )
+    runner.close()
