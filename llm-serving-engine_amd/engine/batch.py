@@ -58,6 +58,7 @@ class StepBatch:
     num_logit_rows: int
     max_query_length: int
     max_context_length: int
+    every_row_wanted: bool = False  # logit_rows is 0, 1, ..., T - 1 (a step of single tokens): nothing to gather
     # Kernel libraries may keep here what they derive from the step's shape on the host (work
     # lists: built once, used by every layer, and still valid when a captured step is replayed) ...
     scratch: dict[str, Any] = field(default_factory=dict)

@@ -81,6 +81,7 @@ def _pack_step(
     facts = {
         "num_tokens": total,
         "num_logit_rows": int(logit_rows.size),
+        "every_row_wanted": bool(logit_rows.size == total and np.array_equal(logit_rows, np.arange(total, dtype=np.int32))),
         "max_query_length": int(counts.max()),
         "max_context_length": int(context.max()),
         "requests": padded,
@@ -108,6 +109,7 @@ def _view_step(
         groups=groups,
         logit_rows=views[6],
         num_logit_rows=facts["num_logit_rows"],
+        every_row_wanted=facts.get("every_row_wanted", False),
         max_query_length=facts["max_query_length"],
         max_context_length=facts["max_context_length"],
     )

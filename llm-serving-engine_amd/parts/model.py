@@ -99,6 +99,9 @@ class DecoderModel:
         """Logits [R, vocab] float32 at `batch.logit_rows`.  `cells[i]` is the
         cache cell of run i."""
         hidden, delta = self._run_layers(batch, cells)
-        rows = self.kernels.gather_rows(hidden, delta, batch.logit_rows)
-        normed = self.final_norm.forward(rows, None)
+        if getattr(batch, "every_row_wanted", False):  # the final norm adds the last layer's delta itself
+            normed = self.final_norm.forward(hidden, delta)
+        else:
+            rows = self.kernels.gather_rows(hidden, delta, batch.logit_rows)
+            normed = self.final_norm.forward(rows, None)
         return self.kernels.linear(normed, self.head, out_dtype=torch.float32)

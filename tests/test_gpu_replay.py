@@ -148,7 +148,7 @@ def test_captured_steps_of_many_rows_at_benchmark_layer_sizes(tmp_path_factory, 
     decoded = 5
     sequences = [random_tokens(3 + (7 * index) % 40 + decoded, WIDE.vocab_size, seed=500 + index) for index in range(requests)]
     loaded = load_model_folder(folder, "bfloat16")
-    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(PAGE_WIDE, 4 * requests + 8, requests))
+    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(PAGE_WIDE, 4 * requests + 8, requests + 1))
     # prompts first, a few requests a step; then `decoded` steps of one token per request
     for first in range(0, requests, 8):
         group = range(first, min(first + 8, requests))
@@ -158,7 +158,12 @@ def test_captured_steps_of_many_rows_at_benchmark_layer_sizes(tmp_path_factory, 
         at = [len(tokens) - decoded + step for tokens in sequences]
         logits = runner.step([StepEntry(f"r{index}", [sequences[index][at[index]]], [0]) for index in range(requests)])
         rows.append((at, logits.clone()))
-    assert runner._graphs, "these steps were meant to be replayed from a graph"
+        # between two replays of the graph: a step launched kernel by kernel (another request's prompt, then gone),
+        # and the host waits for the device
+        runner.step([StepEntry("between", random_tokens(9 + step, WIDE.vocab_size, seed=step), [0])], create_missing=True)
+        runner.end_request("between")
+        torch.cuda.synchronize()
+    assert len(runner._graphs) == 1, "these steps were meant to be replays of one graph"
     expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
     spread = float(torch.cat(expected).std())
     for at, logits in rows:
