@@ -11,5 +11,5 @@ DEFAULT_VARIANTS: dict[str, list[dict[str, object]]] = {
     "attention_generic": [{}],
     "sampling": [{}],
     # head sizes of the tests' models and kernel tests, and of the benchmark
-    "attention_bf16": [{"HEAD_DIM": d} for d in (16, 32, 48, 64, 80, 112, 128, 256)],
+    "attention_bf16": [{"HEAD_DIM": d} for d in (16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 256)],
 }

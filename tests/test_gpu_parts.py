@@ -286,3 +286,60 @@ def test_everything_at_once_matches_the_plain_decoder(model_folders):
     assert any(len(r.generated_token_ids) < s.max_new_tokens for r, s in zip(requests, settings)), "nobody stopped early"
     assert [r.generated_token_ids for r in requests] == expected
     runner.close()
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_random_configurations_against_the_plain_forward(tmp_path, kernels, case):
+    """Configurations drawn at random: head sizes in steps of 16 up to 256, one to five kv heads with
+    one to seventeen query heads each, widths and vocabularies that are no power of two (some no
+    multiple of 32, which the MFMA kernels refuse and the generic ones take), pages of 4 to 64, windows,
+    with and without bias and tied head, both pairings.  Three requests go through the step function in
+    portions of changing size side by side, then decode; every row's logits against the plain forward."""
+    import random
+
+    from llmserve_amd import Qwen2Config
+    from llmserve_amd.weights import write_model_folder
+
+    rng = random.Random(1000 + case)
+    kv_heads, group = rng.choice([1, 2, 3, 5]), rng.choice([1, 2, 3, 6, 7, 17])
+    window = rng.choice([None, None, 5, 19, 40])
+    config = Qwen2Config(
+        vocab_size=rng.choice([61, 128, 257, 1000, 1031]), hidden_size=rng.choice([40, 64, 72, 96, 100, 128, 136, 160, 256, 264]),
+        intermediate_size=rng.choice([48, 56, 96, 100, 128, 160, 256, 384, 392]), num_layers=rng.choice([1, 2, 3]),
+        num_attention_heads=kv_heads * group, num_key_value_heads=kv_heads,
+        head_dim=16 * rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 16]), max_position_embeddings=512,
+        rope_theta=rng.choice([100.0, 10000.0, 1e6]), rms_norm_eps=rng.choice([1e-6, 1e-5, 1e-3]),
+        attention_bias=rng.random() < 0.7, tie_word_embeddings=rng.random() < 0.5, rope_pairing=rng.choice(["adjacent", "half"]),
+        use_sliding_window=window is not None, sliding_window=window or 0, max_window_layers=rng.choice([0, 1]) if window else 0,
+    )
+    page = rng.choice([4, 8, 16, 24, 32, 64])
+    folder = write_model_folder(tmp_path / "model", config, seed=case, norm_std=0.1, std=0.08)
+    plain_config, weights = plain.PlainConfig.from_folder(folder), plain.read_weights(folder)
+    lengths = [rng.choice([1, 2, 7, 33, 70, 130]), rng.choice([3, 17, 64, 65, 97]), rng.choice([5, 40])]
+    sequences = [[rng.randrange(config.vocab_size) for _ in range(n + 6)] for n in lengths]
+    expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
+    for dtype in DTYPES:
+        loaded = load_model_folder(folder, "float32" if dtype == torch.float32 else "bfloat16")
+        pages = sum(-(-len(tokens) // page) for tokens in sequences) + 2
+        runner = ModelRunner(loaded, kernels[dtype], CacheConfig(page, pages, 4))
+        got, fed = [[] for _ in sequences], [0] * len(sequences)
+        while any(fed[i] < lengths[i] for i in range(len(sequences))):
+            entries = []
+            for i, tokens in enumerate(sequences):
+                if fed[i] < lengths[i]:
+                    count = min(rng.choice([1, 2, 5, 16, 50]), lengths[i] - fed[i])
+                    entries.append((i, StepEntry(f"r{i}", tokens[fed[i] : fed[i] + count], list(range(count)))))
+                    fed[i] += count
+            logits, at = runner.step([entry for _, entry in entries], create_missing=True), 0
+            for i, entry in entries:
+                got[i].append(logits[at : at + len(entry.tokens)].clone())
+                at += len(entry.tokens)
+        for step in range(6):
+            logits = runner.step([StepEntry(f"r{i}", [tokens[lengths[i] + step]], [0]) for i, tokens in enumerate(sequences)])
+            for i in range(len(sequences)):
+                got[i].append(logits[i : i + 1].clone())
+        for i in range(len(sequences)):
+            spread = float(expected[i].std())  # bounds in units of the logits' spread, as these models' scales differ
+            bound = dict(atol=1e-4 * spread, rtol=1e-4) if dtype == torch.float32 else dict(atol=0.2 * spread, rtol=5e-2)
+            torch.testing.assert_close(torch.cat(got[i]).cpu().double(), expected[i], **bound, msg=lambda m: f"{config} page {page} request {i}: {m}")
+        runner.close()
