@@ -80,18 +80,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   }
   while (group < groups) {
     const int next = group + WAVES;
+    // this group's x is asked for before the next group's weights: loads come back in the order they
+    // were asked for, and the products below wait for x
+    bf16x8 b[MT][GROUP];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) b[t][u] = x_live[t] ? load8(x_row[t] + (group * GROUP + u) * STEP) : zero;
+    asm volatile("" ::: "memory");  // (the compiler would put the weights first again)
     if (next < groups) {
 #pragma unroll
       for (int u = 0; u < GROUP; ++u) a_next[u] = load8_stream(w_row + (next * GROUP + u) * STEP);
     }
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      bf16x8 b[GROUP];
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int u = 0; u < GROUP; ++u) b[u] = x_live[t] ? load8(x_row[t] + (group * GROUP + u) * STEP) : zero;
-#pragma unroll
-      for (int u = 0; u < GROUP; ++u) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u], acc[t], 0, 0, 0);
-    }
+      for (int u = 0; u < GROUP; ++u) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[t][u], acc[t], 0, 0, 0);
 #pragma unroll
     for (int u = 0; u < GROUP; ++u) a[u] = a_next[u];
     group = next;
