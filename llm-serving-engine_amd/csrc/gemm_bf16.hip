@@ -172,6 +172,108 @@ static int pick_waves(const void* x, const void* w, const void* bias, int bias_i
   return pick_tiles<16, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
 }
 
+// gemm_pair: gemm_skinny for up to 16 rows of x with NT tiles of 16 weight rows a wave, which share
+// the wave's x: every workgroup reads all of x for its K range, M / (16 NT) of what it reads of the
+// weights, and the chiplets' L2 delivers little more than HBM does, so at 16 rows and NT = 1 the
+// x doubles the traffic.  More tiles a wave also means more bytes under way a wave and fewer
+// workgroups: it pays for long K ranges and big weights (7B sizes at 8 rows: gate/up 57.7 -> 52.1 us
+// with two tiles, down 32.1 -> 26.3 us with four; 1.5B sizes at 16 rows: gate/up 18.0 -> 16.9 us).
+template <int WAVES, int NT, typename TO, bool GATED>
+__global__ __launch_bounds__(WAVES * 64) void gemm_pair_kernel(const bf16_t* __restrict__ x,
+                                                               const bf16_t* __restrict__ w,
+                                                               const void* __restrict__ bias, int bias_is_float,
+                                                               TO* __restrict__ out, int M, int N, int K,
+                                                               int k_split) {
+  extern __shared__ float partial[];  // [WAVES][NT][64 lanes][4]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int k_first = blockIdx.y * k_split;
+  const bf16_t* w_row[NT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s)
+    w_row[s] = w + (size_t)min(((int)blockIdx.x * NT + s) * 16 + r, N - 1) * K + k_first + g * 8;
+  const bool x_live = r < M;
+  const bf16_t* x_row = x + (size_t)min(r, M - 1) * K + k_first + g * 8;
+  f32x4 acc[NT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s) acc[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // the bias of the four outputs this lane will finish (wave s finishes tile s) is asked for now
+  float bias_here[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias && blockIdx.y == 0 && wave < NT) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      bias_here[i] = load_as_float(bias, bias_is_float, min(((int)blockIdx.x * NT + wave) * 16 + g * 4 + i, N - 1));
+  }
+  const int groups = k_split / (STEP * GROUP);
+  bf16x8 a[NT][GROUP], a_next[NT][GROUP];
+  int group = wave;
+  if (group < groups) {
+#pragma unroll
+    for (int s = 0; s < NT; ++s)
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) a[s][u] = load8_stream(w_row[s] + (group * GROUP + u) * STEP);
+  }
+  while (group < groups) {
+    const int next = group + WAVES;
+    bf16x8 b[GROUP];
+#pragma unroll
+    for (int u = 0; u < GROUP; ++u) b[u] = x_live ? load8(x_row + (group * GROUP + u) * STEP) : zero;
+    asm volatile("" ::: "memory");
+    if (next < groups) {
+#pragma unroll
+      for (int s = 0; s < NT; ++s)
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) a_next[s][u] = load8_stream(w_row[s] + (next * GROUP + u) * STEP);
+    }
+#pragma unroll
+    for (int u = 0; u < GROUP; ++u)
+#pragma unroll
+      for (int s = 0; s < NT; ++s) acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][u], b[u], acc[s], 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < NT; ++s)
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) a[s][u] = a_next[s][u];
+    group = next;
+  }
+#pragma unroll
+  for (int s = 0; s < NT; ++s) *(f32x4*)(partial + ((wave * NT + s) * 64 + lane) * 4) = acc[s];
+  __syncthreads();
+  if (wave >= NT) return;
+  const int s = wave;
+  f32x4 total = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int v = 0; v < WAVES; ++v) total += *(const f32x4*)(partial + ((v * NT + s) * 64 + lane) * 4);
+  const int m = r;
+  const int n_first = ((int)blockIdx.x * NT + s) * 16 + g * 4;
+  if (m >= M) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) total[i] += bias_here[i];
+  if (GATED) {
+    TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (n_first + 2 * i + 1 < N) {
+        const float gate = total[2 * i], up = total[2 * i + 1];
+        dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+      }
+    }
+  } else {
+    TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n_first + i < N) dst[i] = from_float<TO>(total[i]);
+  }
+}
+
+template <int NT, typename TO, bool GATED>
+static int launch_pair(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
+                       int K, int splits, hipStream_t stream) {
+  const size_t lds = (size_t)4 * NT * 64 * 4 * sizeof(float);
+  hipLaunchKernelGGL((gemm_pair_kernel<4, NT, TO, GATED>), dim3((N + 16 * NT - 1) / (16 * NT), splits), dim3(256), lds,
+                     stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K, K / splits);
+  return LAUNCH_STATUS();
+}
+
 // ---------------------------------------------------------------------------- 16 < M <= 64
 // gemm_medium: the same product for up to 64 rows of x.  With more than one 16-row tile of x,
 // loading x per wave would cost more than streaming the weights, so a workgroup takes 64
@@ -802,6 +904,27 @@ extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bi
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % STEP || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
   if (splits > 1 && (gated || !out_is_float || K % splits || (K / splits) % STEP)) return ERR_BAD_ARGUMENT;
+  if (M <= 16 && (K / splits) % (STEP * GROUP) == 0) {
+    // several weight tiles a wave where a wave has many groups of K to walk (or x is all 16 rows) and
+    // enough workgroups are left (measured at the 1.5B and 7B sizes)
+    const int per_wave = K / splits / (STEP * GROUP) / 4;
+    const long tiles = (N + 15) / 16;
+    const long by_four = (tiles + 3) / 4 * splits, by_two = (tiles + 1) / 2 * splits;  // workgroups
+    const int share = (per_wave >= 8 && by_four >= 128 && (M > 2 || tiles <= 1024)) || (tiles >= 4096 && M >= 4) ? 4
+                      : (per_wave >= 4 || M > 8 || (tiles >= 4096 && M >= 4)) && by_two * 4 >= TARGET_WAVES ? 2
+                                                                                                            : 1;
+#define PAIR_CASE(NT)                                                                                              \
+  if (share == NT) {                                                                                               \
+    if (gated)                                                                                                     \
+      return out_is_float ? launch_pair<NT, float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)       \
+                          : launch_pair<NT, bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);     \
+    return out_is_float ? launch_pair<NT, float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)   \
+                        : launch_pair<NT, bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);      \
+  }
+    PAIR_CASE(2)
+    PAIR_CASE(4)
+#undef PAIR_CASE
+  }
   if (gated)
     return out_is_float ? pick_waves<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
                         : pick_waves<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);

@@ -75,7 +75,9 @@ def test_add_rms_norm(kernels, dtype, width, eps):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows,inner,outer", [(1, 72, 50), (5, 200, 333), (70, 129, 65), (130, 64, 1000),
                                               (1, 256, 48), (8, 1536, 272), (16, 96, 1000), (17, 1184, 50), (33, 512, 24),
-                                              (64, 4480, 130), (64, 160, 2048)])
+                                              (64, 4480, 130), (64, 160, 2048),
+                                              # up to 16 rows with two or four weight tiles a wave: a long K, all 16 rows, a vocabulary-sized N
+                                              (8, 4096, 8192), (13, 512, 16400), (5, 1536, 66000)])
 def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
     k = kernels[dtype]
     # weights scaled so that every output is of order one, whatever `inner` is
@@ -102,7 +104,7 @@ def test_linear_and_gated_linear(kernels, dtype, rows, inner, outer):
 @pytest.mark.parametrize("rows,inner,outer", [(17, 128, 64), (32, 256, 100), (33, 1536, 272), (64, 1280, 130), (64, 8960, 48),
                                               (40, 96, 77), (64, 160, 2048), (100, 256, 40), (65, 32, 128), (130, 1536, 272),
                                               (300, 96, 1000), (2048, 512, 384), (129, 129, 50), (2000, 64, 6500), (2048, 2048, 1500),
-                                              (1100, 2048, 700), (2048, 416, 6400), (1000, 160, 12900), (2040, 96, 6401)])
+                                              (1100, 2048, 700), (2048, 416, 6400), (1000, 160, 12900), (2040, 96, 6401), (8, 18944, 3584)])
 def test_products_without_the_library(own_kernels, rows, inner, outer):
     """17 to 64 rows: the kernel that shares x through LDS (K a multiple of 128), else the
     weight-streaming one with several tiles of x; more rows: the tiled one (K a multiple of 32; its
