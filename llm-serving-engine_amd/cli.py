@@ -71,6 +71,8 @@ async def _benchmark(args) -> None:
     from .benchmark import BenchmarkHarness, LoadProfile
     from .sampling import GenerationConfig
 
+    if args.linear_backend.endswith("int8"):
+        raise SystemExit(f"--linear-backend {args.linear_backend}: this engine keeps weights in bfloat16 or float32, not int8")
     loaded, tokenizer = _load_runtime(args)
     profile = LoadProfile.from_yaml(args.profile)
     if args.requests and profile.groups:
@@ -176,6 +178,14 @@ def build_parser() -> argparse.ArgumentParser:
     benchmark.add_argument("--arrival-rate", type=float)
     benchmark.add_argument("--batch-size", type=int, default=16)
     benchmark.add_argument("--output", default="artifacts/benchmark.json")
+    # The reference's switches between its own back ends (`cli.py:263-271`) parse here too, so that its
+    # command lines carry over: this engine has one attention path and one product path (HIP kernels).
+    benchmark.add_argument("--rebuild-device-metadata", action="store_true",
+                           help="accepted for the reference's command lines: index arrays are rebuilt every step here anyway")
+    benchmark.add_argument("--paged-attention-backend", choices=("hip", "pytorch", "triton"), default="hip",
+                           help="the reference's names are accepted and mean the one back end there is: HIP kernels")
+    benchmark.add_argument("--linear-backend", choices=("bf16", "fp16", "reference-int8", "triton-int8"), default="bf16",
+                           help="bf16 (fp16 is read as: not quantized); the int8 back ends are refused, weights are not quantized here")
     _engine_options(benchmark)
 
     generate = commands.add_parser("generate", help="generate tokens for one prompt")

@@ -26,6 +26,17 @@ def test_benchmark_options_are_the_references():
         build_parser().parse_args(["benchmark", "--policy", "random"])
     with pytest.raises(SystemExit):
         build_parser().parse_args(["serve"])  # servers are outside this engine
+    # the reference's switches between its back ends (cli.py:263-271) parse, so its command lines carry over
+    carried = build_parser().parse_args(["benchmark", "--rebuild-device-metadata", "--paged-attention-backend", "triton",
+                                         "--linear-backend", "fp16"])
+    assert carried.rebuild_device_metadata and carried.paged_attention_backend == "triton" and carried.linear_backend == "fp16"
+    quantized = build_parser().parse_args(["benchmark", "--linear-backend", "triton-int8"])
+    with pytest.raises(SystemExit, match="int8"):  # refused before anything is loaded
+        import asyncio
+
+        from llmserve_amd.cli import _benchmark
+
+        asyncio.run(_benchmark(quantized))
     generate = build_parser().parse_args(["generate", "--prompt-tokens", "1,2,3", "--temperature", "0.8", "--top-p", "0.9"])
     assert (generate.max_tokens, generate.temperature, generate.top_p) == (32, 0.8, 0.9)
     replay = build_parser().parse_args(["replay", "--model", "m", "--out", "o", "--max-tokens", "256"])
