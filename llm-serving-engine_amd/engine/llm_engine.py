@@ -307,9 +307,17 @@ class LLMEngine:
         dtype: torch.dtype | str = torch.bfloat16,
         kernels: Any = None,
         max_sequence_length: int | None = None,
+        paged_attention_backend: str = "hip",
+        cache_device_metadata: bool = True,
     ) -> None:
+        """`paged_attention_backend` and `cache_device_metadata` are the reference's switches between its own
+        back ends (`engine.py:111-125`), taken so that its calls carry over: there is one attention path here
+        (the reference's names "pytorch" and "triton" are read as it), and a step's index arrays are packed
+        anew for every step whatever the second says."""
         from ..weights.loader import run_dtype
 
+        if paged_attention_backend not in ("hip", "pytorch", "triton"):
+            raise ValueError(f"unknown paged_attention_backend {paged_attention_backend!r}")
         dtype = run_dtype(dtype)
         if not isinstance(model, LoadedModel):
             model = load_model_folder(model, dtype)
