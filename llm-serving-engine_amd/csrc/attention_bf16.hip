@@ -237,6 +237,10 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   [[maybe_unused]] int new_slot = -1;
   [[maybe_unused]] int early_k = -1, early_k_hi = -1, early_v = -1;
   const bool early_pages = FUSED && window <= 0 && splits == 1 && (wave * KEYS + KEYS - 1) / page_size < table_width;
+  // (heads up to 128 wide leave the registers for a wave's second step to be asked for together with its first)
+  constexpr bool TWO_STEPS = FUSED && HEAD_DIM <= 128;
+  [[maybe_unused]] int second_k = -1, second_k_hi = -1, second_v = -1;
+  const bool second_pages = TWO_STEPS && early_pages && ((wave + WAVES) * KEYS + KEYS - 1) / page_size < table_width;
   if (FUSED) {
     const bf16_t* k_row = qkv + (size_t)row0 * row_width + (size_t)(heads + kv_head) * D;
     const bf16_t* v_row = k_row + (size_t)kv_heads * D;
@@ -259,6 +263,12 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
       early_k = table[key / page_size];
       early_k_hi = table[(key + 4) / page_size];
       early_v = table[(wave * KEYS + 8 * q) / page_size];
+    }
+    if (second_pages) {
+      const int key = (wave + WAVES) * KEYS + 8 * (c >> 2) + (c & 3);
+      second_k = table[key / page_size];
+      second_k_hi = table[(key + 4) / page_size];
+      second_v = table[((wave + WAVES) * KEYS + 8 * q) / page_size];
     }
   }
   const int last_key = position0 + tokens - 1;
@@ -426,6 +436,46 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
     StepPages pages = early_pages && step0 < step_last ? StepPages{early_k, early_k_hi, early_v} : pages_of(step0);
     fetch_keys(step0, pages, loads);
     fetch_values(step0, pages, loads);
+    if constexpr (TWO_STEPS) {
+      // A step of single tokens is a few trips to memory in a row, and a wave has two or three steps to
+      // walk: its second step's K and V are asked for together with the first's, into registers of their
+      // own, and each of the two sets is filled again as soon as its step has been multiplied.
+      auto multiply = [&](int step, StepLoads& L) {
+        f32x4 s_lo[COLUMN_TILES], s_hi[COLUMN_TILES];
+        scores_of(columns, L, s_lo, s_hi);
+        const int key0 = step * KEYS;
+        const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
+        weigh_and_add(columns, L, s_lo, s_hi, key0, q, interior, last_key,
+                      min(max(key0 + 8 * q, low_limit), high_limit), scale_log2);
+      };
+      StepLoads ahead;
+      const int step1 = step0 + WAVES;
+      if (step1 < step_end) {
+        const StepPages pages1 =
+            second_pages && step1 < step_last ? StepPages{second_k, second_k_hi, second_v} : pages_of(step1);
+        fetch_keys(step1, pages1, ahead);
+        fetch_values(step1, pages1, ahead);
+      }
+      StepPages pages_even = pages, pages_odd = pages;  // of the steps that will fill `loads` and `ahead` again
+      if (step0 + 2 * WAVES < step_end) pages_even = pages_of(step0 + 2 * WAVES);
+      if (step0 + 3 * WAVES < step_end) pages_odd = pages_of(step0 + 3 * WAVES);
+      for (int step = step0; step < step_end; step += 2 * WAVES) {
+        multiply(step, loads);
+        if (step + 2 * WAVES < step_end) {
+          fetch_keys(step + 2 * WAVES, pages_even, loads);
+          fetch_values(step + 2 * WAVES, pages_even, loads);
+          if (step + 4 * WAVES < step_end) pages_even = pages_of(step + 4 * WAVES);
+        }
+        if (step + WAVES < step_end) {
+          multiply(step + WAVES, ahead);
+          if (step + 3 * WAVES < step_end) {
+            fetch_keys(step + 3 * WAVES, pages_odd, ahead);
+            fetch_values(step + 3 * WAVES, pages_odd, ahead);
+            if (step + 5 * WAVES < step_end) pages_odd = pages_of(step + 5 * WAVES);
+          }
+        }
+      }
+    } else {
     if (step0 + WAVES < step_end) pages = pages_of(step0 + WAVES);
     for (int step = step0; step < step_end; step += WAVES) {
       const bool more = step + WAVES < step_end;
@@ -438,6 +488,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
                     min(max(key0 + 8 * q, low_limit), high_limit), scale_log2);
       if (more) fetch_values(step + WAVES, pages, loads);
       if (step + 2 * WAVES < step_end) pages = pages_of(step + 2 * WAVES);
+    }
     }
   }
 
