@@ -12,6 +12,10 @@
 //               first kept entry, in rank order, whose running sum exceeds u * (kept mass).
 // Sums are accumulated in float64 in an order fixed by the block size.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
+#include <stdio.h>
 
 #define SAMPLE_THREADS 1024
 
@@ -126,6 +130,48 @@ extern "C" int llmserve_argmax(const float* logits, float* piece_values, int* pi
                                int vocab, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) return ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(rows, ARGMAX_PIECES), dim3(SAMPLE_THREADS), 0, stream, logits,
+                     piece_values, piece_indices, vocab, ARGMAX_PIECES);
+  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(WAVE), 0, stream, piece_values, piece_indices, out,
+                     ARGMAX_PIECES);
+  return LAUNCH_STATUS();
+}
+
+// The pieces' (value, index) pairs of `llmserve_argmax_static`: values first, then indices.  Each GPU
+// holds its own copy of the array at its own address; host code reaches it only through the address
+// that hipGetSymbolAddress gave for that device, never through the array's name.
+#define ARGMAX_STATIC_SLOTS (LLMSERVE_ARGMAX_STATIC_MAX_ROWS * ARGMAX_PIECES)
+static __device__ __align__(256) unsigned char argmax_static_scratch[ARGMAX_STATIC_SLOTS * (sizeof(float) + sizeof(int))];
+
+#define ARGMAX_STATIC_MAX_DEVICES 64
+static void* argmax_static_address[ARGMAX_STATIC_MAX_DEVICES];  // by device; null until that device's first call
+static std::mutex argmax_static_lock;
+
+extern "C" int llmserve_argmax_static(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0) return ERR_BAD_ARGUMENT;
+  if (rows > LLMSERVE_ARGMAX_STATIC_MAX_ROWS) {
+    fprintf(stderr, "llmserve_argmax_static: %d rows are more than the %d its fixed scratch buffer holds\n", rows,
+            LLMSERVE_ARGMAX_STATIC_MAX_ROWS);
+    return LLMSERVE_ERR_TOO_LARGE;
+  }
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return (int)status;
+  if (device < 0 || device >= ARGMAX_STATIC_MAX_DEVICES) return ERR_BAD_ARGUMENT;
+  void* base = nullptr;
+  {
+    std::lock_guard<std::mutex> guard(argmax_static_lock);
+    base = argmax_static_address[device];
+    if (base == nullptr) {  // once per device, with that device current
+      status = hipGetSymbolAddress(&base, HIP_SYMBOL(argmax_static_scratch));
+      if (status != hipSuccess || base == nullptr) return status != hipSuccess ? (int)status : ERR_BAD_ARGUMENT;
+      argmax_static_address[device] = base;
+    }
+  }
+  // Nothing has to start at zero: the first kernel writes every slot that the second one reads.
+  float* piece_values = (float*)base;
+  int* piece_indices = (int*)((unsigned char*)base + ARGMAX_STATIC_SLOTS * sizeof(float));
   hipLaunchKernelGGL(argmax_pieces_kernel, dim3(rows, ARGMAX_PIECES), dim3(SAMPLE_THREADS), 0, stream, logits,
                      piece_values, piece_indices, vocab, ARGMAX_PIECES);
   hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(WAVE), 0, stream, piece_values, piece_indices, out,
