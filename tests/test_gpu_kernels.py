@@ -186,6 +186,9 @@ ATTENTION_SHAPES = [  # heads, kv_heads, dim, page
     (3, 1, 112, 64),
     (4, 2, 256, 16),  # the widest head the matrix-core kernel takes: one column tile a wave
     (4, 4, 16, 1),
+    (40, 8, 128, 16),  # the 32B sizes: five query heads a kv head
+    (10, 2, 128, 16),
+    (28, 4, 128, 16),  # the 7B sizes: seven
 ]
 
 
@@ -259,7 +262,7 @@ def test_paged_attention_finds_a_far_key_among_hundreds(kernels, dtype):
 
 
 @pytest.mark.parametrize("window", [None, 21, 64])
-@pytest.mark.parametrize("heads,kv_heads,page", [(12, 2, 16), (28, 4, 8), (40, 2, 16), (5, 5, 24), (3, 1, 32)])
+@pytest.mark.parametrize("heads,kv_heads,page", [(12, 2, 16), (28, 4, 8), (40, 2, 16), (5, 5, 24), (3, 1, 32), (40, 8, 16), (10, 2, 16)])
 def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, window):
     """At head size 128 prompt portions may go to the kernel whose four waves share each step's K and V
     through LDS: portions that fill its workgroups, that leave waves empty, that end inside a step of 32
@@ -405,7 +408,7 @@ def test_sampling_edges(kernels):
 
 
 @pytest.mark.parametrize("pairing", ["adjacent", "half", "none"])
-@pytest.mark.parametrize("heads,kv_heads,dim,page", [(12, 2, 128, 16), (6, 1, 64, 8), (5, 5, 32, 4), (4, 2, 48, 16), (40, 2, 64, 16), (2, 1, 256, 16)])
+@pytest.mark.parametrize("heads,kv_heads,dim,page", [(12, 2, 128, 16), (6, 1, 64, 8), (5, 5, 32, 4), (4, 2, 48, 16), (40, 2, 64, 16), (2, 1, 256, 16), (40, 8, 128, 16), (10, 2, 128, 16), (28, 4, 128, 16)])
 def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
     """A step of single tokens: rotation, the store of the new key and value, attention and the
     merge of key splits in one kernel (or, where the sizes do not allow it, in the separate ones):

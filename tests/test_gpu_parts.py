@@ -301,7 +301,7 @@ def test_random_configurations_against_the_plain_forward(tmp_path, kernels, case
     from llmserve_amd.weights import write_model_folder
 
     rng = random.Random(1000 + case)
-    kv_heads, group = rng.choice([1, 2, 3, 5]), rng.choice([1, 2, 3, 6, 7, 17])
+    kv_heads, group = rng.choice([1, 2, 3, 5]), rng.choice([1, 2, 3, 5, 6, 7, 17])
     window = rng.choice([None, None, 5, 19, 40])
     config = Qwen2Config(
         vocab_size=rng.choice([61, 128, 257, 1000, 1031]), hidden_size=rng.choice([40, 64, 72, 96, 100, 128, 136, 160, 256, 264]),

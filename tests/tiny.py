@@ -93,8 +93,47 @@ WIDE = Qwen2Config(
 PAGE_WIDE = 16
 
 
-def write_wide_folder(root: Path) -> Path:
-    return write_model_folder(root / "W", WIDE, seed=31, norm_std=0.1)
+# The 7B layer sizes (seven query heads a kv head, widths 3584 and 18944, untied head), two layers.
+WIDE_7B = Qwen2Config(
+    vocab_size=1019,
+    hidden_size=3584,
+    intermediate_size=18944,
+    num_layers=2,
+    num_attention_heads=28,
+    num_key_value_heads=4,
+    head_dim=128,
+    max_position_embeddings=4096,
+    rope_theta=1e6,
+    rms_norm_eps=1e-6,
+    attention_bias=True,
+    tie_word_embeddings=False,
+    rope_pairing="half",
+)
+
+# The 32B layer sizes (five query heads a kv head, widths 5120 and 27648, eps 1e-5, untied head), one layer:
+# a layer holds 488 million weights, and the plain forward runs on the CPU.
+WIDE_32B = Qwen2Config(
+    vocab_size=1013,
+    hidden_size=5120,
+    intermediate_size=27648,
+    num_layers=1,
+    num_attention_heads=40,
+    num_key_value_heads=8,
+    head_dim=128,
+    max_position_embeddings=4096,
+    rope_theta=1e6,
+    rms_norm_eps=1e-5,
+    attention_bias=True,
+    tie_word_embeddings=False,
+    rope_pairing="half",
+)
+
+WIDE_CONFIGS = {"1.5B": (WIDE, 31), "7B": (WIDE_7B, 37), "32B": (WIDE_32B, 41)}
+
+
+def write_wide_folder(root: Path, sizes: str = "1.5B") -> Path:
+    config, seed = WIDE_CONFIGS[sizes]
+    return write_model_folder(root / f"W{sizes}", config, seed=seed, norm_std=0.1)
 
 
 def write_tiny_folders(root: Path) -> dict[str, Path]:
