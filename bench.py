@@ -39,6 +39,8 @@ def parse() -> argparse.Namespace:
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--seed", type=int, default=7)
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64")
+    parser.add_argument("--skip-context-points", action="store_true",
+                        help="leave out decoding at contexts of 8k and 30k (batch 8) and 4k (batch 64)")
     return parser.parse_args()
 
 
@@ -52,12 +54,12 @@ def main() -> int:
 
     import torch
 
-    from llmserve_amd import CacheConfig, EngineCore, GenerationConfig, ModelRunner, Qwen2Config, SchedulerConfig, StepEntry
-    from llmserve_amd.engine import RequestState
+    from llmserve_amd import CacheConfig, EngineCore, GenerationConfig, ModelRunner, SchedulerConfig, StepEntry
+    from llmserve_amd.engine import Request
     from llmserve_amd.kernels import HipKernels
-    from llmserve_amd.weights import random_model, run_dtype
+    from llmserve_amd.weights import random_model, read_config, run_dtype
 
-    full = Qwen2Config.from_json_file(args.config)
+    _, full = read_config(args.config)  # the architecture is whatever the file names
     config = dataclasses.replace(full, num_layers=args.layers) if args.layers else full
     dtype = run_dtype(args.dtype)
     device = torch.device("cuda:0")
@@ -65,27 +67,40 @@ def main() -> int:
     tensors, spec = loaded.tensors, loaded.spec
     kernels = HipKernels(dtype, device)
     page = 16
-    most = max(64, args.batch)
-    per_request = args.prompt_len + 256 + page
-    pages = most * (-(-per_request // page)) + args.prefill_len // page + 8
+    # (batch, prompt length) of every decode measurement: the headline, batch 1 and 64, and longer contexts
+    headline = (args.batch, args.prompt_len)
+    extra = {} if args.skip_points else {"decode_b1": (1, args.prompt_len), "decode_b64": (64, args.prompt_len)}
+    if not args.skip_points and not args.skip_context_points:
+        extra.update({"decode_b8_ctx8k": (8, 8192), "decode_b8_ctx30k": (8, 30000), "decode_b64_ctx4k": (64, 4096)})
+    longest = getattr(config, "max_position_embeddings", 32768)
+    extra = {name: shape for name, shape in extra.items() if shape[1] + 300 <= longest}
+    most = max(batch for batch, _ in [headline, *extra.values()])
+    pages = max(batch * (-(-(prompt + 256 + page) // page)) for batch, prompt in [headline, *extra.values()])
+    pages += args.prefill_len // page + 8
     runner = ModelRunner(loaded, kernels, CacheConfig(block_size=page, num_blocks=pages, max_sequences=most + 1))
+    # What a decode step has to read: every weight it uses once (of an untied embedding table only the
+    # rows of the step's tokens) and the cache of the live requests.
     weight_bytes = sum(t.numel() * t.element_size() for t in tensors.values())
-    element = 2 if dtype == torch.bfloat16 else 4
-    kv_bytes_per_token = 2 * config.num_layers * config.num_key_value_heads * config.head_dim * element
+    embedding_bytes = 0
+    if not spec.tie_embeddings:
+        table = tensors[spec.embedding_name]
+        embedding_bytes = table.numel() * table.element_size()
+        weight_bytes -= embedding_bytes
+    embedding_row_bytes = spec.hidden_size * tensors[spec.embedding_name].element_size() if embedding_bytes else 0
+    kv_bytes_per_token = runner.cache.bytes_per_token
     generator = torch.Generator().manual_seed(args.seed)
 
     def tokens(count: int) -> list[int]:
-        return torch.randint(4, config.vocab_size, (count,), generator=generator).tolist()
+        return torch.randint(4, spec.vocab_size, (count,), generator=generator).tolist()
 
-    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        """(seconds for `steps` decode steps, mean context length during them)"""
-        core = EngineCore(runner, SchedulerConfig(batch, max(2048, batch)), prefill_chunk_size=512)
-        requests = []
-        for index in range(batch):
-            request = RequestState(f"b{batch}-{index}", tokens(args.prompt_len), warmup + steps + 1)
-            core.submit(request, GenerationConfig(max_new_tokens=warmup + steps + 1))
-            requests.append(request)
-        while any(not r.generated_token_ids for r in requests):
+    def decode(batch: int, prompt_len: int, steps: int, warmup: int) -> dict:
+        """`steps` timed decode steps of `batch` requests after prompts of `prompt_len` tokens."""
+        core = EngineCore(runner, SchedulerConfig(batch, max(2048, batch)), prefill_chunk_size=min(2048, prompt_len))
+        settings = GenerationConfig(max_new_tokens=warmup + steps + 1)
+        requests = [Request(f"b{batch}-{prompt_len}-{index}", tokens(prompt_len), settings) for index in range(batch)]
+        for request in requests:
+            core.submit(request)
+        while any(not request.output for request in requests):
             core.step()
         for _ in range(warmup):
             core.step()
@@ -95,10 +110,19 @@ def main() -> int:
             core.step()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
-        assert all(len(r.generated_token_ids) == 1 + warmup + steps for r in requests)
+        assert all(len(request.output) == 1 + warmup + steps for request in requests)
         for request in requests:
             core.finish(request)
-        return elapsed, args.prompt_len + 1 + warmup + (steps - 1) / 2.0
+        context = prompt_len + 1 + warmup + (steps - 1) / 2.0  # mean context length during the timed steps
+        step_bytes = weight_bytes + batch * embedding_row_bytes + batch * context * kv_bytes_per_token
+        seconds = elapsed / steps
+        return {
+            "tokens_per_s": batch * steps / elapsed,
+            "ms_per_step": 1000 * seconds,
+            "context": context,
+            "achieved_gbs": step_bytes / seconds / 1e9,
+            "generated": 1 + warmup + steps,
+        }
 
     def prefill(length: int, repeats: int = 5) -> float:
         times = []
@@ -113,36 +137,45 @@ def main() -> int:
         return statistics.median(times[1:])
 
     steps = min(args.steps, 250 - args.warmup)
-    elapsed, context = decode(args.batch, steps, args.warmup)
-    value = args.batch * steps / elapsed
-    step_bytes = weight_bytes + args.batch * context * kv_bytes_per_token
-    achieved = step_bytes / (elapsed / steps) / 1e9
+    main_run = decode(*headline, steps, args.warmup)
 
     prefill_seconds = prefill(args.prefill_len)
     layer_weights = sum(
         t.numel() for name, t in tensors.items() if t.ndim == 2 and name != spec.embedding_name and name != spec.head_name
     )
     t = args.prefill_len
-    flops = 2.0 * t * layer_weights + 2.0 * config.vocab_size * config.hidden_size
-    flops += config.num_layers * 4.0 * config.num_attention_heads * config.head_dim * t * (t + 1) / 2
+    flops = 2.0 * t * layer_weights + 2.0 * spec.vocab_size * spec.hidden_size
+    # attention: scores and weighted values, 2 flops each for every (query, key, head, dimension) below the diagonal
+    score_width = sum(
+        need.num_kv_heads * need.head_dim * heads_per_kv
+        for need, heads_per_kv in attention_widths(spec)
+    )
+    flops += 4.0 * score_width * t * (t + 1) / 2
     peak = PEAK_FLOPS["bf16" if dtype == torch.bfloat16 else "fp32"]
 
     points = {}
-    if not args.skip_points:
-        for batch in (1, 64):
-            short = min(steps, 64)
-            seconds, _ = decode(batch, short, min(args.warmup, 8))
-            points[f"decode_b{batch}"] = round(batch * short / seconds, 1)
+    for name, (batch, prompt_len) in extra.items():
+        short = min(steps, 64 if prompt_len <= 4096 else 32)
+        run = decode(batch, prompt_len, short, min(args.warmup, 8))
+        points[name] = round(run["tokens_per_s"], 1)
+        points[name + "_ms_per_step"] = round(run["ms_per_step"], 4)
+        points[name + "_hbm_frac"] = round(run["achieved_gbs"] / HBM_PEAK_GBS, 4)
 
     label = Path(args.config).stem.replace("qwen", "Qwen").replace("b", "B")
+    sizes = {
+        key: getattr(config, key)
+        for key in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size",
+                    "rope_theta", "rms_norm_eps", "max_position_embeddings")
+        if hasattr(config, key)
+    }
     record = {
         "metric": f"decode tok/s at batch {args.batch}, {args.prompt_len}-token prompts ({label} shape)",
-        "value": round(value, 1),
+        "value": round(main_run["tokens_per_s"], 1),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": steps,
         "warmup": args.warmup,
-        "ms_per_step": round(1000 * elapsed / steps, 4),
+        "ms_per_step": round(main_run["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -150,23 +183,17 @@ def main() -> int:
         "data": "synthetic: seeded random weights, uniform random token ids",
         "config": {
             "model": f"{label} layer sizes, random weights",
-            "layers": config.num_layers,
+            "layers": len(spec.run_order),
             "layers_full": full.num_layers,
-            "hidden": config.hidden_size,
-            "heads": config.num_attention_heads,
-            "kv_heads": config.num_key_value_heads,
-            "head_dim": config.head_dim,
-            "intermediate": config.intermediate_size,
-            "vocab": config.vocab_size,
-            "rope_theta": config.rope_theta,
-            "rms_norm_eps": config.rms_norm_eps,
-            "tied_embeddings": config.tie_word_embeddings,
-            "max_context": config.max_position_embeddings,
+            **sizes,
+            "vocab_size": spec.vocab_size,
+            "tied_embeddings": spec.tie_embeddings,
             "page_size": page,
             "global_batch": args.batch,
             "seq_len": args.prompt_len,
-            "decode_context": round(context, 1),
-            "output_tokens": 256,
+            "decode_context": round(main_run["context"], 1),
+            "output_tokens": main_run["generated"],
+            "kv_bytes_per_token": kv_bytes_per_token,
             "parallelism": "none (1 GPU)",
         },
         "prefill": {
@@ -177,15 +204,28 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "achieved": round(achieved, 1),
+            "achieved": round(main_run["achieved_gbs"], 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "frac": round(main_run["achieved_gbs"] / HBM_PEAK_GBS, 4),
         },
         "points": points,
     }
     print(json.dumps(record))
     return 0
+
+
+def attention_widths(spec):
+    """(cache need, query heads per kv head) of every run of the run order whose mixer attends over pages."""
+    from llmserve_amd.parts.base import PagedKeyValue
+
+    found = []
+    for index, run in enumerate(spec.run_order):
+        need = spec.cell_need(index)
+        mixer = getattr(spec.layers[run.layer].block, "mixer", None)
+        if isinstance(need, PagedKeyValue) and hasattr(mixer, "num_heads"):
+            found.append((need, mixer.num_heads // need.num_kv_heads))
+    return found
 
 
 if __name__ == "__main__":

@@ -285,6 +285,51 @@ class CacheManager:
         blocks = math.ceil(record.length / self.page_size)
         return self.groups[group].tables[record.slot, :blocks].tolist()
 
+    # ------------------------------------------------------------------ host-side read paths
+
+    def _paged_cell(self, run: int) -> tuple[PageGroup, int, int]:
+        entry = self._cell_of_run[run] if 0 <= run < len(self._cell_of_run) else None
+        if entry is None or entry[0] != "pages":
+            raise ValueError(f"run {run} of the run order keeps no pages")
+        return self.groups[entry[1]], entry[1], entry[2]
+
+    def iter_pages(self, request_id: str, run: int):
+        """Walks what run `run` of the run order has cached for the request, page by page in logical
+        order: yields (first position, keys [n, kv_heads, head_dim], values [n, kv_heads, head_dim]),
+        the last page cut at the request's length, pages that a window has given back left out.  A
+        debugging and testing aid, as the reference's `iter_kv_blocks` (`kv_cache.py:268-296`): the
+        kernels read through the block tables themselves."""
+        group, group_index, cell = self._paged_cell(run)
+        record = self.sequences[request_id]
+        table = group.tables[record.slot]
+        page_size = self.page_size
+        for block in range(record.released[group_index], math.ceil(record.length / page_size)):
+            held = min(page_size, record.length - block * page_size)
+            page = int(table[block])
+            keys = group.storage[cell, 0, page, :, :held]  # [kv_heads, n, head_dim]
+            # value pages are kept transposed, [kv_heads, head_dim, offset]
+            values = group.storage[cell, 1, page].view(group.need.num_kv_heads, group.need.head_dim, page_size)[:, :, :held]
+            yield block * page_size, keys.transpose(0, 1), values.permute(2, 0, 1)
+
+    def gather(self, request_id: str, run: int) -> tuple[int, torch.Tensor, torch.Tensor]:
+        """(first cached position, keys, values) of the request in run `run` as two contiguous tensors
+        [n, kv_heads, head_dim] (`kv_cache.py:318-342`)."""
+        pages = list(self.iter_pages(request_id, run))
+        if not pages:
+            need = self._paged_cell(run)[0].need
+            empty = torch.empty((0, need.num_kv_heads, need.head_dim), dtype=self.dtype, device=self.device)
+            return self.sequences[request_id].length, empty, empty.clone()
+        return pages[0][0], torch.cat([keys for _, keys, _ in pages]), torch.cat([values for _, _, values in pages])
+
+    def block_table_tensors(self, request_ids: list[str], group: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
+        """A compact [requests, widest] block table (-1 where nothing is held) and the requests'
+        lengths, both int32 on the host (`kv_cache.py:298-316`)."""
+        records = [self.sequences[request_id] for request_id in request_ids]
+        widest = max((math.ceil(record.length / self.page_size) for record in records), default=0)
+        tables = np.stack([self.groups[group].tables[record.slot, :widest] for record in records]) if records else np.zeros((0, 0), np.int32)
+        lengths = np.array([record.length for record in records], dtype=np.int32)
+        return torch.from_numpy(tables.copy()), torch.from_numpy(lengths)
+
     def free(self, request_id: str) -> None:
         """Gives back everything the request holds (reference `kv_cache.py:344-350`)."""
         record = self.sequences.pop(request_id)
@@ -332,6 +377,11 @@ class CacheManager:
     @property
     def capacity_tokens(self) -> int:
         return self.config.num_blocks * self.page_size
+
+    @property
+    def bytes_per_token(self) -> int:
+        """What one cached token takes over all runs of the run order that keep pages."""
+        return sum(group.bytes_per_page for group in self.groups) // self.page_size
 
     def check_invariants(self) -> None:
         """No page lost, held twice, or held by a request that is gone."""

@@ -7,7 +7,10 @@ argparse subcommands, with the reference's option names and meanings where it ha
     llmserve random-model  write a model folder with seeded random weights
 
 The reference's `serve`, `quantize-eval` and `speculative-eval` have no counterpart here:
-servers, quantized weights and speculative decoding are outside this engine.
+servers, quantized weights and speculative decoding are outside this engine.  Nor have its
+switches between back ends (`--paged-attention-backend`, `--linear-backend`,
+`--rebuild-device-metadata`, `cli.py:263-271`): there is one attention path and one product
+path here, and an option that chose nothing would only pretend.
 """
 
 from __future__ import annotations
@@ -27,9 +30,8 @@ def _load_runtime(args):
     """A model folder; or weights drawn from --seed at the sizes of a config.json
     (--random-weights, made on the device: no folder is written); or without either the
     bundled tiny configuration with such weights and the byte tokenizer (`cli.py:22-45`)."""
-    from .config import Qwen2Config
     from .engine.tokenizer import ByteTokenizer, FileTokenizer
-    from .weights import load_model_folder, random_model, write_model_folder
+    from .weights import load_model_folder, random_model, read_config, write_model_folder
 
     if args.model and getattr(args, "random_weights", None):
         raise SystemExit("give --model or --random-weights, not both")
@@ -43,7 +45,7 @@ def _load_runtime(args):
         except FileNotFoundError:
             tokenizer = ByteTokenizer()
         return loaded, tokenizer
-    config = Qwen2Config.from_json_file(ROOT / "configs" / "tiny.json")
+    _, config = read_config(ROOT / "configs" / "tiny.json")  # whatever architecture that file names
     folder = write_model_folder(Path(tempfile.mkdtemp(prefix="llmserve-tiny-")), config, seed=args.seed)
     return load_model_folder(folder, args.dtype), ByteTokenizer()
 
@@ -71,21 +73,19 @@ async def _benchmark(args) -> None:
     from .benchmark import BenchmarkHarness, LoadProfile
     from .sampling import GenerationConfig
 
-    if args.linear_backend.endswith("int8"):
-        raise SystemExit(f"--linear-backend {args.linear_backend}: this engine keeps weights in bfloat16 or float32, not int8")
     loaded, tokenizer = _load_runtime(args)
     profile = LoadProfile.from_yaml(args.profile)
     if args.requests and profile.groups:
         raise SystemExit("--requests cannot change a profile made of groups")
+    batch_size = 1 if args.config in ("naive", "paged") else args.batch_size
+    engine = _engine(args, loaded, tokenizer, batch_size=batch_size, mode="static" if args.config == "static" else "continuous")
     profile = replace(
         profile,
         requests=args.requests or profile.requests,
         arrival_rate=args.arrival_rate or profile.arrival_rate,
-        vocabulary_size=loaded.config.vocab_size,
-    ).fitted(loaded.config.max_position_embeddings)
+        vocabulary_size=engine.runner.vocab_size,
+    ).fitted(engine.cache.max_sequence_length)
     harness = BenchmarkHarness(profile)
-    batch_size = 1 if args.config in ("naive", "paged") else args.batch_size
-    engine = _engine(args, loaded, tokenizer, batch_size=batch_size, mode="static" if args.config == "static" else "continuous")
 
     def settings(count: int) -> GenerationConfig:
         return GenerationConfig(max_new_tokens=count, temperature=0.0, seed=args.seed, stop_token_ids=())
@@ -93,22 +93,25 @@ async def _benchmark(args) -> None:
     if args.config == "naive":
         lock = asyncio.Lock()
 
-        async def generate(spec, callback):
+        async def generate(arrival, callback):
             async with lock:  # reference engine.py:83-105: no cache is kept between tokens
-                prompt, output = list(spec.prompt_token_ids), []
-                for _ in range(spec.max_new_tokens):
-                    token = (await engine.generate(prompt + output, settings(1)))[0]
-                    output.append(token)
-                    callback(token)
-                return output
+                sequence = list(arrival.prompt)
+                for _ in range(arrival.max_new_tokens):
+                    sequence += await engine.generate(sequence, settings(1))
+                    callback(sequence[-1])
+                return sequence[len(arrival.prompt):]
+
+        facts = None
     else:
 
-        async def generate(spec, callback):
+        async def generate(arrival, callback):
             return await engine.generate(
-                list(spec.prompt_token_ids), settings(spec.max_new_tokens), callback, request_id=spec.request_id
+                list(arrival.prompt), settings(arrival.max_new_tokens), callback, request_id=arrival.request_id
             )
 
-    report = await harness.run(f"{args.config}-{args.policy}", generate)
+        facts = engine.request_facts
+
+    report = await harness.run(f"{args.config}-{args.policy}", generate, facts)
     report.cache = engine.cache_stats
     report.metadata["engine"] = engine.iteration_stats
     await engine.close()
@@ -144,10 +147,9 @@ def _replay(args) -> int:
 def _random_model(args) -> None:
     import torch
 
-    from .config import Qwen2Config
-    from .weights import write_model_folder
+    from .weights import read_config, write_model_folder
 
-    config = Qwen2Config.from_json_file(args.config)
+    _, config = read_config(args.config)
     folder = write_model_folder(args.output, config, args.seed, dtype=torch.bfloat16, norm_std=args.norm_std,
                                 bias_std=args.bias_std, std=args.std)
     print(folder)
@@ -178,14 +180,6 @@ def build_parser() -> argparse.ArgumentParser:
     benchmark.add_argument("--arrival-rate", type=float)
     benchmark.add_argument("--batch-size", type=int, default=16)
     benchmark.add_argument("--output", default="artifacts/benchmark.json")
-    # The reference's switches between its own back ends (`cli.py:263-271`) parse here too, so that its
-    # command lines carry over: this engine has one attention path and one product path (HIP kernels).
-    benchmark.add_argument("--rebuild-device-metadata", action="store_true",
-                           help="accepted for the reference's command lines: index arrays are rebuilt every step here anyway")
-    benchmark.add_argument("--paged-attention-backend", choices=("hip", "pytorch", "triton"), default="hip",
-                           help="the reference's names are accepted and mean the one back end there is: HIP kernels")
-    benchmark.add_argument("--linear-backend", choices=("bf16", "fp16", "reference-int8", "triton-int8"), default="bf16",
-                           help="bf16 (fp16 is read as: not quantized); the int8 back ends are refused, weights are not quantized here")
     _engine_options(benchmark)
 
     generate = commands.add_parser("generate", help="generate tokens for one prompt")

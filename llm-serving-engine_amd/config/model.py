@@ -212,5 +212,6 @@ class Qwen2Config(ArchitectureConfig):
         }
         for item in fields(self):
             key = "num_hidden_layers" if item.name == "num_layers" else item.name
-            values[key] = getattr(self, item.name)
+            if getattr(self, item.name) is not None:  # an option that is off has no key (readers that check keys strictly refuse null)
+                values[key] = getattr(self, item.name)
         return values

@@ -1,7 +1,7 @@
 from .batch import CacheCell, GroupBatch, SequenceChunk, StepBatch
-from .llm_engine import EngineCore, LLMEngine, TokenEvent
+from .llm_engine import EngineCore, LLMEngine, RequestTooLongError, TokenEvent
 from .runner import ModelRunner, StepEntry, build_step_batch
-from .scheduler import IterationScheduler, RequestState, choose_victim, plan_iteration
+from .scheduler import Request, Scheduler, Share
 from .tokenizer import ByteTokenizer, FileTokenizer, Tokenizer
 
 __all__ = [
@@ -10,16 +10,16 @@ __all__ = [
     "EngineCore",
     "FileTokenizer",
     "GroupBatch",
-    "IterationScheduler",
     "LLMEngine",
     "ModelRunner",
-    "RequestState",
+    "Request",
+    "RequestTooLongError",
+    "Scheduler",
     "SequenceChunk",
+    "Share",
     "StepBatch",
     "StepEntry",
     "TokenEvent",
     "Tokenizer",
     "build_step_batch",
-    "choose_victim",
-    "plan_iteration",
 ]

@@ -10,6 +10,7 @@ callback, priority=, request_id=)`.
 from __future__ import annotations
 
 import asyncio
+import collections
 import inspect
 import time
 import uuid
@@ -23,13 +24,17 @@ from ..config.serving import CacheConfig, SchedulerConfig
 from ..sampling.sampler import GenerationConfig, Sampler
 from ..weights.loader import LoadedModel, load_model_folder
 from .runner import ModelRunner, StepEntry
-from .scheduler import IterationScheduler, RequestState, TokenCallback, choose_victim, plan_iteration
+from .scheduler import Request, Scheduler, Share, TokenCallback
 from .tokenizer import ByteTokenizer, Tokenizer
+
+
+class RequestTooLongError(ValueError):
+    """Prompt plus the tokens asked for exceed the longest sequence the cache can describe."""
 
 
 @dataclass
 class TokenEvent:
-    request: RequestState
+    request: Request
     token: int
 
 
@@ -37,8 +42,11 @@ class TokenEvent:
 class _StepInFlight:
     """A decode step that was queued before the tokens it consumes had reached the host."""
 
-    requests: list[RequestState]  # row i of `logits` is requests[i]
+    requests: list[Request]  # row i of `logits` is requests[i]
     logits: torch.Tensor
+
+
+_PHASES = ("prefill", "decode", "mixed")
 
 
 class EngineCore:
@@ -55,151 +63,168 @@ class EngineCore:
         look_ahead: bool = True,
         run_ahead: bool = True,
     ) -> None:
-        scheduler_config = scheduler_config or SchedulerConfig()
+        limits = scheduler_config or SchedulerConfig()
         if prefill_chunk_size <= 0:
             raise ValueError("prefill_chunk_size must be positive")
-        if scheduler_config.max_tokens_per_step < scheduler_config.max_batch_size:
+        if limits.max_tokens_per_step < limits.max_batch_size:
             raise ValueError("max_tokens_per_step must allow one token per active request")
-        if scheduler_config.max_batch_size > runner.cache_config.max_sequences:
+        if limits.max_batch_size > runner.cache_config.max_sequences:
             raise ValueError("max_batch_size exceeds the cache's request slots (CacheConfig.max_sequences)")
         self.runner = runner
-        self.scheduler_config = scheduler_config
-        self.scheduler = IterationScheduler(scheduler_config.max_batch_size, scheduler_config.policy, scheduler_mode)
+        self.scheduler_config = limits
+        self.scheduler = Scheduler(limits, scheduler_mode)
         self.prefill_chunk_size = prefill_chunk_size
         self.sampler = Sampler(runner.kernels)
         self.collect_iteration_metrics = collect_iteration_metrics
         self.look_ahead = look_ahead  # prepare the next decode step on the host while the device runs this one
-        self._expected: list[RequestState] | None = None  # the requests of the step that is prepared
+        self._expected: list[Request] | None = None  # the requests of the step that is prepared
         # Queue the next decode step behind the sampling of this one, its tokens passed on the device:
         # the device then never waits for the host between two steps.  A request that turns out to have
         # ended (a stop token) has a row in that step that nobody reads.
         self.run_ahead = run_ahead and look_ahead
         self._in_flight: _StepInFlight | None = None
-        self.generation_configs: dict[str, GenerationConfig] = {}
-        self.finished: list[RequestState] = []
-        self._cpu_ms = {"prefill": 0.0, "decode": 0.0, "mixed": 0.0}
-        self._counts = {"prefill": 0, "decode": 0, "mixed": 0}
-        self._events: dict[str, list] = {"prefill": [], "decode": [], "mixed": []}
-        self._completed_preemptions = 0
-        self._completed_recomputed_tokens = 0
+        self._known: set[str] = set()  # ids of requests that are waiting or running
+        self.finished: list[Request] = []
+        self._host_ms = dict.fromkeys(_PHASES, 0.0)
+        self._iterations = dict.fromkeys(_PHASES, 0)
+        self._device_spans: dict[str, list] = {phase: [] for phase in _PHASES}
+        self._evictions_of_finished = 0
+        self._replayed_by_finished = 0
         self.step_log: list[list[tuple[str, int]]] | None = None  # tests set it to [] to record every plan
 
     # ------------------------------------------------------------------ requests
 
-    def submit(self, request: RequestState, config: GenerationConfig) -> None:
-        if config.max_new_tokens <= 0:
+    def check(self, request: Request) -> None:
+        """Raises for a request that could never run, before it takes a place in the line: only
+        the offender is refused, whatever else is running."""
+        if request.settings.max_new_tokens <= 0:
             raise ValueError("max_new_tokens must be positive")
-        if not request.prompt_token_ids:
+        if not request.prompt:
             raise ValueError("prompt cannot be empty")
-        if request.request_id in self.generation_configs:
+        if min(request.prompt) < 0 or max(request.prompt) >= self.runner.vocab_size:
+            raise ValueError(f"request {request.request_id!r}: a prompt token is outside the vocabulary")
+        longest = self.runner.cache.max_sequence_length
+        if len(request.prompt) + request.settings.max_new_tokens > longest:
+            raise RequestTooLongError(
+                f"request {request.request_id!r}: {len(request.prompt)} prompt tokens and "
+                f"{request.settings.max_new_tokens} new ones exceed the longest sequence, {longest}"
+            )
+        if request.request_id in self._known:
             raise ValueError(f"request {request.request_id!r} is already running")
-        self.generation_configs[request.request_id] = config
-        self.scheduler.add(request)
+
+    def submit(self, request: Request) -> None:
+        self.check(request)
+        self._known.add(request.request_id)
+        self.scheduler.enqueue(request)
 
     @property
     def has_work(self) -> bool:
-        return not self.scheduler.empty
+        return not self.scheduler.idle
 
-    def finish(self, request: RequestState, error: Exception | None = None) -> None:
-        """`engine.py:402-415`."""
-        if request in self.scheduler.active:
-            self.scheduler.finish(request)
-        if request in self.scheduler.waiting:
-            self.scheduler.waiting.remove(request)
+    def finish(self, request: Request, error: Exception | None = None) -> None:
+        """The request leaves the engine, with its tokens or with `error`; what it holds in the
+        cache is given back (`engine.py:402-415`)."""
+        self.scheduler.retire(request)
         if self.runner.has_request(request.request_id):
             self.runner.end_request(request.request_id)
-        self.generation_configs.pop(request.request_id, None)
-        self._completed_preemptions += request.preemptions
-        self._completed_recomputed_tokens += request.recomputed_tokens
-        request.error = error
-        request.finished = True
+        self._known.discard(request.request_id)
+        self._evictions_of_finished += request.evictions
+        self._replayed_by_finished += request.replayed_tokens
+        request.error, request.done = error, True
         self.finished.append(request)
 
     def fail_all(self, error: Exception) -> None:
-        """`engine.py:417-426`."""
-        for request in list(self.scheduler.active) + list(self.scheduler.waiting):
+        """Everything running or waiting ends with `error` (`engine.py:417-426`)."""
+        for request in self.scheduler.running + self.scheduler.waiting:
             self.finish(request, error)
 
     # ------------------------------------------------------------------ one iteration
 
     @staticmethod
-    def _phase(active: list[RequestState]) -> str:
-        prefill = any(request.in_prefill for request in active)
-        decode = any(not request.in_prefill for request in active)
-        return "mixed" if prefill and decode else "prefill" if prefill else "decode"
+    def _phase(batch: list[Request]) -> str:
+        kinds = {request.in_prompt for request in batch}
+        return "mixed" if len(kinds) == 2 else "prefill" if True in kinds else "decode"
 
     def step(self) -> list[TokenEvent]:
         """Admits, plans, makes room, runs one batch, samples (`engine.py:234-346`).
         Returns the tokens generated in this iteration."""
         for request in self.scheduler.admit():
             self.runner.add_request(request.request_id)
-        active = list(self.scheduler.active)
-        if not active:
+        batch = list(self.scheduler.running)
+        if not batch:
             return []
-        phase = self._phase(active)
+        if not self.collect_iteration_metrics:
+            return self._run_iteration(batch)
+        phase = self._phase(batch)
+        on_device = self.runner.device.type == "cuda"
+        began = torch.cuda.Event(enable_timing=True) if on_device else None
+        if began is not None:
+            began.record()
         started = time.perf_counter()
-        events = None
-        if self.collect_iteration_metrics and self.runner.device.type == "cuda":
-            events = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-            events[0].record()
         try:
-            return self._run_iteration(active)
+            return self._run_iteration(batch)
         finally:
-            if self.collect_iteration_metrics:
-                self._cpu_ms[phase] += (time.perf_counter() - started) * 1000
-                self._counts[phase] += 1
-                if events is not None:
-                    events[1].record()
-                    self._events[phase].append(events)
+            self._host_ms[phase] += 1000.0 * (time.perf_counter() - started)
+            self._iterations[phase] += 1
+            if began is not None:
+                ended = torch.cuda.Event(enable_timing=True)
+                ended.record()
+                self._device_spans[phase].append((began, ended))
 
-    def _run_iteration(self, active: list[RequestState]) -> list[TokenEvent]:
+    def _no_arrival_can_join(self, staying: list[Request]) -> bool:
+        """Whether the next step's batch is certain to be `staying` unless a stop token comes: nobody
+        waits, or nobody can be admitted (the batch stays full; a static batch is not empty)."""
+        scheduler = self.scheduler
+        if scheduler.num_waiting == 0:
+            return True
+        if scheduler.mode == "static":
+            return bool(staying)
+        return len(staying) == len(scheduler.running) == scheduler.limits.max_batch_size
+
+    def _run_iteration(self, batch: list[Request]) -> list[TokenEvent]:
         in_flight, self._in_flight = self._in_flight, None
-        if in_flight is not None and any(not request.finished for request in in_flight.requests):
+        if in_flight is not None and any(not request.done for request in in_flight.requests):
             # this iteration's step runs already: its requests each brought the token they had just been given
             rows = in_flight.requests
             logits = in_flight.logits
-            planned = [(request, 1) for request in rows if not request.finished]
+            shares = [Share(request, 1) for request in rows if not request.done]
             if self.step_log is not None:
-                self.step_log.append([(request.request_id, 1) for request, _ in planned])
+                self.step_log.append([(request.request_id, 1) for request, _ in shares])
         else:
             expected, self._expected = self._expected, None
-            if expected is not None and len(expected) == len(active) and all(a is b for a, b in zip(expected, active)):
+            if expected is not None and len(expected) == len(batch) and all(a is b for a, b in zip(expected, batch)):
                 # the step that was prepared while the last one ran: every request brings the token it
                 # has just been given, and the runner holds the cache entries already
-                planned = [(request, 1) for request in active]
+                shares = [Share(request, 1) for request in batch]
             else:
-                planned = self._plan(active)
-                if planned is None:
+                shares = self._plan()
+                if not shares:
                     return []
             if self.step_log is not None:
-                self.step_log.append([(request.request_id, count) for request, count in planned])
-
+                self.step_log.append([(request.request_id, count) for request, count in shares])
             entries, rows = [], []
-            for request, count in planned:
-                tokens = request.tokens_between(request.processed_tokens, request.processed_tokens + count)
-                last = request.processed_tokens + count == len(request.prompt_token_ids) + len(request.generated_token_ids)
-                entries.append(StepEntry(request.request_id, tokens, (count - 1,) if last else ()))
-                if last:  # otherwise: a portion of a prompt, or a replay after preemption
+            for request, count in shares:
+                catches_up = count == request.owed  # else: a portion of a prompt, or of a replay after giving way
+                entries.append(StepEntry(request.request_id, request.next_tokens(count), (count - 1,) if catches_up else ()))
+                if catches_up:
                     rows.append(request)
             logits = self.runner.step(entries, fits_checked=True)
-        for request, count in planned:
-            request.processed_tokens += count
-        sampled = [request for request in rows if not request.finished]
-        if not sampled:
+        for request, count in shares:
+            request.cached += count
+        if all(request.done for request in rows):
             return []
-        greedy = GenerationConfig()
-        configs = [self.generation_configs.get(request.request_id, greedy) for request in rows]
-        steps = [len(request.generated_token_ids) for request in rows]
+        settings = [request.settings for request in rows]
+        draws = [len(request.output) for request in rows]
         tokens = None
-        if self.look_ahead and len(sampled) == len(rows) == len(planned) == len(active) and not self.scheduler.waiting:
-            # Every running request has just decoded and nothing waits: unless a stop token comes,
-            # the next step is these requests again, less those at their last token.  The runner does
-            # its host work for that step now, while the device is still busy with this one.
-            staying = [r for r in sampled if len(r.generated_token_ids) + 1 < r.max_new_tokens]
-            if self.runner.prepare_decode([r.request_id for r in staying]):
+        if self.look_ahead and len(rows) == len(shares) == len(batch) and not any(request.done for request in rows):
+            # Every running request has just decoded: unless a stop token comes, the next step is these
+            # requests again, less those at their last token.  The runner does its host work for that
+            # step now, while the device is still busy with this one.
+            staying = [request for request in rows if request.output_left > 1]
+            if self._no_arrival_can_join(staying) and self.runner.prepare_decode([r.request_id for r in staying]):
                 if self.run_ahead and len(staying) == len(rows):
                     # and queues it: the tokens go from the sampler to the step on the device
-                    chosen = self.sampler.sample_on_device(logits, configs, steps)
+                    chosen = self.sampler.sample_on_device(logits, settings, draws)
                     fetch = self.runner.fetch_later(chosen)
                     next_logits = self.runner.step_from_device([r.request_id for r in staying], chosen)
                     self._in_flight = _StepInFlight(staying, next_logits)
@@ -207,34 +232,40 @@ class EngineCore:
                 else:
                     self._expected = staying
         if tokens is None:
-            tokens = self.sampler.sample(logits, configs, steps)
+            tokens = self.sampler.sample(logits, settings, draws)
         produced = []
-        for request, config, token in zip(rows, configs, tokens):
-            if request.finished:  # a row of a step queued before its request's end was known
+        for request, token in zip(rows, tokens):
+            if request.done:  # a row of a step queued before its request's end was known
                 continue
-            request.generated_token_ids.append(token)
+            request.output.append(token)
             produced.append(TokenEvent(request, token))
-            if len(request.generated_token_ids) >= request.max_new_tokens or token in config.stop_token_ids:
+            if request.output_left <= 0 or token in request.settings.stop_token_ids:
                 self.finish(request)
         return produced
 
-    def _plan(self, active: list[RequestState]) -> list[tuple[RequestState, int]] | None:
-        """Who brings how many tokens to this step; requests give way until it fits the cache."""
-        planned = plan_iteration(active, self.scheduler_config.max_tokens_per_step, self.prefill_chunk_size)
+    def _plan(self) -> list[Share]:
+        """Who brings how many tokens to this step.  A request that has outgrown the longest sequence
+        ends alone, with an error of its own; when pages run out, requests give way (never the
+        oldest) until the rest fits, and one that cannot fit even alone fails with `CacheFullError`."""
+        shares = self.scheduler.plan(self.prefill_chunk_size)
+        longest = self.runner.cache.max_sequence_length
+        for request, count in shares:
+            if request.cached + count > longest:  # `check` keeps such requests out; nobody else pays for one
+                self.finish(request, RequestTooLongError(f"request {request.request_id!r} exceeds the longest sequence, {longest}"))
+        shares = [share for share in shares if not share.request.done]
 
-        def as_plan(items):
-            return [(request.request_id, count) for request, count in items]
+        def fits() -> bool:
+            return self.runner.fits([(request.request_id, count) for request, count in shares])
 
-        # Pages run out: requests give way (never the oldest) until the rest fits.
-        while not self.runner.fits(as_plan(planned)) and len(planned) > 1:
-            victim = choose_victim(planned, self.scheduler_config.preemption)
+        while len(shares) > 1 and not fits():
+            victim = self.scheduler.victim(shares)
             self.runner.end_request(victim.request_id)
-            self.scheduler.preempt(victim)
-            planned = [item for item in planned if item[0] is not victim]
-        if not self.runner.fits(as_plan(planned)):
-            self.finish(planned[0][0], CacheFullError("one sequence exceeds total KV cache capacity"))
-            return None
-        return planned
+            self.scheduler.evict(victim)
+            shares = [share for share in shares if share.request is not victim]
+        if shares and not fits():
+            self.finish(shares[0].request, CacheFullError("one sequence exceeds total KV cache capacity"))
+            return []
+        return shares
 
     # ------------------------------------------------------------------ synchronous use
 
@@ -247,18 +278,16 @@ class EngineCore:
         """Runs the given prompts to completion and returns their generated tokens in order."""
         if configs is None or isinstance(configs, GenerationConfig):
             configs = [configs or GenerationConfig()] * len(prompts)
-        requests = []
-        for index, (prompt, config) in enumerate(zip(prompts, configs)):
-            request_id = request_ids[index] if request_ids else f"request-{index:06d}"
-            request = RequestState(request_id, list(prompt), config.max_new_tokens)
-            self.submit(request, config)
-            requests.append(request)
+        names = request_ids or [f"request-{index:06d}" for index in range(len(prompts))]
+        requests = [Request(name, list(prompt), config) for name, prompt, config in zip(names, prompts, configs)]
+        for request in requests:
+            self.submit(request)
         while self.has_work:
             self.step()
-        for request in requests:
-            if request.error is not None:
-                raise request.error
-        return [request.generated_token_ids for request in requests]
+        failed = next((request for request in requests if request.error is not None), None)
+        if failed is not None:
+            raise failed.error
+        return [request.output for request in requests]
 
     # ------------------------------------------------------------------ accounting
 
@@ -268,29 +297,29 @@ class EngineCore:
 
     @property
     def iteration_stats(self) -> dict[str, float | int]:
-        """`engine.py:438-458`."""
-        device_ms = {phase: 0.0 for phase in self._events}
-        if self.collect_iteration_metrics and self.runner.device.type == "cuda":
-            torch.cuda.synchronize(self.runner.device)
-            device_ms = {
-                phase: sum(start.elapsed_time(end) for start, end in pairs) for phase, pairs in self._events.items()
-            }
-        result: dict[str, float | int] = {
-            "preemptions": self._completed_preemptions,
-            "recomputed_tokens": self._completed_recomputed_tokens,
+        """The reference's keys (`engine.py:438-458`): iterations and host and device time by kind of
+        iteration, what packing the steps' index arrays cost, and the evictions of finished requests."""
+        stats: dict[str, float | int] = {
+            "metadata_construction_ms": self.runner.packing_ms,
+            "preemptions": self._evictions_of_finished,
+            "recomputed_tokens": self._replayed_by_finished,
         }
-        for phase in ("prefill", "decode", "mixed"):
-            result[f"{phase}_iterations"] = self._counts[phase]
-            result[f"{phase}_cpu_ms"] = self._cpu_ms[phase]
-            result[f"{phase}_cuda_ms"] = device_ms[phase]
-        return result
+        if any(self._device_spans.values()):
+            torch.cuda.synchronize(self.runner.device)
+        for phase in _PHASES:
+            stats[f"{phase}_iterations"] = self._iterations[phase]
+            stats[f"{phase}_cpu_ms"] = self._host_ms[phase]
+            stats[f"{phase}_cuda_ms"] = sum(began.elapsed_time(ended) for began, ended in self._device_spans[phase])
+        return stats
 
 
 class LLMEngine:
-    """Asynchronous iteration-level engine (`engine.py:108-242`).
+    """The asynchronous entry point, with the reference's signature (`engine.py:108-242`).
 
     `model` is a model folder, or what `load_model_folder` returned.  `kernels`
     is the kernel library; by default the HIP library for `dtype` on `device`.
+    Requests go into an inbox; one task serves them, an iteration at a time, and
+    sleeps on an event while there is nothing to do.
     """
 
     def __init__(
@@ -307,17 +336,9 @@ class LLMEngine:
         dtype: torch.dtype | str = torch.bfloat16,
         kernels: Any = None,
         max_sequence_length: int | None = None,
-        paged_attention_backend: str = "hip",
-        cache_device_metadata: bool = True,
     ) -> None:
-        """`paged_attention_backend` and `cache_device_metadata` are the reference's switches between its own
-        back ends (`engine.py:111-125`), taken so that its calls carry over: there is one attention path here
-        (the reference's names "pytorch" and "triton" are read as it), and a step's index arrays are packed
-        anew for every step whatever the second says."""
         from ..weights.loader import run_dtype
 
-        if paged_attention_backend not in ("hip", "pytorch", "triton"):
-            raise ValueError(f"unknown paged_attention_backend {paged_attention_backend!r}")
         dtype = run_dtype(dtype)
         if not isinstance(model, LoadedModel):
             model = load_model_folder(model, dtype)
@@ -337,13 +358,14 @@ class LLMEngine:
             collect_iteration_metrics=collect_iteration_metrics,
         )
         self.device = self.runner.device
-        self._incoming: asyncio.Queue[RequestState] = asyncio.Queue()
-        self._worker: asyncio.Task | None = None
+        self._inbox: collections.deque[Request] = collections.deque()
+        self._wake = asyncio.Event()
+        self._server: asyncio.Task | None = None
         self._closed = False
-        self._pending_configs: dict[str, GenerationConfig] = {}
+        self._facts: dict[str, dict[str, float | int | None]] = {}
 
     @property
-    def scheduler(self) -> IterationScheduler:
+    def scheduler(self) -> Scheduler:
         return self.core.scheduler
 
     @property
@@ -359,77 +381,78 @@ class LLMEngine:
         priority: int = 0,
         request_id: str | None = None,
     ) -> list[int]:
-        """`engine.py:188-221`."""
-        config = config or GenerationConfig()
+        """Generates for one prompt (text, or token ids) and returns the new tokens; `callback` gets
+        each as it is produced.  A request that can never run is refused here, with `ValueError`."""
         if self._closed:
             raise RuntimeError("engine is closed")
-        if config.max_new_tokens <= 0:
-            raise ValueError("max_new_tokens must be positive")
-        if self._worker is None:
-            self._worker = asyncio.create_task(self._run())
-        prompt_tokens = self.tokenizer.encode(prompt) if isinstance(prompt, str) else list(prompt)
-        if not prompt_tokens:
-            raise ValueError("prompt cannot be empty")
-        request_id = request_id or str(uuid.uuid4())
-        future = asyncio.get_running_loop().create_future()
-        state = RequestState(
-            request_id=request_id,
-            prompt_token_ids=prompt_tokens,
-            max_new_tokens=config.max_new_tokens,
-            callback=callback,
-            priority=priority,
-            future=future,
-        )
-        self._pending_configs[request_id] = config
-        await self._incoming.put(state)
-        return await future
+        tokens = self.tokenizer.encode(prompt) if isinstance(prompt, str) else list(prompt)
+        request = Request(request_id or uuid.uuid4().hex, tokens, config or GenerationConfig(), priority, callback)
+        self.core.check(request)
+        request.outcome = asyncio.get_running_loop().create_future()
+        self._inbox.append(request)
+        self._wake.set()
+        if self._server is None:
+            self._server = asyncio.create_task(self._serve())
+        return await request.outcome
 
-    def _take(self, request: RequestState) -> None:
-        try:
-            self.core.submit(request, self._pending_configs.pop(request.request_id))
-        except Exception as error:
-            if request.future and not request.future.done():
-                request.future.set_exception(error)
+    def request_facts(self, request_id: str) -> dict[str, float | int | None]:
+        """What the engine knows about a finished request beside its tokens: when it was first
+        admitted (monotonic seconds), how often it gave way and how many tokens that cost.  Kept until asked for."""
+        return self._facts.pop(request_id, {})
 
-    async def _run(self) -> None:
-        """`engine.py:223-242`."""
-        try:
-            while not self._closed:
-                if not self.core.has_work:
-                    self._take(await self._incoming.get())
-                while True:
-                    try:
-                        self._take(self._incoming.get_nowait())
-                    except asyncio.QueueEmpty:
-                        break
-                events = self.core.step()
-                for event in events:
-                    if event.request.callback:
-                        result = event.request.callback(event.token)
-                        if inspect.isawaitable(result):
-                            await result
-                self._resolve()
-                await asyncio.sleep(0)
-        except asyncio.CancelledError:
-            pass
-        except Exception as error:
-            self.core.fail_all(error)
-            self._resolve()
-
-    def _resolve(self) -> None:
+    def _settle(self) -> None:
+        """Hands every finished request's tokens, or its error, to whoever awaits it."""
         for request in self.core.finished:
-            if request.future and not request.future.done():
-                if request.error is not None:
-                    request.future.set_exception(request.error)
-                else:
-                    request.future.set_result(request.generated_token_ids)
+            self._facts[request.request_id] = {
+                "admitted_s": request.admitted_at,
+                "preemptions": request.evictions,
+                "recomputed_tokens": request.replayed_tokens,
+            }
+            waiter = request.outcome
+            if waiter is None or waiter.done():
+                continue
+            if request.error is None:
+                waiter.set_result(request.output)
+            else:
+                waiter.set_exception(request.error)
         self.core.finished.clear()
+
+    async def _serve(self) -> None:
+        try:
+            while True:
+                while self._inbox:
+                    request = self._inbox.popleft()
+                    try:
+                        self.core.submit(request)
+                    except Exception as error:  # e.g. an id that is in use: only this request fails
+                        request.outcome.set_exception(error)
+                if not self.core.has_work:
+                    self._wake.clear()
+                    await self._wake.wait()
+                    continue
+                for event in self.core.step():
+                    notify = event.request.on_token
+                    if notify is not None:
+                        pending = notify(event.token)
+                        if inspect.isawaitable(pending):
+                            await pending
+                self._settle()
+                await asyncio.sleep(0)  # callers run: new requests arrive, tokens are consumed
+        except asyncio.CancelledError:
+            raise
+        except Exception as error:  # the step function failed: nobody can go on
+            for request in self._inbox:
+                request.outcome.set_exception(error)
+            self._inbox.clear()
+            self.core.fail_all(error)
+            self._settle()
 
     async def close(self) -> None:
         self._closed = True
-        if self._worker:
-            self._worker.cancel()
-            await asyncio.gather(self._worker, return_exceptions=True)
+        server, self._server = self._server, None
+        if server is not None:
+            server.cancel()
+            await asyncio.gather(server, return_exceptions=True)
 
     @property
     def cache_stats(self) -> dict[str, float]:

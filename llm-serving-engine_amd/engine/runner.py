@@ -11,6 +11,7 @@ counterpart is the second half of `LLMEngine._step` plus
 from __future__ import annotations
 
 import contextlib
+import time
 from dataclasses import dataclass, field
 from typing import Any
 
@@ -180,7 +181,9 @@ class ModelRunner:
         self.vocab_size = loaded.spec.vocab_size
         self.use_graphs = self.device.type == "cuda" if use_graphs is None else use_graphs
         self.use_graphs = self.use_graphs and self.model.replayable  # a part that looks at values on the host is not replayed
-        self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self._graphs: dict[tuple[int, int], _DecodeGraph] = {}  # in order of last use, the latest last
+        self.max_graphs = 24  # each holds only a step's activations
+        self.packing_ms = 0.0  # host time spent on the steps' index arrays
         # What `prepare_decode` has done for the step to come: each request's reservation of one
         # token, and, where decode steps replay a graph, the step's index arrays already packed.
         self._ahead: dict[str, Reservation] = {}
@@ -330,7 +333,9 @@ class ModelRunner:
             if packed_ahead is not None and packed_ahead[0] == tuple(entry.request_id for entry in entries):
                 return self._decode_with_graph(reservations, entries, packed_ahead[1:])
             return self._decode_with_graph(reservations, entries)
+        started = time.perf_counter()
         batch = build_step_batch(reservations, entries, self.cache, self.device)
+        self.packing_ms += 1000.0 * (time.perf_counter() - started)
         return self.forward(batch)
 
     def _stream_scope(self):
@@ -356,10 +361,13 @@ class ModelRunner:
 
     def _pack_decode(self, reservations: list[Reservation], entries: list[StepEntry]):
         """The index arrays of a step of single tokens, padded to its graph's shape; first the graph's key."""
+        started = time.perf_counter()
         requests = self._bucket(len(reservations))
         blocks = max(-(-(r.start + 1) // self.cache.page_size) for r in reservations)
         width = min(self._bucket(blocks), self._bucket(self.cache.max_blocks_per_sequence))
-        return ((requests, width), *_pack_step(reservations, entries, self.cache, pad_to=requests, width=width))
+        packed = _pack_step(reservations, entries, self.cache, pad_to=requests, width=width)
+        self.packing_ms += 1000.0 * (time.perf_counter() - started)
+        return ((requests, width), *packed)
 
     @torch.inference_mode()
     def _decode_with_graph(
@@ -378,9 +386,10 @@ class ModelRunner:
                 packed[: len(entries)] = [entry.tokens[0] for entry in entries]
         else:
             key, packed, sizes, widths, facts = self._pack_decode(reservations, entries)
-        graph = self._graphs.get(key)
+        graph = self._graphs.pop(key, None)
         if graph is None:
             graph = self._capture(key, packed, sizes, widths, facts)
+        self._graphs[key] = graph  # the one used last stands last
         turn = graph.turn
         graph.turn = 1 - turn
         if graph.copied[turn] is not None:
@@ -397,7 +406,10 @@ class ModelRunner:
 
     def _capture(self, key, packed, sizes, widths, facts) -> _DecodeGraph:
         requests, width = key
-        if len(self._graphs) >= 24:  # keep the newest; each holds only a step's activations
+        if len(self._graphs) >= self.max_graphs:
+            # The graph that was used longest ago goes.  A replay of it may still be queued (a step that was
+            # queued ahead), and its kernels read the buffers it owns: the device finishes first.
+            torch.cuda.synchronize(self.device)
             self._graphs.pop(next(iter(self._graphs)))
         static = torch.from_numpy(packed).to(self.device)
         chunks = [SequenceChunk(f"#{index}", 0, 0, 1) for index in range(requests)]
@@ -415,6 +427,4 @@ class ModelRunner:
         with torch.cuda.graph(captured), self._stream_scope():
             logits = self.model.forward(batch, self.cells)
         host = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
-        graph = _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)
-        self._graphs[key] = graph
-        return graph
+        return _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)

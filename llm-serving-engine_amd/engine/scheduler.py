@@ -1,167 +1,208 @@
-"""Iteration-level scheduling: who is admitted, how many tokens each request
-brings to a step, and who gives way when the cache is full.
+"""Iteration-level scheduling: who runs, how many tokens each request brings to a
+step, and who gives way when the cache is full.
 
-Queues, policies and admission follow the reference's `IterationScheduler`
-(`scheduler.py:40-97`); the step plan and the victim choice follow its engine
-(`engine.py:255-267,372-400`).  They sit together here because both are
-decisions, made on the host, that the tests check without a model.
+The behaviour is the reference's (`scheduler.py:40-97` for queues, policies and
+admission; `engine.py:255-267,372-400` for the step plan and the choice of a
+victim): first-come, shortest-job or priority order, admission every iteration
+or only into an empty batch, one token for everybody and then prompt portions
+while the step's budget lasts.  The structures are this engine's own: a request
+carries its generation settings, the line of waiting requests is a heap keyed
+by the policy, and planning and the victim rule are the scheduler's methods,
+so every decision the tests check without a model sits in one object.
 """
 
 from __future__ import annotations
 
-import itertools
+import heapq
 import time
 from collections.abc import Awaitable, Callable
 from dataclasses import dataclass, field
-from typing import Any
+from typing import Any, NamedTuple
+
+from ..config.serving import SchedulerConfig
+from ..sampling.sampler import GenerationConfig
 
 TokenCallback = Callable[[int], Awaitable[None] | None]
 
 
-@dataclass
-class RequestState:
-    """`scheduler.py:12-37`."""
+@dataclass(eq=False)
+class Request:
+    """One request from its arrival to its last token.
+
+    `cached` counts the tokens of prompt + output whose keys and values the
+    cache holds; what is still `owed` to the model is the rest.  A request that
+    gave way starts again at `cached = 0` and replays prompt and output without
+    emitting anything until it has caught up.
+    """
 
     request_id: str
-    prompt_token_ids: list[int]
-    max_new_tokens: int
-    callback: TokenCallback | None = None
+    prompt: list[int]
+    settings: GenerationConfig = field(default_factory=GenerationConfig)
     priority: int = 0
-    arrival_order: int = 0
-    arrival_time: float = field(default_factory=time.monotonic)
-    generated_token_ids: list[int] = field(default_factory=list)
-    processed_tokens: int = 0
-    preemptions: int = 0
-    recomputed_tokens: int = 0
-    future: Any = None
+    on_token: TokenCallback | None = None
+    output: list[int] = field(default_factory=list)
+    cached: int = 0
+    ticket: int = -1  # arrival number, given by the scheduler; ties in every policy go to the lower
+    arrived_at: float = field(default_factory=time.monotonic)
+    admitted_at: float | None = None  # first admission
+    evictions: int = 0  # times it gave way
+    replayed_tokens: int = 0  # tokens computed again because of that
+    outcome: Any = None  # a future, for the asynchronous entry point
     error: Exception | None = None
-    finished: bool = False
+    done: bool = False
 
     @property
-    def all_tokens(self) -> list[int]:
-        return self.prompt_token_ids + self.generated_token_ids
-
-    def tokens_between(self, start: int, end: int) -> list[int]:
-        """all_tokens[start:end] without joining the two lists (a decode step asks for one token)."""
-        prompt = len(self.prompt_token_ids)
-        if start >= prompt:
-            return self.generated_token_ids[start - prompt : end - prompt]
-        if end <= prompt:
-            return self.prompt_token_ids[start:end]
-        return self.prompt_token_ids[start:] + self.generated_token_ids[: end - prompt]
+    def length(self) -> int:
+        return len(self.prompt) + len(self.output)
 
     @property
-    def remaining_input_tokens(self) -> int:
-        return len(self.prompt_token_ids) + len(self.generated_token_ids) - self.processed_tokens
+    def owed(self) -> int:
+        return self.length - self.cached
 
     @property
-    def remaining_output_tokens(self) -> int:
-        return self.max_new_tokens - len(self.generated_token_ids)
+    def output_left(self) -> int:
+        return self.settings.max_new_tokens - len(self.output)
 
     @property
-    def in_prefill(self) -> bool:
-        return self.processed_tokens < len(self.prompt_token_ids)
+    def in_prompt(self) -> bool:
+        return self.cached < len(self.prompt)
+
+    def next_tokens(self, count: int) -> list[int]:
+        """The `count` tokens after the cached ones (a decode step asks for one: no list is joined for it)."""
+        first, last, border = self.cached, self.cached + count, len(self.prompt)
+        if first >= border:
+            return self.output[first - border : last - border]
+        if last <= border:
+            return self.prompt[first:last]
+        return self.prompt[first:] + self.output[: last - border]
 
 
-class IterationScheduler:
-    """Waiting and active lists with first-come, shortest-job or priority order,
-    admitting every iteration (continuous) or only into an empty batch (static)."""
+class Share(NamedTuple):
+    """A request's share of one step."""
 
-    def __init__(self, max_batch_size: int, policy: str = "fcfs", mode: str = "continuous") -> None:
-        if policy not in {"fcfs", "sjf", "priority"}:
-            raise ValueError("policy must be fcfs, sjf, or priority")
-        if mode not in {"continuous", "static"}:
+    request: Request
+    count: int
+
+
+_ORDERINGS: dict[str, Callable[[Request], tuple]] = {
+    "fcfs": lambda request: (request.ticket,),
+    "sjf": lambda request: (request.output_left, request.ticket),
+    "priority": lambda request: (-request.priority, request.ticket),
+}
+
+
+class Scheduler:
+    """The line of waiting requests and the running batch.
+
+    A request's place in the line is fixed when it joins it (its key cannot
+    change while it waits: output is produced only while running), so the line
+    is a heap and admission pops its head.  A request that gives way rejoins
+    with its old ticket: under first-come order it is the next to be admitted.
+    """
+
+    def __init__(self, limits: SchedulerConfig | None = None, mode: str = "continuous") -> None:
+        self.limits = limits or SchedulerConfig()
+        if self.limits.policy not in _ORDERINGS:
+            raise ValueError(f"policy must be one of {', '.join(_ORDERINGS)}")
+        if mode not in ("continuous", "static"):
             raise ValueError("mode must be continuous or static")
-        if max_batch_size <= 0:
+        if self.limits.max_batch_size <= 0:
             raise ValueError("max_batch_size must be positive")
-        self.max_batch_size = max_batch_size
-        self.policy = policy
+        if self.limits.preemption not in ("largest", "latest"):
+            raise ValueError("preemption must be largest or latest")
         self.mode = mode
-        self.waiting: list[RequestState] = []
-        self.active: list[RequestState] = []
-        self._counter = itertools.count()
+        self.running: list[Request] = []
+        self._line: list[tuple[tuple, Request]] = []
+        self._key = _ORDERINGS[self.limits.policy]
+        self._tickets = 0
 
-    def add(self, request: RequestState) -> None:
-        request.arrival_order = next(self._counter)
-        self.waiting.append(request)
+    # ------------------------------------------------------------------ the line
 
-    def _order(self, request: RequestState):
-        if self.policy == "fcfs":
-            return (request.arrival_order,)
-        if self.policy == "sjf":
-            return (request.remaining_output_tokens, request.arrival_order)
-        return (-request.priority, request.arrival_order)
+    def enqueue(self, request: Request) -> None:
+        request.ticket = self._tickets
+        self._tickets += 1
+        heapq.heappush(self._line, (self._key(request), request))
 
-    def admit(self) -> list[RequestState]:
-        """`scheduler.py:75-83`: no memory check here; pages are found, or a
-        request gives way, when the step is planned."""
-        if self.mode == "static" and self.active:
+    @property
+    def waiting(self) -> list[Request]:
+        """The line in the order in which it would be admitted."""
+        return [request for _, request in sorted(self._line, key=lambda item: item[0])]
+
+    @property
+    def num_waiting(self) -> int:
+        return len(self._line)
+
+    @property
+    def idle(self) -> bool:
+        return not self._line and not self.running
+
+    def admit(self) -> list[Request]:
+        """Moves requests from the head of the line into the batch: every iteration while
+        there is room (continuous), or only into an empty batch (static).  Memory is not
+        asked about here (`scheduler.py:75-83`): pages are found, or somebody gives way,
+        when the step is planned."""
+        if self.mode == "static" and self.running:
             return []
-        self.waiting.sort(key=self._order)
-        count = min(self.max_batch_size - len(self.active), len(self.waiting))
-        admitted = self.waiting[:count]
-        del self.waiting[:count]
-        self.active.extend(admitted)
+        admitted = []
+        now = time.monotonic()
+        while self._line and len(self.running) < self.limits.max_batch_size:
+            _, request = heapq.heappop(self._line)
+            if request.admitted_at is None:
+                request.admitted_at = now
+            self.running.append(request)
+            admitted.append(request)
         return admitted
 
-    def finish(self, request: RequestState) -> None:
-        self.active.remove(request)
+    def retire(self, request: Request) -> None:
+        """Takes the request out of the batch, or out of the line."""
+        if request in self.running:
+            self.running.remove(request)
+        else:
+            remaining = [item for item in self._line if item[1] is not request]
+            if len(remaining) != len(self._line):
+                self._line = remaining
+                heapq.heapify(self._line)
 
-    def preempt(self, request: RequestState) -> None:
-        """`scheduler.py:88-93`: back to the waiting list with its arrival order
-        kept; everything it had processed will be computed again."""
-        self.active.remove(request)
-        request.recomputed_tokens += request.processed_tokens
-        request.processed_tokens = 0
-        request.preemptions += 1
-        self.waiting.append(request)
+    def evict(self, request: Request) -> None:
+        """The request gives way: back into the line, everything it had cached to be
+        computed again (`scheduler.py:88-93`)."""
+        self.running.remove(request)
+        request.replayed_tokens += request.cached
+        request.cached = 0
+        request.evictions += 1
+        heapq.heappush(self._line, (self._key(request), request))
 
-    @property
-    def empty(self) -> bool:
-        return not self.waiting and not self.active
+    # ------------------------------------------------------------------ one step
 
+    def plan(self, chunk: int) -> list[Share]:
+        """Everybody in the batch brings one token; what the step's budget then has left
+        goes, in batch order, to requests that owe more, up to `chunk` tokens each
+        (`engine.py:372-391`).  A decoding request owes one token and stays at one."""
+        spare = self.limits.max_tokens_per_step - len(self.running)
+        shares = []
+        for request in self.running:
+            if request.owed <= 0:
+                raise RuntimeError(f"request {request.request_id!r} is in the batch and owes no token")
+            more = min(max(spare, 0), min(chunk, request.owed) - 1)
+            spare -= more
+            shares.append(Share(request, 1 + more))
+        return shares
 
-def plan_iteration(
-    active: list[RequestState], max_tokens_per_step: int, prefill_chunk_size: int
-) -> list[tuple[RequestState, int]]:
-    """Every active request gets one token; what is left of the step's budget
-    then tops requests up, in order, to `prefill_chunk_size` tokens or to what
-    they still have to process (`engine.py:372-391`).  A decoding request has one
-    token left and stays at one."""
-    budget = max_tokens_per_step
-    planned: list[tuple[RequestState, int]] = []
-    for request in active:
-        if request.remaining_input_tokens <= 0:
-            raise RuntimeError("active request has no input token to process")
-        planned.append((request, 1))
-        budget -= 1
-    for index, (request, count) in enumerate(planned):
-        if budget <= 0:
-            break
-        desired = min(prefill_chunk_size, request.remaining_input_tokens)
-        extra = min(desired - count, budget)
-        planned[index] = (request, count + extra)
-        budget -= extra
-    return planned
+    def victim(self, shares: list[Share]) -> Request:
+        """Who gives way when the step's pages do not fit.
 
-
-def choose_victim(planned: list[tuple[RequestState, int]], policy: str = "largest") -> RequestState:
-    """Who gives way when the step's pages do not fit.
-
-    "largest": the planned request that has processed most tokens
-    (`engine.py:258`): it frees most pages, at the price of most recomputation.
-    "latest": the one that arrived last.  Under both the request that arrived
-    first never gives way.  The reference has no such exemption, and with its
-    rule two requests that cannot both fit may evict each other for ever, each
-    overtaking the other while it replays; with the exemption the oldest
-    request always finishes, then the next oldest.
-    """
-    if policy not in ("largest", "latest"):
-        raise ValueError("preemption must be largest or latest")
-    oldest = min(planned, key=lambda item: item[0].arrival_order)[0]
-    candidates = [item[0] for item in planned if item[0] is not oldest]
-    if not candidates:
-        raise ValueError("a single request cannot give way to itself")
-    if policy == "largest":
-        return max(candidates, key=lambda request: request.processed_tokens)
-    return max(candidates, key=lambda request: request.arrival_order)
+        "largest": the one with most tokens cached (`engine.py:258`): it frees most
+        pages, at the price of most recomputation.  "latest": the one that arrived
+        last.  Under both, the request that arrived first never gives way.  The
+        reference has no such exemption, and with its rule two requests that cannot
+        both fit may evict each other for ever, each overtaking the other while it
+        replays; with the exemption the oldest always finishes, then the next oldest.
+        """
+        requests = [share.request for share in shares]
+        eldest = min(requests, key=lambda request: request.ticket)
+        others = [request for request in requests if request is not eldest]
+        if not others:
+            raise ValueError("a single request cannot give way to itself")
+        if self.limits.preemption == "largest":
+            return max(others, key=lambda request: (request.cached, -request.ticket))
+        return max(others, key=lambda request: request.ticket)

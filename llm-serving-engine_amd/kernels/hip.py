@@ -60,6 +60,7 @@ _SIGNATURES = {
     "llmserve_attention_portions": "pippppippiiiiifip",
     "llmserve_attention_can_fuse": "i",
     "llmserve_argmax": "ppppiip",
+    "llmserve_argmax_static": "ppiip",
     "llmserve_sample": "ppppppiip",
 }
 _TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}

@@ -70,7 +70,10 @@ def run_dtype(name: Any) -> torch.dtype:
 
 
 def read_config(folder: str | Path) -> tuple[Architecture, ArchitectureConfig]:
-    path = Path(folder) / "config.json"
+    """The architecture and typed configuration of a model folder, or of a config.json given by its path."""
+    path = Path(folder)
+    if path.is_dir():
+        path = path / "config.json"
     if not path.is_file():
         raise FileNotFoundError(f"no config.json under {folder}")
     values = json.loads(path.read_text())

@@ -10,7 +10,8 @@ from llmserve_amd.benchmark import (
     BenchmarkHarness, BenchmarkReport, LengthDistribution, LoadProfile, RequestMetrics, generate_workload, percentile,
 )
 from llmserve_amd.cli import ROOT, build_parser
-from llmserve_amd.engine import RequestState, choose_victim
+from llmserve_amd import GenerationConfig, SchedulerConfig
+from llmserve_amd.engine import Request, Scheduler, Share
 from llmserve_amd.engine.tokenizer import ByteTokenizer
 
 
@@ -26,17 +27,10 @@ def test_benchmark_options_are_the_references():
         build_parser().parse_args(["benchmark", "--policy", "random"])
     with pytest.raises(SystemExit):
         build_parser().parse_args(["serve"])  # servers are outside this engine
-    # the reference's switches between its back ends (cli.py:263-271) parse, so its command lines carry over
-    carried = build_parser().parse_args(["benchmark", "--rebuild-device-metadata", "--paged-attention-backend", "triton",
-                                         "--linear-backend", "fp16"])
-    assert carried.rebuild_device_metadata and carried.paged_attention_backend == "triton" and carried.linear_backend == "fp16"
-    quantized = build_parser().parse_args(["benchmark", "--linear-backend", "triton-int8"])
-    with pytest.raises(SystemExit, match="int8"):  # refused before anything is loaded
-        import asyncio
-
-        from llmserve_amd.cli import _benchmark
-
-        asyncio.run(_benchmark(quantized))
+    # the reference's switches between back ends it alone has (cli.py:263-271) are not options here
+    for switch in (["--rebuild-device-metadata"], ["--paged-attention-backend", "triton"], ["--linear-backend", "fp16"]):
+        with pytest.raises(SystemExit):
+            build_parser().parse_args(["benchmark", *switch])
     generate = build_parser().parse_args(["generate", "--prompt-tokens", "1,2,3", "--temperature", "0.8", "--top-p", "0.9"])
     assert (generate.max_tokens, generate.temperature, generate.top_p) == (32, 0.8, 0.9)
     replay = build_parser().parse_args(["replay", "--model", "m", "--out", "o", "--max-tokens", "256"])
@@ -50,10 +44,10 @@ def test_workload_is_fixed_by_its_seed():
     assert profile.prompt == LengthDistribution(128, 0.9, 8, 1024) and profile.output == LengthDistribution(64, 0.7, 4, 256)
     first, again = generate_workload(profile), generate_workload(profile)
     assert first == again and len(first) == 100
-    assert first[0].arrival_offset_s == 0.0 and all(a.arrival_offset_s <= b.arrival_offset_s for a, b in zip(first, first[1:]))
-    assert all(8 <= len(spec.prompt_token_ids) <= 1024 and 4 <= spec.max_new_tokens <= 256 for spec in first)
-    assert all(4 <= token < 32000 for spec in first for token in spec.prompt_token_ids)  # reserved ids 0-3 avoided
-    lengths = sorted(len(spec.prompt_token_ids) for spec in first)
+    assert first[0].at_s == 0.0 and all(a.at_s <= b.at_s for a, b in zip(first, first[1:]))
+    assert all(8 <= len(spec.prompt) <= 1024 and 4 <= spec.max_new_tokens <= 256 for spec in first)
+    assert all(4 <= token < 32000 for spec in first for token in spec.prompt)  # reserved ids 0-3 avoided
+    lengths = sorted(len(spec.prompt) for spec in first)
     assert 60 <= lengths[50] <= 260  # the median is near 128, the tail is long
     assert lengths[-1] > 3 * lengths[50]
 
@@ -62,13 +56,16 @@ def test_latency_metrics():
     """reference benchmark/metrics.py:11-58,71-94"""
     assert percentile([], 0.5) == 0.0 and percentile([1.0, 3.0], 0.5) == 2.0 and percentile([1, 2, 3, 4], 0.95) == pytest.approx(3.85)
     record = RequestMetrics("r", arrival_s=10.0, prompt_tokens=5, requested_output_tokens=4, first_token_s=10.5,
-                            finished_s=12.0, output_tokens=4)
+                            finished_s=12.0, output_tokens=4, preemptions=2, recomputed_tokens=30)
     assert (record.ttft_ms, record.tpot_ms, record.e2e_ms) == (500.0, 500.0, 2000.0)
     failed = RequestMetrics("f", 10.0, 5, 4, error="CacheFullError: x")
+    assert failed.ttft_ms is None and failed.tpot_ms is None and RequestMetrics("one", 1.0, 2, 1, None, 2.0, 2.0, 1).tpot_ms is None
     report = BenchmarkReport("continuous-fcfs", 10.0, 12.0, [record, failed], cache={"blocks_used": 0.0})
     summary = report.summary
     assert summary["successful_requests"] == 1 and summary["throughput_tokens_per_s"] == 2.0
     assert summary["ttft_ms_p50"] == 500.0 and summary["cache_blocks_used"] == 0.0
+    assert (summary["preemptions"], summary["recomputed_tokens"]) == (2, 30)
+    assert {"admitted_s", "preemptions", "recomputed_tokens", "ttft_ms"} <= set(record.to_dict())  # reference metrics.py:29,33-34
 
 
 def test_harness_sends_requests_at_their_arrival_times(tmp_path):
@@ -81,7 +78,9 @@ def test_harness_sends_requests_at_their_arrival_times(tmp_path):
             callback(token)
         return list(range(spec.max_new_tokens))
 
-    report = asyncio.run(BenchmarkHarness(profile).run("stub", generate))
+    facts = lambda request_id: {"admitted_s": 1.5, "preemptions": 1, "recomputed_tokens": 7}
+    report = asyncio.run(BenchmarkHarness(profile).run("stub", generate, facts))
+    assert [(r.admitted_s, r.preemptions, r.recomputed_tokens) for r in report.requests] == [(1.5, 1, 7)] * 5
     assert [r.output_tokens for r in report.requests] == [spec.max_new_tokens for spec in generate_workload(profile)]
     report.write_json(tmp_path / "r.json")
     report.write_csv(tmp_path / "r.csv")
@@ -89,16 +88,17 @@ def test_harness_sends_requests_at_their_arrival_times(tmp_path):
 
 
 def test_who_gives_way():
-    requests = [RequestState(name, [1], 4, arrival_order=order, processed_tokens=done)
+    requests = [Request(name, [1], GenerationConfig(max_new_tokens=4), ticket=order, cached=done)
                 for name, order, done in (("old", 0, 90), ("big", 1, 70), ("young", 2, 10))]
-    planned = [(request, 1) for request in requests]
-    assert choose_victim(planned, "largest").request_id == "big"  # most processed, but never the oldest
-    assert choose_victim(planned, "latest").request_id == "young"
-    assert choose_victim(planned[:2], "largest").request_id == "big"
+    shares = [Share(request, 1) for request in requests]
+    largest, latest = Scheduler(SchedulerConfig(preemption="largest")), Scheduler(SchedulerConfig(preemption="latest"))
+    assert largest.victim(shares).request_id == "big"  # most tokens cached, but never the oldest
+    assert latest.victim(shares).request_id == "young"
+    assert largest.victim(shares[:2]).request_id == "big"
     with pytest.raises(ValueError):
-        choose_victim(planned[:1])
+        largest.victim(shares[:1])
     with pytest.raises(ValueError):
-        choose_victim(planned, "random")
+        Scheduler(SchedulerConfig(preemption="random"))
 
 
 def test_byte_tokenizer_round_trip():
@@ -127,13 +127,13 @@ def test_workload_groups_arrive_in_order_and_fit_the_context():
     long = RequestGroup(3, LengthDistribution(600, 0.0, 600, 600), LengthDistribution(8, 0.0, 8, 8))
     profile = LoadProfile(requests=8, arrival_rate=10.0, groups=(short, long), vocabulary_size=50)
     specs = generate_workload(profile)
-    assert [len(spec.prompt_token_ids) <= 40 for spec in specs] == [True] * 5 + [False] * 3
-    assert [len(spec.prompt_token_ids) for spec in specs[5:]] == [600] * 3
+    assert [len(spec.prompt) <= 40 for spec in specs] == [True] * 5 + [False] * 3
+    assert [len(spec.prompt) for spec in specs[5:]] == [600] * 3
     assert all(90 <= spec.max_new_tokens <= 110 for spec in specs[:5]) and all(spec.max_new_tokens == 8 for spec in specs[5:])
-    assert [spec.arrival_offset_s for spec in specs] == sorted(spec.arrival_offset_s for spec in specs)
+    assert [spec.at_s for spec in specs] == sorted(spec.at_s for spec in specs)
     assert specs == generate_workload(profile)
     fitted = generate_workload(profile.fitted(500))
-    assert [len(spec.prompt_token_ids) for spec in fitted[5:]] == [492] * 3
+    assert [len(spec.prompt) for spec in fitted[5:]] == [492] * 3
     with pytest.raises(ValueError):
         LoadProfile(requests=7, groups=(short, long))
     mix = LoadProfile.from_yaml(ROOT / "configs" / "workload-long-context-mix.yaml")

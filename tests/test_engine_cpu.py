@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from llmserve_amd import CacheConfig, CacheFullError, GenerationConfig, LLMEngine, SchedulerConfig, StepEntry
-from llmserve_amd.engine import EngineCore, IterationScheduler, ModelRunner, RequestState, plan_iteration
+from llmserve_amd.engine import EngineCore, ModelRunner, Request, RequestTooLongError, Scheduler
 from llmserve_amd.sampling import uniform_for
 from llmserve_amd.weights import load_model_folder
 from tests.plain import qwen2_plain as plain
@@ -106,53 +106,124 @@ def test_a_step_that_does_not_fit_changes_nothing(model_folders):
     assert runner.step([StepEntry("a", [1, 2, 3], [])], create_missing=True).shape == (0, 256)
 
 
+def test_the_pages_of_one_layer_hold_the_rotated_keys_and_the_values(model_folders):
+    """The host-side read paths (reference kv_cache.py:268-342): after a prompt was fed in portions, the
+    first layer's pages hold, position by position, the keys the plain implementation computes (bias added,
+    rotated) and the values; in B's windowed layers the pages a window has passed are gone."""
+    for name in ("A", "B"):
+        config, weights = oracle(model_folders, name)
+        tokens = random_tokens(61, config.vocab_size, seed=4)
+        runner = make_runner(model_folders, name)
+        for start, end in ((0, 23), (23, 24), (24, 61)):
+            runner.step([StepEntry("r", tokens[start:end], [])], create_missing=True)
+        h = weights["embed_tokens.weight"][torch.tensor(tokens)]
+        normed = plain.rms_norm(h, weights["layers.0.input_layernorm.weight"], config.rms_norm_eps)
+        prefix = "layers.0.self_attn."
+        keys = (normed @ weights[prefix + "k_proj.weight"].T + weights[prefix + "k_proj.bias"]).view(61, config.num_kv_heads, config.head_dim)
+        values = (normed @ weights[prefix + "v_proj.weight"].T + weights[prefix + "v_proj.bias"]).view(61, config.num_kv_heads, config.head_dim)
+        rotate = plain.rope_half if config.rope_pairing == "half" else plain.rope_adjacent
+        keys = rotate(keys, plain.rope_angles(config.head_dim, config.rope_theta, torch.arange(61)))
+        first, cached_keys, cached_values = runner.cache.gather("r", 0)
+        assert first == 0 and cached_keys.shape == (61, config.num_kv_heads, config.head_dim)
+        close(cached_keys, keys)
+        close(cached_values, values)
+        page = CONFIGS[name][1]
+        starts = [start for start, _, _ in runner.cache.iter_pages("r", 0)]
+        assert starts == list(range(0, 61, page))
+        tables, lengths = runner.cache.block_table_tensors(["r"])
+        assert lengths.tolist() == [61] and tables.shape == (1, -(-61 // page)) and (tables >= 0).all()
+        if name == "B":  # layers 1 and 2 see 24 keys: pages wholly before them go when the next token is reserved
+            assert runner.cache.gather("r", 1)[0] == 0
+            runner.step([StepEntry("r", [5], [])])
+            first, windowed, _ = runner.cache.gather("r", 1)  # the query at 61 reads keys 38 to 61
+            assert first == (38 // page) * page and windowed.shape[0] == 62 - first
+            assert runner.cache.gather("r", 0)[0] == 0  # the first layer sees everything
+        with pytest.raises(ValueError):
+            runner.cache.gather("r", 99)
+
+
 # --------------------------------------------------------------------------- scheduler decisions
+
+
+def request(name, prompt, max_new_tokens=4, **fields):
+    return Request(name, list(prompt), GenerationConfig(max_new_tokens=max_new_tokens), **fields)
 
 
 def test_policies_and_the_static_barrier():
     """reference tests/test_engine.py:323-334"""
-    scheduler = IterationScheduler(2, policy="sjf", mode="static")
-    long, short, later = RequestState("long", [1], 20), RequestState("short", [1], 2), RequestState("later", [1], 1)
-    scheduler.add(long)
-    scheduler.add(short)
+    scheduler = Scheduler(SchedulerConfig(2, policy="sjf"), mode="static")
+    long, short, later = request("long", [1], 20), request("short", [1], 2), request("later", [1], 1)
+    scheduler.enqueue(long)
+    scheduler.enqueue(short)
+    assert [r.request_id for r in scheduler.waiting] == ["short", "long"]
     assert [r.request_id for r in scheduler.admit()] == ["short", "long"]
-    scheduler.add(later)
+    assert short.admitted_at is not None
+    scheduler.enqueue(later)
     assert scheduler.admit() == []
-    scheduler.finish(short)
+    scheduler.retire(short)
     assert scheduler.admit() == []
-    scheduler.finish(long)
-    assert scheduler.admit() == [later]
+    scheduler.retire(long)
+    assert scheduler.admit() == [later] and not scheduler.idle
+    scheduler.retire(later)
+    assert scheduler.idle
 
-    by_priority = IterationScheduler(2, policy="priority")
-    for name, priority in (("low", 0), ("high", 5), ("mid", 2)):
-        by_priority.add(RequestState(name, [1], 4, priority=priority))
+    by_priority = Scheduler(SchedulerConfig(2, policy="priority"))
+    for name, priority in (("low", 0), ("high", 5), ("mid", 2), ("mid-too", 2)):
+        by_priority.enqueue(request(name, [1], priority=priority))
     assert [r.request_id for r in by_priority.admit()] == ["high", "mid"]
+    assert [r.request_id for r in by_priority.waiting] == ["mid-too", "low"] and by_priority.num_waiting == 2
+    by_priority.retire(by_priority.waiting[0])  # a request may leave the line too
+    assert [r.request_id for r in by_priority.waiting] == ["low"]
 
-    first_come = IterationScheduler(1, policy="fcfs")
-    a, b = RequestState("a", [1, 2], 4), RequestState("b", [1], 4)
-    first_come.add(a)
-    first_come.add(b)
+    first_come = Scheduler(SchedulerConfig(1, policy="fcfs"))
+    a, b = request("a", [1, 2]), request("b", [1])
+    first_come.enqueue(a)
+    first_come.enqueue(b)
     assert first_come.admit() == [a]
-    a.processed_tokens = 2
-    first_come.preempt(a)  # scheduler.py:88-93
-    assert (a.processed_tokens, a.recomputed_tokens, a.preemptions) == (0, 2, 1)
-    assert first_come.admit() == [a]  # it keeps its place in arrival order
+    a.cached = 2
+    first_admission = a.admitted_at
+    first_come.evict(a)  # scheduler.py:88-93
+    assert (a.cached, a.replayed_tokens, a.evictions) == (0, 2, 1)
+    assert first_come.admit() == [a] and a.admitted_at == first_admission  # it keeps its place in arrival order
     with pytest.raises(ValueError):
-        IterationScheduler(2, policy="random")
+        Scheduler(SchedulerConfig(2, policy="random"))
+    with pytest.raises(ValueError):
+        Scheduler(SchedulerConfig(2), mode="sometimes")
+
+
+def test_shortest_job_counts_what_is_left_when_a_request_rejoins_the_line():
+    scheduler = Scheduler(SchedulerConfig(1, policy="sjf"))
+    long, short = request("long", [1], 10), request("short", [1], 4)
+    scheduler.enqueue(long)
+    assert scheduler.admit() == [long]
+    scheduler.enqueue(short)
+    long.output = [5] * 8  # two tokens left: fewer than the short one's four
+    long.cached = 9
+    scheduler.evict(long)
+    assert [r.request_id for r in scheduler.waiting] == ["long", "short"]
 
 
 def test_plan_gives_everyone_one_token_then_tops_up():
     """reference engine.py:372-391"""
-    decoding = RequestState("d", [1, 2], 8, generated_token_ids=[3], processed_tokens=2)
-    long = RequestState("l", list(range(40)), 8)
-    short = RequestState("s", list(range(5)), 8)
-    plan = plan_iteration([decoding, long, short], 2048, 16)
-    assert [count for _, count in plan] == [1, 16, 5]
-    assert [count for _, count in plan_iteration([decoding, long, short], 10, 16)] == [1, 8, 1]
-    assert [count for _, count in plan_iteration([long, short], 2, 16)] == [1, 1]
-    done = RequestState("x", [1], 8, processed_tokens=1)
+    decoding = request("d", [1, 2], 8, output=[3], cached=2)
+    long = request("l", range(40), 8)
+    short = request("s", range(5), 8)
+
+    def counts(batch, budget, chunk):
+        scheduler = Scheduler(SchedulerConfig(max_batch_size=8, max_tokens_per_step=budget))
+        scheduler.running = list(batch)
+        return [share.count for share in scheduler.plan(chunk)]
+
+    assert counts([decoding, long, short], 2048, 16) == [1, 16, 5]
+    assert counts([decoding, long, short], 10, 16) == [1, 8, 1]
+    assert counts([long, short], 2, 16) == [1, 1]
+    assert counts([long, short], 1, 16) == [1, 1]  # everybody brings a token whatever the budget says
+    assert long.next_tokens(3) == [0, 1, 2] and decoding.next_tokens(1) == [3]
+    straddling = request("x", [1, 2, 3], 8, output=[7, 8], cached=2)
+    assert straddling.next_tokens(3) == [3, 7, 8] and straddling.owed == 3 and straddling.in_prompt
+    done = request("x", [1], 8, cached=1)
     with pytest.raises(RuntimeError):
-        plan_iteration([done], 8, 4)
+        counts([done], 8, 4)
 
 
 def core_for(model_folders, name="A", num_blocks=64, batch=4, budget=64, chunk=16, mode="continuous", policy="fcfs"):
@@ -199,11 +270,11 @@ def test_chunked_prefill_equals_token_at_a_time(model_folders):
 def test_late_prompt_portions_run_beside_decoding(model_folders):
     """reference tests/test_engine.py:105-143"""
     core = core_for(model_folders, "A", batch=2, budget=32, chunk=16)
-    long = RequestState("long", list(range(1, 41)), 5)
-    core.submit(long, GenerationConfig(max_new_tokens=5))
-    while not long.generated_token_ids:
+    long = request("long", range(1, 41), 5)
+    core.submit(long)
+    while not long.output:
         core.step()
-    core.submit(RequestState("short", [7, 8, 9, 10], 2), GenerationConfig(max_new_tokens=2))
+    core.submit(request("short", [7, 8, 9, 10], 2))
     while core.has_work:
         core.step()
     assert any(dict(plan).get("long") == 1 and dict(plan).get("short", 0) > 1 for plan in core.step_log)
@@ -212,10 +283,10 @@ def test_late_prompt_portions_run_beside_decoding(model_folders):
 def test_static_mode_keeps_a_late_request_behind_the_barrier(model_folders):
     """reference tests/test_engine.py:146-185"""
     core = core_for(model_folders, "A", batch=2, budget=32, mode="static")
-    first = RequestState("first", list(range(1, 25)), 4)
-    core.submit(first, GenerationConfig(max_new_tokens=4))
+    first = request("first", range(1, 25), 4)
+    core.submit(first)
     core.step()
-    core.submit(RequestState("late", [9, 10], 2), GenerationConfig(max_new_tokens=2))
+    core.submit(request("late", [9, 10], 2))
     while core.has_work:
         core.step()
     assert not any({"first", "late"} <= set(dict(plan)) for plan in core.step_log)
@@ -230,17 +301,16 @@ def test_pages_run_out_the_largest_gives_way_and_replays(model_folders):
     streamed = {"request-000000": [], "request-000001": []}
     requests = []
     for index, prompt in enumerate(prompts):
-        request = RequestState(f"request-{index:06d}", prompt, 14)
-        core.submit(request, GenerationConfig(max_new_tokens=14))
-        requests.append(request)
+        requests.append(request(f"request-{index:06d}", prompt, 14))
+        core.submit(requests[-1])
     while core.has_work:
         for event in core.step():
             streamed[event.request.request_id].append(event.token)
         core.runner.cache.check_invariants()
-    assert sum(r.preemptions for r in requests) > 0 and sum(r.recomputed_tokens for r in requests) > 0
-    assert [r.generated_token_ids for r in requests] == expected  # replay changes nothing
+    assert sum(r.evictions for r in requests) > 0 and sum(r.replayed_tokens for r in requests) > 0
+    assert [r.output for r in requests] == expected  # replay changes nothing
     assert [streamed[r.request_id] for r in requests] == expected  # and no token is streamed twice
-    assert core.iteration_stats["preemptions"] == sum(r.preemptions for r in requests)
+    assert core.iteration_stats["preemptions"] == sum(r.evictions for r in requests)
     assert core.runner.cache.used_pages == 0
 
 
@@ -266,21 +336,22 @@ def test_looking_ahead_changes_no_decision(model_folders):
             return _inner(*args, **kwargs)
 
         core.runner.step_from_device = counted
-        requests = [RequestState(f"r{i}", prompt, 12) for i, prompt in enumerate(prompts)]
-        for request, stop in zip(requests[:2], stops):
-            core.submit(request, GenerationConfig(max_new_tokens=12, stop_token_ids=stop))
+        requests = [Request(f"r{i}", prompt, GenerationConfig(max_new_tokens=12, stop_token_ids=stop))
+                    for i, (prompt, stop) in enumerate(zip(prompts, stops))]
+        for each in requests[:2]:
+            core.submit(each)
         steps = 0
         while core.has_work or steps < 8:
             if steps == 4:
-                core.submit(requests[2], GenerationConfig(max_new_tokens=12, stop_token_ids=stops[2]))
+                core.submit(requests[2])
             if steps == 7:
-                core.submit(requests[3], GenerationConfig(max_new_tokens=12))
+                core.submit(requests[3])
             core.step()
             core.runner.cache.check_invariants()
             steps += 1
         assert not core.runner._ahead and core.runner.cache.used_pages == 0
-        assert all(request.error is None for request in requests)
-        outcomes.append((core.step_log, [r.generated_token_ids for r in requests], [r.preemptions for r in requests]))
+        assert all(each.error is None for each in requests)
+        outcomes.append((core.step_log, [r.output for r in requests], [r.evictions for r in requests]))
     assert outcomes[0] == outcomes[1] == outcomes[2]
     assert queued_ahead[0] > 5 and queued_ahead[1:] == [0, 0]
     assert sum(outcomes[0][2]) > 0  # pages did run out
@@ -292,18 +363,61 @@ def test_looking_ahead_changes_no_decision(model_folders):
 def test_a_request_that_can_never_fit_fails_alone(model_folders):
     """reference tests/test_engine.py:261-277"""
     core = core_for(model_folders, "A", num_blocks=2, batch=2)
-    small = RequestState("small", [1, 2, 3], 2)
-    huge = RequestState("huge", list(range(1, 60)), 2)
-    core.submit(small, GenerationConfig(max_new_tokens=2))
-    core.submit(huge, GenerationConfig(max_new_tokens=2))
+    small = request("small", [1, 2, 3], 2)
+    huge = request("huge", range(1, 60), 2)
+    core.submit(small)
+    core.submit(huge)
     while core.has_work:
         core.step()
-    assert isinstance(huge.error, CacheFullError) and small.error is None and len(small.generated_token_ids) == 2
+    assert isinstance(huge.error, CacheFullError) and small.error is None and len(small.output) == 2
     assert core.runner.cache.used_pages == 0 and not core.runner.cache.sequences
     with pytest.raises(ValueError):
-        core.submit(RequestState("empty", [], 2), GenerationConfig(max_new_tokens=2))
+        core.submit(request("empty", [], 2))
     with pytest.raises(ValueError):
         EngineCore(core.runner, SchedulerConfig(max_batch_size=8, max_tokens_per_step=4))
+
+
+def test_a_request_that_outgrows_the_longest_sequence_costs_nobody_else(model_folders):
+    """Prompt plus new tokens beyond the longest sequence the cache can describe is not a shortage of
+    pages: such a request is refused when it is submitted, and one that slipped into the batch ends
+    alone with an error of its own, while nobody gives way for it."""
+    config, weights = oracle(model_folders, "C")  # max_position_embeddings 256
+    core = core_for(model_folders, "C", num_blocks=64, batch=3, budget=64)
+    assert core.runner.cache.max_sequence_length == 256
+    with pytest.raises(RequestTooLongError):
+        core.submit(request("long", random_tokens(199, config.vocab_size, seed=1), 100))
+    with pytest.raises(ValueError, match="vocabulary"):
+        core.submit(request("alien", [1, 2, config.vocab_size], 4))
+    with pytest.raises(ValueError, match="vocabulary"):
+        core.submit(request("negative", [1, -2], 4))
+    prompts = [random_tokens(n, config.vocab_size, seed=n) for n in (30, 41)]
+    others = [request(f"ok{index}", prompt, 6) for index, prompt in enumerate(prompts)]
+    for each in others:
+        core.submit(each)
+    smuggled = request("smuggled", random_tokens(250, config.vocab_size, seed=3), 20)
+    core.scheduler.enqueue(smuggled)  # past the check, as if the limit had changed under it
+    while core.has_work:
+        core.step()
+        core.runner.cache.check_invariants()
+    assert isinstance(smuggled.error, RequestTooLongError) and len(smuggled.output) == 7  # 256 cached tokens give the seventh; it cannot be fed
+    assert [each.evictions for each in others] == [0, 0] and all(each.error is None for each in others)
+    assert [each.output for each in others] == [plain.generate(weights, config, prompt, 6) for prompt in prompts]
+    assert core.iteration_stats["preemptions"] == 0 and core.runner.cache.used_pages == 0
+
+
+def test_a_full_batch_decodes_ahead_while_others_wait(model_folders):
+    """Requests in the line do not stop the engine from preparing (and queueing) the next decode step
+    as long as none of them can be admitted: the batch is full and stays so."""
+    config, weights = oracle(model_folders, "A")
+    prompts = [random_tokens(n, config.vocab_size, seed=80 + n) for n in (5, 9, 4, 7)]
+    expected = [plain.generate(weights, config, prompt, 9) for prompt in prompts]
+    core = core_for(model_folders, "A", batch=2, budget=32, chunk=16)
+    queued = []
+    inner = core.runner.step_from_device
+    core.runner.step_from_device = lambda ids, tokens: (queued.append((list(ids), core.scheduler.num_waiting)), inner(ids, tokens))[1]
+    assert core.generate(prompts, GenerationConfig(max_new_tokens=9)) == expected
+    assert any(waiting > 0 for _, waiting in queued), "no step was queued ahead while requests waited"
+    assert core.runner.cache.used_pages == 0 and not core.runner._ahead
 
 
 # --------------------------------------------------------------------------- the asynchronous entry point

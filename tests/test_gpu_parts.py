@@ -144,9 +144,9 @@ def test_toy_architecture_on_the_gpu(tmp_path, kernels):
 # ------------------------------------------------------------------------------- entry points
 
 
+@pytest.mark.parametrize("name", ["B", "B-loud"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_greedy_generation_through_the_entry_point(model_folders, dtype):
-    name = "B"
+def test_greedy_generation_through_the_entry_point(model_folders, dtype, name):
     config, page = CONFIGS[name]
     plain_config, weights = plain.PlainConfig.from_folder(model_folders[name]), plain.read_weights(model_folders[name])
     prompts = [random_tokens(n, config.vocab_size, seed=n) for n in (2, 9, 23, 40, 64, 100)]
@@ -168,9 +168,13 @@ def test_greedy_generation_through_the_entry_point(model_folders, dtype):
     assert streamed == outputs
     if dtype == "float32":
         assert outputs == expected
-    else:  # bfloat16 may turn a near-tie; the tokens before the first such turn must agree
+    else:  # bfloat16 may turn a near-tie: every token must be the plain decoder's choice, or within rounding of it
+        from tests.tiny import unjustified_greedy_tokens
+
+        for prompt, got in zip(prompts, outputs):
+            assert len(got) == 12 and not unjustified_greedy_tokens(plain, weights, plain_config, prompt, got)
         agreeing = sum(a == b for got, want in zip(outputs, expected) for a, b in zip(got, want))
-        assert agreeing >= 0.8 * 12 * len(prompts), (outputs, expected)
+        print(f"{name}: {agreeing} of {12 * len(prompts)} tokens equal the plain decoder's")
 
 
 def test_sampled_generation_is_the_plain_decoders(model_folders):
@@ -191,17 +195,24 @@ def test_sampled_generation_is_the_plain_decoders(model_folders):
 def test_long_decoding_and_first_tokens(model_folders, dtype):
     """300 tokens decoded one by one after a one-token prompt (the first tokens of a sequence,
     then many captured steps, page after page), each step's logits against the plain forward."""
-    config, page = CONFIGS["A"]
-    plain_config, weights = plain.PlainConfig.from_folder(model_folders["A"]), plain.read_weights(model_folders["A"])
+    from tests.tiny import BF16_LARGEST, BF16_MEAN
+
+    name = "A-loud"  # weights wide enough that attention decides the logits
+    config, page = CONFIGS[name]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders[name]), plain.read_weights(model_folders[name])
     tokens = random_tokens(300, config.vocab_size, seed=4)
     expected = plain.forward(weights, plain_config, tokens)
     from llmserve_amd.kernels import HipKernels
 
-    loaded = load_model_folder(model_folders["A"], dtype)
+    loaded = load_model_folder(model_folders[name], dtype)
     runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(page, 24, 2))
     rows = [runner.step([StepEntry("r", [token], [0])], create_missing=True).clone() for token in tokens]
-    tolerance = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=4e-2, rtol=4e-2)
-    torch.testing.assert_close(torch.cat(rows).cpu().double(), expected, **tolerance)
+    got = torch.cat(rows).cpu().double()
+    spread = float(expected.std())
+    tolerance = dict(atol=2e-5 * max(1.0, spread / 0.3), rtol=1e-4) if dtype == "float32" else dict(atol=BF16_LARGEST * spread, rtol=3e-2)
+    torch.testing.assert_close(got, expected, **tolerance)
+    if dtype == "bfloat16":
+        assert float((got - expected).abs().mean()) < BF16_MEAN * spread
     runner.close()
 
 
@@ -248,7 +259,7 @@ def test_everything_at_once_matches_the_plain_decoder(model_folders):
     decode steps, the next step prepared and queued ahead): greedy and sampled requests side by side,
     some with stop tokens, late arrivals, and so few pages that requests give way and replay.  Every
     request's tokens are the plain decoder's."""
-    from llmserve_amd.engine import RequestState
+    from llmserve_amd.engine import Request
     from llmserve_amd.kernels import HipKernels
 
     config, page = CONFIGS["B"]
@@ -268,23 +279,22 @@ def test_everything_at_once_matches_the_plain_decoder(model_folders):
     loaded = load_model_folder(model_folders["B"], "float32")
     runner = ModelRunner(loaded, HipKernels(torch.float32), CacheConfig(page, 14, 6))  # 14 pages of 8: 112 tokens
     core = EngineCore(runner, SchedulerConfig(5, 48), prefill_chunk_size=16)
-    requests = [RequestState(f"r{index}", prompt, s.max_new_tokens) for index, (prompt, s) in enumerate(zip(prompts, settings))]
-    waiting = list(zip(requests, settings))
-    for request, setting in waiting[:5]:
-        core.submit(request, setting)
-    waiting = waiting[5:]
+    requests = [Request(f"r{index}", prompt, s) for index, (prompt, s) in enumerate(zip(prompts, settings))]
+    for request in requests[:5]:
+        core.submit(request)
+    waiting = requests[5:]
     turn = 0
     while core.has_work or waiting:
         if waiting and turn % 3 == 0:  # the others arrive one by one while the engine runs
-            core.submit(*waiting.pop(0))
+            core.submit(waiting.pop(0))
         core.step()
         turn += 1
         assert turn < 2000
     runner.cache.check_invariants()
     assert runner.cache.used_pages == 0
-    assert sum(r.preemptions for r in requests) > 0, "the pool was meant to be too small"
-    assert any(len(r.generated_token_ids) < s.max_new_tokens for r, s in zip(requests, settings)), "nobody stopped early"
-    assert [r.generated_token_ids for r in requests] == expected
+    assert sum(r.evictions for r in requests) > 0, "the pool was meant to be too small"
+    assert any(len(r.output) < s.max_new_tokens for r, s in zip(requests, settings)), "nobody stopped early"
+    assert [r.output for r in requests] == expected
     runner.close()
 
 

@@ -11,13 +11,13 @@ import torch
 
 from tests.gpu_helpers import TraceBuilder, replay
 from tests.plain import qwen2_plain as plain
-from tests.tiny import CONFIGS, PAGE_WIDE, WIDE_CONFIGS, random_tokens, write_wide_folder
+from tests.tiny import BF16_LARGEST, BF16_MEAN, CONFIGS, PAGE_WIDE, WIDE_CONFIGS, random_tokens, write_wide_folder
 
 pytestmark = pytest.mark.gpu
 
-# float32: rounding only.  bfloat16: activations are rounded to 8 bits of mantissa between
-# kernels; logits of these models are of order 1, and the same bound holds for every way of cutting.
-TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
+# float32: rounding only.  bfloat16: activations are rounded to 8 bits of mantissa between kernels; the
+# bound is stated in units of the logits' spread (tests/tiny.py), the same for every way of cutting.
+TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4)}
 LENGTHS = {"A": [1, 5, 17, 33, 70, 100], "B": [2, 9, 23, 40, 64, 100], "C": [3, 48, 65]}
 
 
@@ -67,27 +67,38 @@ def build_trace(prompts: dict[str, list[int]], page: int, budget: int = 4 * 64):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "A-loud", "B-loud", "C-loud"])
 def test_replay_matches_plain_under_every_cut(model_folders, tmp_path, name, dtype):
+    """The "loud" folders hold the same configurations with weights wide enough that attention decides the
+    logits: there the bfloat16 bound can see a wrong rotation or a lost bias (test_plain.py shows it does)."""
     config, page = CONFIGS[name]
     folder = model_folders[name]
     plain_config, weights = plain.PlainConfig.from_folder(folder), plain.read_weights(folder)
-    prompts = {f"p{n}": random_tokens(n, config.vocab_size, seed=100 + n) for n in LENGTHS[name]}
+    prompts = {f"p{n}": random_tokens(n, config.vocab_size, seed=100 + n) for n in LENGTHS[name[0]]}
     expected = {key: plain.forward(weights, plain_config, tokens) for key, tokens in prompts.items()}
     trace = build_trace(prompts, page)
     results = replay(folder, dtype, trace.steps, tmp_path / "out", max_tokens=4 * 64, block_size=page,
                      vocab=config.vocab_size)
     rows = trace.collect(results)
-    checked = 0
+    spread = float(torch.cat(list(expected.values())).std())
+    # float32: 2e-5 where the logits spread by up to 0.3 (the quiet folders); rounding grows with the size of
+    # the sums, so in proportion to the spread above that (the loud folders' is three to five times wider)
+    bound = dict(atol=2e-5 * max(1.0, spread / 0.3), rtol=1e-4) if dtype == "float32" else dict(atol=BF16_LARGEST * spread, rtol=3e-2)
+    checked, total, count = 0, 0.0, 0
     for (request, position), logits in rows.items():
         mode, key = request.split("-", 1)
         torch.testing.assert_close(
-            logits.double(), expected[key][position], **TOLERANCE[dtype],
+            logits.double(), expected[key][position], **bound,
             msg=lambda m: f"{mode} {key} position {position}: {m}",
         )
+        total += float((logits.double() - expected[key][position]).abs().sum())
+        count += logits.numel()
         checked += 1
     whole = sum(len(t) for t in prompts.values())
     assert checked >= 3 * whole  # whole, cut and mixed give every position; tails add theirs
+    print(f"{name} {dtype}: mean error {total / count / spread:.2e} of the spread {spread:.3f}")
+    if dtype == "bfloat16":  # a fault that stays under the bound for the largest element still moves the mean
+        assert total / count < BF16_MEAN * spread
 
 
 def test_float32_cuts_agree_with_each_other_to_rounding(model_folders, tmp_path):
@@ -139,7 +150,7 @@ def test_replay_at_benchmark_layer_sizes(wide_models, tmp_path, sizes, dtype):
     # largest element again lies near five times the typical one.
     spread = float(torch.cat(list(expected.values())).std())
     walk = math.sqrt(WIDE.intermediate_size) * 2.0 ** -24 * spread
-    bound = dict(atol=5 * walk, rtol=1e-4) if dtype == "float32" else dict(atol=0.06 * spread, rtol=3e-2)
+    bound = dict(atol=5 * walk, rtol=1e-4) if dtype == "float32" else dict(atol=BF16_LARGEST * spread, rtol=3e-2)
     total, count = 0.0, 0
     for (request, position), logits in trace.collect(results).items():
         mode, key = request.split("-", 1)
@@ -151,7 +162,7 @@ def test_replay_at_benchmark_layer_sizes(wide_models, tmp_path, sizes, dtype):
         count += logits.numel()
     print(f"{dtype}: mean error {total / count:.3e}, spread {spread:.3f}")
     # a systematic fault that stays under the bound for the largest element still moves the mean
-    assert total / count < (walk if dtype == "float32" else 0.01 * spread)
+    assert total / count < (walk if dtype == "float32" else BF16_MEAN * spread)
 
 
 @pytest.mark.parametrize("sizes,requests", [("1.5B", 20), ("1.5B", 40), ("7B", 20), ("7B", 40), ("32B", 20), ("32B", 8)])
@@ -191,7 +202,7 @@ def test_captured_steps_of_many_rows_at_benchmark_layer_sizes(wide_models, sizes
     for at, logits in rows:
         for index in range(requests):
             torch.testing.assert_close(
-                logits[index].cpu().double(), expected[index][at[index]], atol=0.06 * spread, rtol=3e-2,
+                logits[index].cpu().double(), expected[index][at[index]], atol=BF16_LARGEST * spread, rtol=3e-2,
                 msg=lambda m: f"request {index} position {at[index]}: {m}",
             )
     runner.close()

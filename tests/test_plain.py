@@ -210,3 +210,36 @@ def test_generate_stops_and_keeps_the_stop_token(model_folders):
     assert len(free) == 6
     stopped = plain.generate(weights, config, [1, 2, 3], 6, stop_token_ids=(free[2],))
     assert stopped == free[: free.index(free[2]) + 1]
+
+
+@pytest.mark.parametrize("name", ["A-loud", "B-loud", "C-loud"])
+def test_the_bfloat16_bounds_can_see_a_wrong_rotation_and_a_lost_bias(model_folders, name):
+    """The GPU tests allow a bfloat16 run BF16_LARGEST of the logits' spread at the largest element and
+    BF16_MEAN of it on average.  At the "loud" folders both plausible mistakes of the attention part exceed
+    that, by the plain implementation's own account: pairing the rotation the other way, and dropping the key
+    bias (which matters only through the rotation: an unrotated bias adds the same to every score of a query)."""
+    import dataclasses
+
+    from tests.tiny import BF16_LARGEST, BF16_MEAN, random_tokens
+
+    config, weights = plain.PlainConfig.from_folder(model_folders[name]), plain.read_weights(model_folders[name])
+    prompts = [random_tokens(n, config.vocab_size, seed=100 + n) for n in (17, 33, 70)]
+    right = torch.cat([plain.forward(weights, config, prompt) for prompt in prompts])
+    spread = float(right.std())
+
+    def visible(other: torch.Tensor) -> bool:
+        error = (other - right).abs()
+        return float(error.max()) > 2 * BF16_LARGEST * spread and float(error.mean()) > 2 * BF16_MEAN * spread
+
+    swapped = dataclasses.replace(config, rope_pairing="adjacent" if config.rope_pairing == "half" else "half")
+    assert visible(torch.cat([plain.forward(weights, swapped, prompt) for prompt in prompts]))
+    if config.attention_bias:
+        without = {key: torch.zeros_like(value) if key.endswith("k_proj.bias") else value for key, value in weights.items()}
+        assert visible(torch.cat([plain.forward(without, config, prompt) for prompt in prompts]))
+    quiet = name.split("-")[0]  # the reference's own initialisation hides both: that is why the loud folders exist
+    config, weights = plain.PlainConfig.from_folder(model_folders[quiet]), plain.read_weights(model_folders[quiet])
+    if config.attention_bias:
+        right = torch.cat([plain.forward(weights, config, prompt) for prompt in prompts])
+        without = {key: torch.zeros_like(value) if key.endswith("k_proj.bias") else value for key, value in weights.items()}
+        lost = torch.cat([plain.forward(without, config, prompt) for prompt in prompts])
+        assert float((lost - right).abs().max()) < BF16_LARGEST * float(right.std())

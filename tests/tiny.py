@@ -136,6 +136,18 @@ def write_wide_folder(root: Path, sizes: str = "1.5B") -> Path:
     return write_model_folder(root / f"W{sizes}", config, seed=seed, norm_std=0.1)
 
 
+# How the "loud" folders are drawn.  At N(0, 0.02) a model this narrow barely attends: every score is
+# near zero, and a wrong rotation or a lost bias moves the logits by less than bfloat16 rounding does.
+# Four times wider weights and biases of 0.3 make attention decide the logits, so that the bfloat16
+# bounds below can see such faults (test_plain.py shows that they do).
+LOUD = dict(std=0.08, bias_std=0.3)
+
+# What a bfloat16 run may differ from the plain implementation by, in units of the logits' spread (their
+# standard deviation): the largest element, and the mean over all elements.  Each of the ten or so roundings
+# of an activation between kernels adds about 2^-9 of the spread.
+BF16_LARGEST, BF16_MEAN = 0.06, 0.01
+
+
 def write_tiny_folders(root: Path) -> dict[str, Path]:
     return {
         # norm weights 1.0 as the reference initialises them, biases drawn
@@ -143,10 +155,29 @@ def write_tiny_folders(root: Path) -> dict[str, Path]:
         # norm weights N(1, 0.1), stored in 32-bit so that they stay so in a bfloat16 run
         "B": write_model_folder(root / "B", TINY_B, seed=23, norm_std=0.1, wide_roles=("norm",)),
         "C": write_model_folder(root / "C", TINY_C, seed=5, norm_std=0.1, std=0.05),
+        "A-loud": write_model_folder(root / "A-loud", TINY_A, seed=12, norm_std=0.0, **LOUD),
+        "B-loud": write_model_folder(root / "B-loud", TINY_B, seed=24, norm_std=0.1, wide_roles=("norm",), **LOUD),
+        "C-loud": write_model_folder(root / "C-loud", TINY_C, seed=6, norm_std=0.1, **LOUD),
     }
 
 
 CONFIGS = {"A": (TINY_A, PAGE_A), "B": (TINY_B, PAGE_B), "C": (TINY_C, PAGE_C)}
+CONFIGS.update({f"{name}-loud": CONFIGS[name] for name in ("A", "B", "C")})
+
+
+def unjustified_greedy_tokens(plain, weights, config, prompt: list[int], generated: list[int], largest: float = BF16_LARGEST):
+    """Checks greedy tokens of a reduced-precision run one by one: token j must be, for the plain
+    implementation fed the run's own prefix, the best token or within rounding of it (two logits, each
+    off by at most `largest` of the spread).  Returns [(j, token, how far below the best, allowed)] of
+    those that are not; an exact run returns none because it equals the plain decoder."""
+    bad = []
+    for index, token in enumerate(generated):
+        logits = plain.forward(weights, config, list(prompt) + list(generated[:index]))[-1]
+        allowed = 2 * largest * float(logits.std())
+        short = float(logits.max() - logits[token])
+        if short > allowed:
+            bad.append((index, token, short, allowed))
+    return bad
 
 
 def random_tokens(count: int, vocab: int, seed: int) -> list[int]:
