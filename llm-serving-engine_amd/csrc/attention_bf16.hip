@@ -79,6 +79,8 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
   const float2* table;        // [rows][D / 2] (cos, sin) of each token's angles, or null
   int pairing;
   const int* slots;           // [rows] page * page_size + offset of each token, negative: store nothing
+  int unmerged;               // key splits are left for the reader to merge: each split's result is divided by its own
+                              // sum of weights and stored as bfloat16 where partial_acc points, [rows][heads][splits][D]
 };
 
 // One step's operands as a lane holds them: its slices of the K rows of the two 16-row tiles and,
@@ -221,6 +223,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   // the work list runs from early to late tokens; late ones walk more keys, so they start first
   // (when FUSED every request brings one token: tile i is request i and row i, nothing to look up)
   const int* item = work + (size_t)(gridDim.x - 1 - blockIdx.x) * 4;
+  // an item of no columns pads a work list to the length a captured step was recorded with: nothing to do
+  if (!FUSED && item[3] <= 0) return;
   const int request = FUSED ? (int)blockIdx.x : item[0], row0 = FUSED ? (int)blockIdx.x : item[1];
   const ColumnMap map = {heads_here, FUSED ? 0 : item[2], FUSED ? (group <= 16 ? heads_here : 1) : item[3], group <= 16};
   const int tokens = map.tokens();
@@ -536,9 +540,16 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
         for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
       } else {
         const size_t slot = (row * heads + head) * splits + blockIdx.z;
-        float* dst = partial_acc + slot * D + d4;
+        if (fused.unmerged) {
+          bf16_t* dst = (bf16_t*)partial_acc + slot * D + d4;
+          const float inverse = total > 0.f ? 1.f / total : 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dst[i] = merged[i];
+          for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
+        } else {
+          float* dst = partial_acc + slot * D + d4;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[i] = merged[i];
+        }
         if (d4 == 0) {
           partial_ml[slot * 2] = best;
           partial_ml[slot * 2 + 1] = total;
@@ -841,6 +852,9 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // of the step must lie in one of the tiles: a second kernel merges the splits of all rows.
 // With `fuse` tile i is row i, the one token of request i (`work` is not read), qkv is as the projection left it, and the kernel
 // rotates (table of cos and sin per row, pairing) and stores the token's key and value at slots[row] itself.
+// `fuse` + 2 leaves the key splits unmerged for a reader that merges them itself (gemm_merged): partial_acc is
+// then bfloat16 [rows * heads * splits * D], each split's result divided by its own sum of weights, and
+// partial_ml holds each split's maximum (in units of log2) and sum of weights as before.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
                                         float* partial_ml, void* keys, void* values,
                                         const int* block_tables, int table_width, const int* positions,
@@ -854,7 +868,9 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   if ((long)kv_heads * page_size * D >= (1L << 31)) return ERR_BAD_ARGUMENT;  // a page's elements are counted in 32 bits
   const int group = heads / kv_heads;
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
-  FusedDecode fused = {(const float2*)table, pairing, slots};
+  const bool unmerged = (fuse & 2) != 0 && splits > 1;  // the splits stay as they are: whoever reads them merges them
+  fuse &= 1;
+  FusedDecode fused = {(const float2*)table, pairing, slots, unmerged ? 1 : 0};
   int status;
   if (fuse) {
     if (column_tiles != 1 || tiles != rows || !slots || !llmserve_attention_can_fuse(pairing) || (pairing != 0 && !table))
@@ -877,7 +893,7 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   } else {
     return ERR_BAD_ARGUMENT;
   }
-  if (status != 0 || splits == 1) return status;
+  if (status != 0 || splits == 1 || unmerged) return status;
   hipLaunchKernelGGL(attention_merge_kernel, dim3(rows * heads), dim3(64), 0, stream, partial_acc, partial_ml,
                      (bf16_t*)out, splits);
   return LAUNCH_STATUS();

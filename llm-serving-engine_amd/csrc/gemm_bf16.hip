@@ -274,6 +274,122 @@ static int launch_pair(const void* x, const void* w, const void* bias, int bias_
   return LAUNCH_STATUS();
 }
 
+// ---------------------------------------------------------------------------- key splits merged on the way in
+// gemm_merged: gemm_skinny for up to 16 rows whose x is the output of decode attention that was left in
+// key splits (attention_bf16.hip, `unmerged`): for every (row, head) S results, each divided by its own sum
+// of weights, with each split's maximum m_s (in units of log2) and sum of weights l_s.  The row's true
+// x[head] = sum_s c_s x_s[head] with c_s = l_s 2^(m_s - m) / sum_t l_t 2^(m_t - m), m the largest m_s.
+// A kernel of its own that merges costs a decode step as much as the attention itself (a launch and two
+// trips to memory); here the lanes that load x for the MFMA's B operand merge as they load.  Heads are
+// 128 wide, a group of K (128 k), so a wave's group is one head and its S coefficients are made once.
+template <int WAVES, int S>
+__global__ __launch_bounds__(WAVES * 64) void gemm_merged_kernel(const bf16_t* __restrict__ split_x,
+                                                                 const float* __restrict__ split_ml,
+                                                                 const bf16_t* __restrict__ w,
+                                                                 const void* __restrict__ bias, int bias_is_float,
+                                                                 float* __restrict__ out, int M, int N, int K,
+                                                                 int k_split) {
+  extern __shared__ float partial[];  // [WAVES][64 lanes][4]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int n = min((int)blockIdx.x * 16 + r, N - 1);
+  const int heads = K / (STEP * GROUP);
+  const int head_first = blockIdx.y * (k_split / (STEP * GROUP));
+  const bf16_t* w_row = w + (size_t)n * K + (size_t)head_first * (STEP * GROUP) + g * 8;
+  const bool x_live = r < M;
+  const int row = min(r, M - 1);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  const bool with_bias = bias && blockIdx.y == 0;
+  float bias_here[4] = {0.f, 0.f, 0.f, 0.f};
+  if (with_bias) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      bias_here[i] = load_as_float(bias, bias_is_float, min((int)blockIdx.x * 16 + g * 4 + i, N - 1));
+  }
+  const int groups = k_split / (STEP * GROUP);
+  for (int group = wave; group < groups; group += WAVES) {
+    bf16x8 a[GROUP];
+#pragma unroll
+    for (int u = 0; u < GROUP; ++u) a[u] = load8_stream(w_row + (group * GROUP + u) * STEP);
+    const size_t slot = ((size_t)row * heads + head_first + group) * S;
+    float2 ml[S];
+    bf16x8 piece[S][GROUP];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      ml[s] = *(const float2*)(split_ml + (slot + s) * 2);
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u) piece[s][u] = load8(split_x + (slot + s) * (STEP * GROUP) + u * STEP + g * 8);
+    }
+    float best = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < S; ++s) best = fmaxf(best, ml[s].x);
+    float share[S], total = 0.f;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      share[s] = ml[s].x == -INFINITY ? 0.f : ml[s].y * __builtin_amdgcn_exp2f(ml[s].x - best);  // a split that saw no key
+      total += share[s];
+    }
+    const float inverse = total > 0.f ? 1.f / total : 0.f;
+#pragma unroll
+    for (int u = 0; u < GROUP; ++u) {
+      float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+        const float c = share[s] * inverse;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = fmaf(c, share[s] > 0.f ? (float)piece[s][u][i] : 0.f, x[i]);
+      }
+      bf16x8 b;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) b[i] = x_live ? (bf16_t)x[i] : (bf16_t)0.f;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc, 0, 0, 0);
+    }
+  }
+  *(f32x4*)(partial + (wave * 64 + lane) * 4) = acc;
+  __syncthreads();
+  if (wave > 0) return;
+  f32x4 total_tile = {0.f, 0.f, 0.f, 0.f};
+  for (int v = 0; v < WAVES; ++v) total_tile += *(const f32x4*)(partial + (v * 64 + lane) * 4);
+  const int n_first = blockIdx.x * 16 + g * 4;
+  if (r >= M) return;
+  float* dst = out + ((size_t)blockIdx.y * M + r) * N + n_first;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (n_first + i < N) dst[i] = total_tile[i] + bias_here[i];
+}
+
+template <int S>
+static int launch_merged(const void* split_x, const float* split_ml, const void* w, const void* bias, int bias_is_float,
+                         float* out, int M, int N, int K, int k_splits, hipStream_t stream) {
+  const int groups = K / k_splits / (STEP * GROUP);
+  const dim3 grid((N + 15) / 16, k_splits);
+  if (groups <= 4)
+    hipLaunchKernelGGL((gemm_merged_kernel<4, S>), grid, dim3(256), 4 * 64 * 4 * sizeof(float), stream,
+                       (const bf16_t*)split_x, split_ml, (const bf16_t*)w, bias, bias_is_float, out, M, N, K, K / k_splits);
+  else
+    hipLaunchKernelGGL((gemm_merged_kernel<8, S>), grid, dim3(512), 8 * 64 * 4 * sizeof(float), stream,
+                       (const bf16_t*)split_x, split_ml, (const bf16_t*)w, bias, bias_is_float, out, M, N, K, K / k_splits);
+  return LAUNCH_STATUS();
+}
+
+// out [k_splits, M, N] float32 partial sums of x . w^T (+ bias in the first), x [M, K] being the merge of
+// split_x bfloat16 [M, K / 128, splits, 128] with split_ml float32 [M, K / 128, splits, 2] as above.
+// M <= 16; K a multiple of 128 * k_splits; splits 2, 3, 4, 6 or 8.
+extern "C" int llmserve_gemm_merged(const void* split_x, const float* split_ml, int splits, const void* w,
+                                    const void* bias, int bias_is_float, float* out, int M, int N, int K,
+                                    int k_splits, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K <= 0 || k_splits < 1 || K % (STEP * GROUP * k_splits)) return ERR_BAD_ARGUMENT;
+  switch (splits) {
+    case 2: return launch_merged<2>(split_x, split_ml, w, bias, bias_is_float, out, M, N, K, k_splits, stream);
+    case 3: return launch_merged<3>(split_x, split_ml, w, bias, bias_is_float, out, M, N, K, k_splits, stream);
+    case 4: return launch_merged<4>(split_x, split_ml, w, bias, bias_is_float, out, M, N, K, k_splits, stream);
+    case 6: return launch_merged<6>(split_x, split_ml, w, bias, bias_is_float, out, M, N, K, k_splits, stream);
+    case 8: return launch_merged<8>(split_x, split_ml, w, bias, bias_is_float, out, M, N, K, k_splits, stream);
+    default: return ERR_BAD_ARGUMENT;
+  }
+}
+
 // ---------------------------------------------------------------------------- 16 < M <= 64
 // gemm_medium: the same product for up to 64 rows of x.  With more than one 16-row tile of x,
 // loading x per wave would cost more than streaming the weights, so a workgroup takes 64

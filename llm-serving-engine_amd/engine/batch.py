@@ -59,6 +59,10 @@ class StepBatch:
     max_query_length: int
     max_context_length: int
     every_row_wanted: bool = False  # logit_rows is 0, 1, ..., T - 1 (a step of single tokens): nothing to gather
+    # (tokens, requests) that the arrays are padded to when the step's kernels are captured into a graph for
+    # replay with other steps of the same padded shape: the arrays hold rows beyond the real ones (tokens that
+    # are stored nowhere and whose results nobody reads, requests without tokens), `chunks` only the real requests.
+    padded_to: tuple[int, int] | None = None
     # Kernel libraries may keep here what they derive from the step's shape on the host (work
     # lists: built once, used by every layer, and still valid when a captured step is replayed) ...
     scratch: dict[str, Any] = field(default_factory=dict)

@@ -306,6 +306,8 @@ class EngineCore:
         }
         if any(self._device_spans.values()):
             torch.cuda.synchronize(self.runner.device)
+        for how, count in getattr(self.runner, "step_counts", {}).items():
+            stats[f"steps_{how}"] = count  # replayed from a graph, captured into one, launched kernel by kernel
         for phase in _PHASES:
             stats[f"{phase}_iterations"] = self._iterations[phase]
             stats[f"{phase}_cpu_ms"] = self._host_ms[phase]

@@ -43,28 +43,46 @@ def _pack_step(
     *,
     pad_to: int | None = None,
     width: int | None = None,
+    pad_tokens_to: int | None = None,
+    pad_rows_to: int | None = None,
 ) -> tuple[np.ndarray, list[int], list[int], dict]:
     """The step's index arrays as one int32 array: token ids, positions, request index per
     token, query starts, context lengths, state slots, wanted rows, then per cache group the
-    slot of every token and the requests' block-table rows.  With `pad_to`, requests are
-    padded to that many (one token each, stored nowhere, reading page 0), for a captured graph."""
+    slot of every token and the requests' block-table rows.  Padding, for a captured graph: with
+    `pad_to`, requests are padded to that many; a padding request brings one token, or, with
+    `pad_tokens_to`, the first of them brings all the tokens that are missing to that count and the
+    others none.  Padding tokens are stored nowhere and read page 0.  `pad_rows_to` pads the wanted
+    rows (with row 0); without it a padded step wants every request's row."""
     counts = np.array([r.count for r in reservations], dtype=np.int64)
     requests = len(reservations)
     padded = pad_to if pad_to is not None else requests
-    extra = padded - requests
-    total = int(counts.sum()) + extra
+    if pad_tokens_to is None:
+        padding = np.ones(padded - requests, np.int64)
+    else:
+        padding = np.zeros(padded - requests, np.int64)
+        missing = pad_tokens_to - int(counts.sum())
+        if missing < 0 or (missing > 0 and padded == requests):
+            raise ValueError("the step does not fit the shape it is padded to")
+        if missing:
+            padding[0] = missing
+    extra = int(padding.sum())
+    all_counts = np.concatenate([counts, padding])
+    total = int(all_counts.sum())
     query_start = np.zeros(padded + 1, dtype=np.int32)
-    query_start[1:] = np.cumsum(np.concatenate([counts, np.ones(extra, np.int64)]))
+    query_start[1:] = np.cumsum(all_counts)
     token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries] + [np.zeros(extra, np.int32)])
     positions = np.concatenate(
         [np.arange(r.start, r.start + r.count, dtype=np.int32) for r in reservations] + [np.zeros(extra, np.int32)]
     )
-    token_sequence = np.repeat(np.arange(padded, dtype=np.int32), np.concatenate([counts, np.ones(extra, np.int64)]))
-    context = np.array([r.start + r.count for r in reservations] + [1] * extra, dtype=np.int32)
-    slots = np.array([r.slot for r in reservations] + [0] * extra, dtype=np.int32)
+    token_sequence = np.repeat(np.arange(padded, dtype=np.int32), all_counts)
+    context = np.array([r.start + r.count for r in reservations] + [1] * (padded - requests), dtype=np.int32)
+    slots = np.array([r.slot for r in reservations] + [0] * (padded - requests), dtype=np.int32)
     rows = [query_start[b] + np.asarray(e.want, dtype=np.int32) for b, e in enumerate(entries)]
     logit_rows = np.concatenate(rows).astype(np.int32) if rows else np.zeros(0, np.int32)
-    if pad_to is not None:
+    wanted = int(logit_rows.size)
+    if pad_rows_to is not None:
+        logit_rows = np.concatenate([logit_rows, np.zeros(pad_rows_to - wanted, np.int32)])
+    elif pad_to is not None:
         logit_rows = np.arange(padded, dtype=np.int32)
     pieces = [token_ids, positions, token_sequence, query_start, context, slots, logit_rows]
     widths = []
@@ -82,6 +100,7 @@ def _pack_step(
     facts = {
         "num_tokens": total,
         "num_logit_rows": int(logit_rows.size),
+        "wanted": wanted,
         "every_row_wanted": bool(logit_rows.size == total and np.array_equal(logit_rows, np.arange(total, dtype=np.int32))),
         "max_query_length": int(counts.max()),
         "max_context_length": int(context.max()),
@@ -91,7 +110,8 @@ def _pack_step(
 
 
 def _view_step(
-    on_device: torch.Tensor, sizes: list[int], widths: list[int], facts: dict, chunks: list[SequenceChunk], page_size: int
+    on_device: torch.Tensor, sizes: list[int], widths: list[int], facts: dict, chunks: list[SequenceChunk], page_size: int,
+    padded_to: tuple[int, int] | None = None,
 ) -> StepBatch:
     views = list(torch.split(on_device, sizes))
     groups = []
@@ -113,6 +133,7 @@ def _view_step(
         every_row_wanted=facts.get("every_row_wanted", False),
         max_query_length=facts["max_query_length"],
         max_context_length=facts["max_context_length"],
+        padded_to=padded_to,
     )
 
 
@@ -131,7 +152,7 @@ def build_step_batch(
 
 @dataclass
 class _DecodeGraph:
-    """One captured decode step: `requests` single tokens against block tables `width` wide."""
+    """One captured step: `requests` requests (in a decode step one token each) against block tables `width` wide."""
 
     requests: int
     width: int
@@ -183,6 +204,14 @@ class ModelRunner:
         self.use_graphs = self.use_graphs and self.model.replayable  # a part that looks at values on the host is not replayed
         self._graphs: dict[tuple[int, int], _DecodeGraph] = {}  # in order of last use, the latest last
         self.max_graphs = 24  # each holds only a step's activations
+        # Steps that are not single tokens (prompt portions, portions beside decoded tokens) are captured too,
+        # by padded shape, up to this many tokens: below it the host's launches take longer than the device's
+        # work.  A shape is captured when it comes for the second time.
+        self.graph_token_limit = 512
+        self.max_step_graphs = 48
+        self._step_graphs: dict[tuple, _DecodeGraph] = {}
+        self._shape_seen: dict[tuple, int] = {}
+        self.step_counts = {"replayed": 0, "captured": 0, "launched": 0}  # how steps reached the device
         self.packing_ms = 0.0  # host time spent on the steps' index arrays
         # What `prepare_decode` has done for the step to come: each request's reservation of one
         # token, and, where decode steps replay a graph, the step's index arrays already packed.
@@ -192,9 +221,10 @@ class ModelRunner:
     def close(self) -> None:
         """Drops the captured graphs (while the device runtime is still up)."""
         self._packed_ahead = None
-        if self._graphs:
+        if self._graphs or self._step_graphs:
             torch.cuda.synchronize(self.device)
         self._graphs.clear()
+        self._step_graphs.clear()
 
     def add_request(self, request_id: str) -> int:
         return self.cache.create(request_id)
@@ -333,6 +363,10 @@ class ModelRunner:
             if packed_ahead is not None and packed_ahead[0] == tuple(entry.request_id for entry in entries):
                 return self._decode_with_graph(reservations, entries, packed_ahead[1:])
             return self._decode_with_graph(reservations, entries)
+        if self.use_graphs and not self.cache.states:
+            logits = self._step_with_graph(reservations, entries)
+            if logits is not None:
+                return logits
         started = time.perf_counter()
         batch = build_step_batch(reservations, entries, self.cache, self.device)
         self.packing_ms += 1000.0 * (time.perf_counter() - started)
@@ -387,6 +421,7 @@ class ModelRunner:
         else:
             key, packed, sizes, widths, facts = self._pack_decode(reservations, entries)
         graph = self._graphs.pop(key, None)
+        self.step_counts["replayed" if graph is not None else "captured"] += 1
         if graph is None:
             graph = self._capture(key, packed, sizes, widths, facts)
         self._graphs[key] = graph  # the one used last stands last
@@ -403,6 +438,98 @@ class ModelRunner:
             graph.static[: len(reservations)].copy_(device_tokens)
         graph.graph.replay()
         return graph.logits[: len(reservations)]
+
+    # ------------------------------------------------------------------ captured steps of any shape
+
+    @staticmethod
+    def _token_bucket(tokens: int) -> int:
+        for size in (16, 32, 64, 96, 128, 192, 256, 384, 512, 768, 1024):
+            if tokens <= size:
+                return size
+        return -(-tokens // 512) * 512
+
+    @torch.inference_mode()
+    def _step_with_graph(self, reservations: list[Reservation], entries: list[StepEntry]) -> torch.Tensor | None:
+        """A step of any mix of portions and single tokens, replayed from a HIP graph of its padded shape:
+        tokens rounded up to a bucket (the padding belongs to one request more, stored nowhere, read by
+        nobody), requests and block-table width to powers of two, the wanted rows to the requests' bucket.
+        The kernel library pads its own work lists likewise and makes them anew for every replay
+        (`refresh_step`).  Returns None where the step is launched kernel by kernel instead: a kernel library
+        without that hook, more tokens than `graph_token_limit`, or a shape that has not come twice yet."""
+        if not hasattr(self.kernels, "refresh_step"):
+            return None
+        tokens = sum(r.count for r in reservations)
+        if tokens > self.graph_token_limit:
+            self.step_counts["launched"] += 1
+            return None
+        started = time.perf_counter()
+        wanted = sum(len(e.want) for e in entries)
+        padded_tokens = self._token_bucket(tokens)
+        requests = self._bucket(len(reservations) + 1)  # one more: the request that owns the padding tokens
+        blocks = max(-(-(r.start + r.count) // self.cache.page_size) for r in reservations)
+        width = min(self._bucket(blocks), self._bucket(self.cache.max_blocks_per_sequence))
+        rows = 0 if wanted == 0 else requests  # wanted rows are padded to the requests' bucket: fewer shapes
+        key = (padded_tokens, requests, width, rows)
+        graph = self._step_graphs.pop(key, None)
+        if graph is None:
+            seen = self._shape_seen.get(key, 0) + 1
+            self._shape_seen[key] = seen
+            if seen < 2:
+                self.step_counts["launched"] += 1
+                return None
+        self.step_counts["replayed" if graph is not None else "captured"] += 1
+        packed, sizes, widths, facts = _pack_step(
+            reservations, entries, self.cache, pad_to=requests, width=width, pad_tokens_to=padded_tokens, pad_rows_to=rows
+        )
+        chunks = [SequenceChunk(r.request_id, r.slot, r.start, r.count) for r in reservations]
+        self.packing_ms += 1000.0 * (time.perf_counter() - started)
+        if graph is None:
+            graph = self._capture_step(key, packed, sizes, widths, facts, chunks)
+        self._step_graphs[key] = graph  # the one used last stands last
+        turn = graph.turn
+        graph.turn = 1 - turn
+        if graph.copied[turn] is not None:
+            graph.copied[turn].synchronize()  # the staging buffer's last copy has left it
+        graph.host[turn].copy_(torch.from_numpy(packed))
+        graph.static.copy_(graph.host[turn], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        graph.copied[turn] = event
+        graph.batch.chunks = chunks
+        self.kernels.refresh_step(graph.batch)
+        graph.graph.replay()
+        if wanted == 0:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        return graph.logits[:wanted]
+
+    def _capture_step(self, key, packed, sizes, widths, facts, chunks) -> _DecodeGraph:
+        padded_tokens, requests, width, rows = key
+        if len(self._step_graphs) >= self.max_step_graphs:
+            torch.cuda.synchronize(self.device)  # a replay of the graph that goes may still be queued
+            self._step_graphs.pop(next(iter(self._step_graphs)))
+        static = torch.from_numpy(packed).to(self.device)
+        # what decides which kernels run, and with how many workgroups, is the padded shape and never the step
+        facts = dict(facts, max_context_length=width * self.cache.page_size, max_query_length=padded_tokens,
+                     every_row_wanted=False)
+        batch = _view_step(static, sizes, widths, facts, chunks, self.cache.page_size, padded_to=(padded_tokens, requests))
+        stream = torch.cuda.Stream(self.device)
+        stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(stream), self._stream_scope():
+            self._forward_batch(batch)  # loads libraries, builds the work lists kept on `batch`
+        torch.cuda.current_stream(self.device).wait_stream(stream)
+        torch.cuda.synchronize(self.device)
+        batch.computed.clear()  # what kernels computed from the warm-up's values is recorded anew
+        captured = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(captured), self._stream_scope():
+            logits = self._forward_batch(batch)
+        host = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        return _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)
+
+    def _forward_batch(self, batch: StepBatch) -> torch.Tensor | None:
+        if batch.num_logit_rows == 0:
+            self.model.forward_without_logits(batch, self.cells)
+            return None
+        return self.model.forward(batch, self.cells)
 
     def _capture(self, key, packed, sizes, widths, facts) -> _DecodeGraph:
         requests, width = key

@@ -53,6 +53,7 @@ _SIGNATURES = {
     "llmserve_gemm_generic": "pipipipiiiip",
     "llmserve_gemm_skinny": "pppipiiiiiip",
     "llmserve_gemm_medium": "pppipiiiiiip",
+    "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
     "llmserve_gemm_wide": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifip",
@@ -133,6 +134,7 @@ class HipKernels:
         self.library_products = library_products
         self.shared_portions = shared_portions
         self.wide_products = wide_products
+        self.merge_in_product = True  # decode attention leaves its key splits to the product that reads them
         name = torch.cuda.get_device_properties(self.device).gcnArchName
         if not name.startswith("gfx950"):
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
@@ -466,37 +468,77 @@ class HipKernels:
             self._attention_bf16[head_dim] = _declared(load_module("attention_bf16", {"HEAD_DIM": head_dim}))
         return self._attention_bf16[head_dim]
 
+    @staticmethod
+    def _work_items(chunks, group: int, column_tiles: int, longer_than: int, up_to: int | None):
+        """Work items (request, first row, first head, columns), int32 [items, 4], for the requests of
+        the step whose token count lies in (longer_than, up_to], and about how many 32-key steps the
+        items walk all together.  With up to 16 query heads a kv head (`group`) an item is a run of
+        `column_tiles` * 16 (token, head) pairs of a request, token by token and head by head, wherever
+        in a token it begins; with more, `column_tiles` tokens (and "columns" counts tokens)."""
+        import numpy as np
+
+        counts = np.array([chunk.count for chunk in chunks], dtype=np.int64)
+        starts = np.concatenate([[0], np.cumsum(counts)[:-1]])
+        chosen = counts > longer_than
+        if up_to is not None:
+            chosen &= counts <= up_to
+        which = np.nonzero(chosen)[0]
+        packed = group <= 16
+        per_token = group if packed else 1
+        per_item = column_tiles * (16 if packed else 1)
+        totals = counts[which] * per_token
+        items = -(-totals // per_item)
+        request = np.repeat(which, items)
+        inside = np.arange(int(items.sum())) - np.repeat(np.cumsum(items) - items, items)
+        first = inside * per_item
+        columns = np.minimum(per_item, np.repeat(totals, items) - first)
+        work = np.stack([request, starts[request] + first // per_token, first % per_token, columns], axis=1).astype(np.int32)
+        begins = np.array([chunk.start for chunk in chunks], dtype=np.int64)[which]
+        steps = int((items * ((begins + counts[which] / 2) / 32 + 1)).sum())
+        return work, steps
+
+    @staticmethod
+    def _work_capacity(padded_to: tuple[int, int], group: int, column_tiles: int) -> int:
+        """The most items a work list can have in a step of `padded_to` = (tokens, requests)."""
+        tokens, requests = padded_to
+        per_token = group if group <= 16 else 1
+        per_item = column_tiles * (16 if group <= 16 else 1)
+        return -(-tokens * per_token // per_item) + requests
+
     def _attention_work(self, batch, group: int, column_tiles: int, longer_than: int, up_to: int | None):
-        """Work items (request, first row, first head, columns) for the requests of the step whose
-        token count lies in (longer_than, up_to].  With up to 16 query heads a kv head (`group`) an
-        item is a run of `column_tiles` * 16 (token, head) pairs of a request, token by token and
-        head by head, wherever in a token it begins; with more, `column_tiles` tokens (and
-        "columns" counts tokens).  Built once per step and kept on the batch."""
+        """The work list of `_work_items` on the device, built once per step and kept on the batch:
+        (tensor or None, items, steps).  A batch that is `padded_to` (tokens, requests) for a captured
+        step gets a list of the most items such a step can have, the unused ones of no columns: the
+        captured launch covers whatever step is replayed, once `refresh_step` has filled in its items."""
         key = ("attention_work", group, column_tiles, longer_than, up_to)
         if key not in batch.scratch:
-            import numpy as np
+            work, steps = self._work_items(batch.chunks, group, column_tiles, longer_than, up_to)
+            padded_to = getattr(batch, "padded_to", None)
+            if padded_to is not None:
+                import numpy as np
 
-            counts = np.array([chunk.count for chunk in batch.chunks], dtype=np.int64)
-            starts = np.concatenate([[0], np.cumsum(counts)[:-1]])
-            chosen = counts > longer_than
-            if up_to is not None:
-                chosen &= counts <= up_to
-            which = np.nonzero(chosen)[0]
-            packed = group <= 16
-            per_token = group if packed else 1
-            per_item = column_tiles * (16 if packed else 1)
-            totals = counts[which] * per_token
-            items = -(-totals // per_item)
-            request = np.repeat(which, items)
-            inside = np.arange(int(items.sum())) - np.repeat(np.cumsum(items) - items, items)
-            first = inside * per_item
-            columns = np.minimum(per_item, np.repeat(totals, items) - first)
-            work = np.stack([request, starts[request] + first // per_token, first % per_token, columns], axis=1).astype(np.int32)
-            # about how many 32-key steps the items walk, all together
-            begins = np.array([chunk.start for chunk in batch.chunks], dtype=np.int64)[which]
-            steps = int((items * ((begins + counts[which] / 2) / 32 + 1)).sum())
+                capacity = self._work_capacity(padded_to, group, column_tiles)
+                if len(work) > capacity:
+                    raise KernelError("a step holds more attention work than its padded shape allows")
+                work = np.concatenate([work, np.zeros((capacity - len(work), 4), np.int32)])
             batch.scratch[key] = (self.to_device(torch.from_numpy(work)) if len(work) else None, len(work), steps)
         return batch.scratch[key]
+
+    def refresh_step(self, batch) -> None:
+        """For a batch whose kernels were captured: `batch.chunks` now describes another step of the
+        same padded shape; everything this library derived from the chunks on the host (the attention
+        work lists) is made anew, in place, at the addresses the captured kernels read."""
+        import numpy as np
+
+        for key, (tensor, capacity, _) in batch.scratch.items():
+            if key[0] != "attention_work" or tensor is None:
+                continue
+            work, _ = self._work_items(batch.chunks, *key[1:])
+            if len(work) > capacity:
+                raise KernelError("a step holds more attention work than the captured step has room for")
+            padded = np.zeros((capacity, 4), np.int32)
+            padded[: len(work)] = work
+            tensor.copy_(torch.from_numpy(padded), non_blocking=False)
 
     def paged_attention(self, qkv, layout, batch, cell, scale: float, window: int | None) -> torch.Tensor:
         tokens = qkv.shape[0]
@@ -517,11 +559,13 @@ class HipKernels:
         _check(status, "paged_attention")
         return out
 
-    def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None) -> None:
+    def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None, unmerged=False):
         """The MFMA kernel: requests that bring a few tokens (decoding) one column tile per
         wave, split over the keys when there are few of them; longer portions two or four
         tiles per wave.  `fuse` = (rotary table, pairing) lets a step of single tokens rotate and
-        store inside the same kernel."""
+        store inside the same kernel.  With `unmerged` (a step of single tokens whose reader merges
+        key splits itself) the keys are split more finely and the splits are returned as they are,
+        (bfloat16 [T, heads, splits, D], float32 [T, heads, splits, 2], splits), instead of `out`."""
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
         per_tile = max(1, 16 // (heads // kv_heads))
@@ -530,7 +574,8 @@ class HipKernels:
         group_size = heads // kv_heads
         launches = [(1, *self._attention_work(batch, group_size, 1, 0, per_tile)[:2])]
         shared = False
-        if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never":
+        padded = getattr(batch, "padded_to", None) is not None  # a captured step: the same launches whatever it holds
+        if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never" and not padded:
             # Prompt portions at this head size may go to the kernel whose waves share each step's K and V
             # through LDS (a quarter of the cache traffic).  Its workgroups walk all their keys step after
             # step, so it needs several workgroups a CU to be ahead: long prompts, or many of them.
@@ -566,23 +611,51 @@ class HipKernels:
                 blocks = items * kv_heads * head_tiles
                 steps = -(-batch.max_context_length // 32)
                 splits = max(1, min(-(-steps // 32), max(1, 2048 // blocks), 64))
+                if unmerged:
+                    # Nothing merges in a kernel of its own here, so a split costs only what its reader pays to
+                    # read it (about 0.8 us a split in the product): a workgroup's eight waves get one step each.
+                    # Attention and product together at 8 rows of the 1.5B sizes, captured, against 15.3 us
+                    # unsplit at 530 keys and 22.1 at 1,000: two splits 14.5 and 18.6, four 14.7 and 16.5, eight
+                    # 17.0 and 17.8.
+                    # The product takes up to eight splits.  Where the walk is so long that more are wanted
+                    # even at 32 steps a split (beyond 8,192 keys), the kernel that merges is a small share of
+                    # it and that way stays (8 rows of the 1.5B sizes, a whole step: 8,192 keys 2.46 ms with the
+                    # merging kernel, 2.32 with eight splits merged by the product; 30,000 keys 2.62 and 2.92).
+                    if splits <= 8:
+                        wanted = min(-(-steps // 8), max(1, 1024 // blocks), 8)
+                        splits = next(allowed for allowed in (1, 2, 3, 4, 6, 8) if allowed >= wanted)
+                    else:
+                        unmerged = False
                 if splits > 1:
-                    partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), torch.float32)
+                    partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), qkv.dtype if unmerged else torch.float32)
                     partial_ml = self._empty((tokens * heads * splits * 2,), torch.float32)
             table, pairing = fuse if fuse is not None else (None, "none")
             status = library.llmserve_attention_tiles(
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
                 _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
-                group.page_size, scale, window, splits, 1 if fuse is not None else 0,
+                group.page_size, scale, window, splits, (1 if fuse is not None else 0) + (2 if unmerged else 0),
                 _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), self._stream,
             )
             _check(status, "paged_attention")
+            if unmerged and splits > 1:
+                return partial_acc, partial_ml, splits
+        return None
 
     def rotate_store_attend(
-        self, qkv, layout, batch, cell, inverse_frequencies, pairing: str, scale: float, window: int | None
+        self, qkv, layout, batch, cell, inverse_frequencies, pairing: str, scale: float, window: int | None,
+        project: LinearWeights | None = None,
     ) -> torch.Tensor:
         """`rotate_and_store` followed by `paged_attention`; one kernel when every request of
-        the step brings a single token and the MFMA kernel takes the sizes."""
+        the step brings a single token and the MFMA kernel takes the sizes.  With `project`, the result
+        is `linear(that, project, float32, partial=True)`: for up to 16 single tokens at head size 128
+        the attention leaves its key splits unmerged and the product merges them as it loads its x."""
+        out = self._rotate_store_attend(qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window, project)
+        if project is None or out.dtype == torch.float32:
+            return out
+        return self.linear(out, project, out_dtype=torch.float32, partial=True)
+
+    def _rotate_store_attend(self, qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window, project):
+        """The attention's output, or, where the key splits were left to the product, the product's."""
         group = batch.groups[cell.group]
         dim = layout.head_dim
         if (
@@ -597,8 +670,30 @@ class HipKernels:
         ):
             out = self._empty((qkv.shape[0], layout.num_heads * dim), qkv.dtype)
             table = self.rotary_table(batch, inverse_frequencies) if pairing != "none" else None
-            self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), fuse=(table, pairing))
-            return out
+            rows = qkv.shape[0]
+            merging = (
+                project is not None
+                and self.merge_in_product
+                and dim == 128
+                and rows <= 16
+                and project.weight.dtype == torch.bfloat16
+                and project.in_features == layout.num_heads * dim
+            )
+            left = self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), fuse=(table, pairing), unmerged=merging)
+            if left is None:
+                return out
+            split_x, split_ml, splits = left
+            k_splits = self._partial_splits(project.out_features, project.in_features)
+            shape = (rows, project.out_features) if k_splits == 1 else (k_splits, rows, project.out_features)
+            result = self._empty(shape, torch.float32)
+            bias = project.bias
+            status = self._gemm_bf16.llmserve_gemm_merged(
+                _pointer(split_x), _pointer(split_ml), splits, _pointer(project.weight), _pointer(bias),
+                _is_float(bias) if bias is not None else 0, _pointer(result), rows, project.out_features,
+                project.in_features, k_splits, self._stream,
+            )
+            _check(status, "linear over unmerged key splits")
+            return result
         self.rotate_and_store(qkv, layout, batch, cell, inverse_frequencies, pairing)
         return self.paged_attention(qkv, layout, batch, cell, scale, window)
 

@@ -56,8 +56,11 @@ class Kernels(Protocol):
     def rotate_store_attend(
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any,
         inverse_frequencies: torch.Tensor | None, pairing: str, scale: float, window: int | None,
+        project: Any = None,
     ) -> torch.Tensor:
-        """`rotate_and_store` followed by `paged_attention` (a library may fuse them)."""
+        """`rotate_and_store` followed by `paged_attention` (a library may fuse them); with `project` (what
+        `prepare_linear` returned), followed by `linear(that, project, float32, partial=True)`, whose result
+        is returned instead (a library may let that product finish what the attention left undone)."""
 
     def gather_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
         """float32 (hidden + delta)[rows]."""

@@ -87,7 +87,8 @@ class Attention(Mixer):
 
     def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
         qkv = self.kernels.linear(x, self.qkv)
-        mixed = self.position.encode_store_attend(
-            qkv, self.layout, batch, cell, self.spec.scale, self.spec.window
+        # the output projection goes with the attention: a kernel library may fuse the two (key splits of
+        # a decode step merged by the product that reads them)
+        return self.position.encode_store_attend(
+            qkv, self.layout, batch, cell, self.spec.scale, self.spec.window, project=self.out
         )
-        return self.kernels.linear(mixed, self.out, out_dtype=torch.float32, partial=True)

@@ -41,11 +41,15 @@ class PositionEncoding(Part):
         position and, if `cell` is writable, stores k and v in the cell's pages."""
         raise NotImplementedError
 
-    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window) -> "torch.Tensor":
-        """`encode_and_store`, then attention over the cell's pages.  An encoding that
-        a kernel can apply on the way (rotary) overrides this to let the kernel library fuse the two."""
+    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window, project=None) -> "torch.Tensor":
+        """`encode_and_store`, then attention over the cell's pages; with `project` (a prepared linear),
+        then that product of the result, in float32, possibly as partial sums.  An encoding that a kernel
+        can apply on the way (rotary) overrides this to let the kernel library fuse what it can."""
         self.encode_and_store(qkv, layout, batch, cell)
-        return self.kernels.paged_attention(qkv, layout, batch, cell, scale, window)
+        mixed = self.kernels.paged_attention(qkv, layout, batch, cell, scale, window)
+        if project is None:
+            return mixed
+        return self.kernels.linear(mixed, project, out_dtype=torch.float32, partial=True)
 
 
 @POSITIONS.register("rotary")
@@ -73,9 +77,9 @@ class Rotary(PositionEncoding):
             qkv, layout, batch, cell, self.inverse_frequencies, self.spec.pairing
         )
 
-    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window):
+    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window, project=None):
         return self.kernels.rotate_store_attend(
-            qkv, layout, batch, cell, self.inverse_frequencies, self.spec.pairing, scale, window
+            qkv, layout, batch, cell, self.inverse_frequencies, self.spec.pairing, scale, window, project=project
         )
 
 
@@ -86,5 +90,5 @@ class NoPosition(PositionEncoding):
     def encode_and_store(self, qkv, layout: HeadLayout, batch, cell) -> None:
         self.kernels.rotate_and_store(qkv, layout, batch, cell, None, "none")
 
-    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window):
-        return self.kernels.rotate_store_attend(qkv, layout, batch, cell, None, "none", scale, window)
+    def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window, project=None):
+        return self.kernels.rotate_store_attend(qkv, layout, batch, cell, None, "none", scale, window, project=project)

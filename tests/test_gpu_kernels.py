@@ -472,3 +472,41 @@ def test_fused_decode_attention_over_long_contexts(kernels, requests):
         torch.testing.assert_close(got, full, **TOLERANCE[dtype])
         for head in (0, 6):
             torch.testing.assert_close(got[head], rounded(v, dtype)[far, head // 6], atol=0.05, rtol=0.05)
+
+
+@pytest.mark.parametrize("heads,kv_heads,outer,requests", [(12, 2, 1536, 8), (40, 8, 272, 16), (28, 4, 1000, 3), (2, 1, 100, 1)])
+def test_decode_attention_whose_key_splits_the_output_projection_merges(kernels, heads, kv_heads, outer, requests):
+    """A step of up to 16 single tokens at head size 128 followed by the output projection: the attention
+    leaves its key splits unmerged and the product merges them while it loads its x.  Contexts from one
+    key (all splits but one see no key) to thousands, a far key planted to dominate a head; against
+    plain attention followed by the plain product, and against the library's own unfused pair."""
+    from llmserve_amd.kernels import HipKernels
+
+    dtype, dim, page = torch.bfloat16, 128, 16
+    lengths = ([1, 2, 700, 33, 2049, 301, 64, 17, 4100, 530, 65, 1500, 5, 999, 129, 48])[:requests]
+    counts = [1] * requests
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=heads)
+    for q, k, v in per_request:
+        if k.shape[0] > 40:
+            k[k.shape[0] // 3] = 3.0 * q[-1, :: heads // kv_heads]  # the first head of every kv head finds this key
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    weight, bias = torch.randn(outer, heads * dim) / math.sqrt(heads * dim), torch.randn(outer)
+    k = kernels[dtype]
+    project = k.prepare_linear([on_gpu(weight, dtype)], [on_gpu(bias, dtype)])
+    got = k.rotate_store_attend(qkv.clone(), layout, batch, cell, None, "none", 0.3, None, project=project)
+    got = (got if got.ndim == 2 else got.sum(0)).cpu().double()
+    attended = torch.cat([
+        plain.causal_attention(rounded(q, dtype), rounded(key, dtype), rounded(v, dtype), 0.3)[-1:].flatten(1)
+        for q, key, v in per_request
+    ])
+    expected = attended @ rounded(weight, dtype).T + rounded(bias, dtype)
+    # the attention's output is rounded to bfloat16 on its way into the product (once, or twice where splits
+    # are merged): 2^-8 of values of order 1, through a product whose weights have unit row norm
+    torch.testing.assert_close(got, expected, atol=2e-2, rtol=2e-2)
+    apart = HipKernels(dtype)
+    apart.merge_in_product = False
+    other = apart.rotate_store_attend(qkv.clone(), layout, batch, cell, None, "none", 0.3, None, project=project)
+    other = (other if other.ndim == 2 else other.sum(0)).cpu().double()
+    torch.testing.assert_close(got, other, atol=1e-2, rtol=1e-2)
+    assert float((got - expected).abs().mean()) < 1.5 * float((other - expected).abs().mean()) + 1e-4

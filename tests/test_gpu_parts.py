@@ -353,3 +353,35 @@ def test_random_configurations_against_the_plain_forward(tmp_path, kernels, case
             bound = dict(atol=1e-4 * spread, rtol=1e-4) if dtype == torch.float32 else dict(atol=0.2 * spread, rtol=5e-2)
             torch.testing.assert_close(torch.cat(got[i]).cpu().double(), expected[i], **bound, msg=lambda m: f"{config} page {page} request {i}: {m}")
         runner.close()
+
+
+def test_captured_graphs_are_dropped_by_last_use_and_captured_again(model_folders):
+    """More shapes of decode steps than the runner keeps graphs for: the graph used longest ago goes (after
+    the device has finished with it), a shape that comes back is captured again, and every step's logits
+    are the plain forward's whatever was dropped in between."""
+    from llmserve_amd.kernels import HipKernels
+
+    name = "A-loud"
+    config, page = CONFIGS[name]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders[name]), plain.read_weights(model_folders[name])
+    sequences = [random_tokens(40, config.vocab_size, seed=900 + index) for index in range(5)]
+    expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
+    loaded = load_model_folder(model_folders[name], "float32")
+    runner = ModelRunner(loaded, HipKernels(torch.float32), CacheConfig(page, 32, 8))
+    runner.max_graphs = 2
+    runner.step([StepEntry(f"r{index}", tokens[:8], []) for index, tokens in enumerate(sequences)], create_missing=True)
+    fed = [8] * 5
+    seen = []
+    # batches of 1, 2, 3 (padded to 4), 5 (padded to 8) requests, coming back to earlier shapes
+    for group in ([0], [0, 1], [0, 1, 2], [0], [0, 1, 2, 3, 4], [0, 1], [2, 3, 4], [0], [1, 2, 3, 4, 0], [3]):
+        logits = runner.step([StepEntry(f"r{index}", [sequences[index][fed[index]]], [0]) for index in group])
+        for row, index in enumerate(group):
+            torch.testing.assert_close(logits[row].cpu().double(), expected[index][fed[index]], atol=5e-5, rtol=1e-4)
+            fed[index] += 1
+        seen.append(list(runner._graphs))
+        assert len(runner._graphs) <= 2
+    assert seen[0] == [(1, 1)] and seen[1] == [(1, 1), (2, 1)]
+    assert seen[2] == [(2, 1), (4, 1)]  # the third shape pushed out the one used longest ago
+    assert seen[3] == [(4, 1), (1, 1)]  # which was captured again when it came back
+    assert seen[5][-1] == (2, 1) and seen[-1][-1] == (1, 1)
+    runner.close()

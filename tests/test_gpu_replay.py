@@ -206,3 +206,46 @@ def test_captured_steps_of_many_rows_at_benchmark_layer_sizes(wide_models, sizes
                 msg=lambda m: f"request {index} position {at[index]}: {m}",
             )
     runner.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_mixed_steps_at_benchmark_layer_sizes(wide_models, dtype):
+    """Steps that are not single tokens are replayed from graphs of their padded shape once a shape has come
+    twice: portions of prompts beside decoded tokens at the 1.5B widths, the same shape over and over with other
+    requests, lengths and pages in it, steps launched kernel by kernel and waits between the replays (a library
+    call that records a memory clear into a graph shows on replays after the first).  Every step's logits
+    against the plain forward."""
+    from llmserve_amd import CacheConfig, ModelRunner, StepEntry
+    from llmserve_amd.kernels import HipKernels
+    from llmserve_amd.weights import load_model_folder
+
+    WIDE = WIDE_CONFIGS["1.5B"][0]
+    folder, plain_config, weights = wide_models("1.5B")
+    sequences = [random_tokens(150 + 13 * index, WIDE.vocab_size, seed=700 + index) for index in range(5)]
+    expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
+    spread = float(torch.cat(expected).std())
+    walk = math.sqrt(WIDE.intermediate_size) * 2.0 ** -24 * spread
+    bound = dict(atol=5 * walk, rtol=1e-4) if dtype == "float32" else dict(atol=BF16_LARGEST * spread, rtol=3e-2)
+    loaded = load_model_folder(folder, dtype)
+    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(PAGE_WIDE, 80, 8))
+    fed = [0] * 5
+    # requests 0 and 1 are ahead and decode; 2 to 4 bring portions of 16 tokens (the reference's default chunk)
+    runner.step([StepEntry(f"r{index}", sequences[index][:40], []) for index in (0, 1)], create_missing=True)
+    fed[0] = fed[1] = 40
+    for turn in range(9):
+        group = [0, 1] + [2 + (turn + offset) % 3 for offset in range(2)]  # two decoding, two of the three others
+        entries = []
+        for index in group:
+            count = 1 if index < 2 else 16
+            entries.append(StepEntry(f"r{index}", sequences[index][fed[index] : fed[index] + count], [count - 1]))
+        logits = runner.step(entries, create_missing=True).clone()
+        for row, (index, entry) in enumerate(zip(group, entries)):
+            fed[index] += len(entry.tokens)
+            torch.testing.assert_close(logits[row].cpu().double(), expected[index][fed[index] - 1], **bound,
+                                       msg=lambda m: f"turn {turn} request {index} position {fed[index] - 1}: {m}")
+        # between two replays: a step of another shape launched kernel by kernel, and the host waits
+        runner.step([StepEntry("between", random_tokens(40 + turn, WIDE.vocab_size, seed=turn), [0])], create_missing=True)
+        runner.end_request("between")
+        torch.cuda.synchronize()
+    assert any(key[:2] == (64, 8) for key in runner._step_graphs) and runner.step_counts["replayed"] >= 8, runner.step_counts
+    runner.close()

@@ -104,9 +104,10 @@ class TorchKernels:
                 row += 1
         return out.reshape(tokens, heads * dim).to(self.dtype)
 
-    def rotate_store_attend(self, qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window):
+    def rotate_store_attend(self, qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window, project=None):
         self.rotate_and_store(qkv, layout, batch, cell, inverse_frequencies, pairing)
-        return self.paged_attention(qkv, layout, batch, cell, scale, window)
+        mixed = self.paged_attention(qkv, layout, batch, cell, scale, window)
+        return mixed if project is None else self.linear(mixed, project, out_dtype=torch.float32, partial=True)
 
     def gather_rows(self, hidden, delta, rows):
         picked = hidden[rows.long()]
