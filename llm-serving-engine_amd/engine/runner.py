@@ -468,7 +468,9 @@ class ModelRunner:
         requests = self._bucket(len(reservations) + 1)  # one more: the request that owns the padding tokens
         blocks = max(-(-(r.start + r.count) // self.cache.page_size) for r in reservations)
         width = min(self._bucket(blocks), self._bucket(self.cache.max_blocks_per_sequence))
-        rows = 0 if wanted == 0 else requests  # wanted rows are padded to the requests' bucket: fewer shapes
+        # wanted rows are padded to the requests' bucket (a row a request, as serving wants them) or, where more
+        # are wanted, to the tokens' bucket: few shapes
+        rows = 0 if wanted == 0 else requests if wanted <= requests else padded_tokens
         key = (padded_tokens, requests, width, rows)
         graph = self._step_graphs.pop(key, None)
         if graph is None:

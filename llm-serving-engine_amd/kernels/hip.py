@@ -649,13 +649,13 @@ class HipKernels:
         the step brings a single token and the MFMA kernel takes the sizes.  With `project`, the result
         is `linear(that, project, float32, partial=True)`: for up to 16 single tokens at head size 128
         the attention leaves its key splits unmerged and the product merges them as it loads its x."""
-        out = self._rotate_store_attend(qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window, project)
-        if project is None or out.dtype == torch.float32:
+        out, projected = self._rotate_store_attend(qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window, project)
+        if project is None or projected:
             return out
         return self.linear(out, project, out_dtype=torch.float32, partial=True)
 
     def _rotate_store_attend(self, qkv, layout, batch, cell, inverse_frequencies, pairing, scale, window, project):
-        """The attention's output, or, where the key splits were left to the product, the product's."""
+        """(the attention's output, False) or, where the key splits were left to the product, (the product's, True)."""
         group = batch.groups[cell.group]
         dim = layout.head_dim
         if (
@@ -681,7 +681,7 @@ class HipKernels:
             )
             left = self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), fuse=(table, pairing), unmerged=merging)
             if left is None:
-                return out
+                return out, False
             split_x, split_ml, splits = left
             k_splits = self._partial_splits(project.out_features, project.in_features)
             shape = (rows, project.out_features) if k_splits == 1 else (k_splits, rows, project.out_features)
@@ -693,9 +693,9 @@ class HipKernels:
                 project.in_features, k_splits, self._stream,
             )
             _check(status, "linear over unmerged key splits")
-            return result
+            return result, True
         self.rotate_and_store(qkv, layout, batch, cell, inverse_frequencies, pairing)
-        return self.paged_attention(qkv, layout, batch, cell, scale, window)
+        return self.paged_attention(qkv, layout, batch, cell, scale, window), False
 
     # ------------------------------------------------------------------ sampling
 
