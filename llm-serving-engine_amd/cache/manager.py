@@ -117,8 +117,9 @@ class CacheManager:
                 entry = ("pages", group, len(self.groups[group].cells) - 1)
             elif isinstance(need, FixedState):
                 self._state_needs.append(need)
+                # one slot more than there are requests: the state of the requests that pad a captured step
                 self.states.append(
-                    torch.zeros((config.max_sequences, *need.shape), dtype=torch.float32, device=self.device)
+                    torch.zeros((config.max_sequences + 1, *need.shape), dtype=torch.float32, device=self.device)
                 )
                 entry = ("state", len(self.states) - 1, 0)
             else:
@@ -377,6 +378,11 @@ class CacheManager:
     @property
     def capacity_tokens(self) -> int:
         return self.config.num_blocks * self.page_size
+
+    @property
+    def spare_slot(self) -> int:
+        """The state slot of requests that only pad a step to a captured shape: real requests never get it."""
+        return self.config.max_sequences
 
     @property
     def bytes_per_token(self) -> int:

@@ -5,6 +5,10 @@
 // page).  It serves prompt portions and single decoded tokens alike: what differs between
 // them is only how many tokens of a request are in the step.  This is the true 32-bit path
 // and the path for head sizes without an MFMA kernel.
+// Two things may change a score before the softmax, for position encodings and models that want
+// them (the reference has neither): `soft_cap` > 0 squashes it to cap * tanh(score / cap), and
+// `slopes` (one per query head) then adds -slope * (query position - key position), a bias that
+// grows with distance.
 #include "common.h"
 
 #define KEYS_PER_TILE 128
@@ -15,7 +19,7 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, T* __restrict__ out, const T* __restrict__ keys,
     const T* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ token_sequence, const int* __restrict__ positions, int heads, int kv_heads, int dim,
-    int page_size, float scale, int window) {
+    int page_size, float scale, int window, const float* __restrict__ slopes, float soft_cap) {
   __shared__ float query[MAX_DIM];
   __shared__ float weights[KEYS_PER_TILE];
   __shared__ float shared[17];
@@ -28,6 +32,7 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
   __syncthreads();
 
   const int first = window > 0 ? max(0, position - window + 1) : 0;
+  const float slope = slopes ? slopes[head] : 0.f;
   const int per_thread = (dim + KEYS_PER_TILE - 1) / KEYS_PER_TILE;  // output dims per thread, <= 4
   float acc[MAX_DIM / KEYS_PER_TILE] = {};
   float running_max = -INFINITY, running_sum = 0.f;
@@ -41,6 +46,8 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
       float dot = 0.f;
       for (int d = 0; d < dim; ++d) dot = fmaf(query[d], to_float(k[d]), dot);
       score = dot;
+      if (soft_cap > 0.f) score = soft_cap * tanhf(score / soft_cap);
+      score -= slope * (float)(position - key);
     }
     const float tile_max = block_max(score, shared);
     const float next_max = fmaxf(running_max, tile_max);
@@ -76,17 +83,17 @@ extern "C" int llmserve_attention_generic(const void* qkv, int row_width, void* 
                                           const void* values, const int* block_tables, int table_width,
                                           const int* token_sequence, const int* positions, int tokens, int heads,
                                           int kv_heads, int dim, int page_size, float scale, int window,
-                                          hipStream_t stream) {
+                                          const float* slopes, float soft_cap, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (dim > MAX_DIM || dim <= 0 || heads % kv_heads || page_size <= 0) return ERR_BAD_ARGUMENT;
   dim3 grid(tokens, heads);
   if (is_float)
     hipLaunchKernelGGL(attention_generic_kernel<float>, grid, dim3(KEYS_PER_TILE), 0, stream, (const float*)qkv,
                        row_width, (float*)out, (const float*)keys, (const float*)values, block_tables, table_width,
-                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window);
+                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap);
   else
     hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, dim3(KEYS_PER_TILE), 0, stream, (const bf16_t*)qkv,
                        row_width, (bf16_t*)out, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width,
-                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window);
+                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap);
   return LAUNCH_STATUS();
 }

@@ -76,7 +76,7 @@ def _pack_step(
     )
     token_sequence = np.repeat(np.arange(padded, dtype=np.int32), all_counts)
     context = np.array([r.start + r.count for r in reservations] + [1] * (padded - requests), dtype=np.int32)
-    slots = np.array([r.slot for r in reservations] + [0] * (padded - requests), dtype=np.int32)
+    slots = np.array([r.slot for r in reservations] + [cache.spare_slot] * (padded - requests), dtype=np.int32)
     rows = [query_start[b] + np.asarray(e.want, dtype=np.int32) for b, e in enumerate(entries)]
     logit_rows = np.concatenate(rows).astype(np.int32) if rows else np.zeros(0, np.int32)
     wanted = int(logit_rows.size)
@@ -248,7 +248,7 @@ class ModelRunner:
         otherwise costs nothing: reservations of requests it holds are used, the others are
         taken back.  Returns False, having done nothing, if the cache has no room."""
         self._cancel_ahead()
-        if not request_ids or self.cache.states:
+        if not request_ids:
             return False
         plan = [(request_id, 1) for request_id in request_ids]
         if any(request_id not in self.cache.sequences for request_id in request_ids) or not self.cache.fits(plan):
@@ -359,11 +359,11 @@ class ModelRunner:
                 ahead = None
             reservations.append(ahead or self.cache.reserve(request_id, count, checked=True))
         self._cancel_ahead()  # requests that were expected and did not come
-        if self.use_graphs and not self.cache.states and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
+        if self.use_graphs and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
             if packed_ahead is not None and packed_ahead[0] == tuple(entry.request_id for entry in entries):
                 return self._decode_with_graph(reservations, entries, packed_ahead[1:])
             return self._decode_with_graph(reservations, entries)
-        if self.use_graphs and not self.cache.states:
+        if self.use_graphs:
             logits = self._step_with_graph(reservations, entries)
             if logits is not None:
                 return logits
@@ -516,7 +516,7 @@ class ModelRunner:
         batch = _view_step(static, sizes, widths, facts, chunks, self.cache.page_size, padded_to=(padded_tokens, requests))
         stream = torch.cuda.Stream(self.device)
         stream.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(stream), self._stream_scope():
+        with torch.cuda.stream(stream), self._stream_scope(), self._states_kept():
             self._forward_batch(batch)  # loads libraries, builds the work lists kept on `batch`
         torch.cuda.current_stream(self.device).wait_stream(stream)
         torch.cuda.synchronize(self.device)
@@ -526,6 +526,18 @@ class ModelRunner:
             logits = self._forward_batch(batch)
         host = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         return _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)
+
+    @contextlib.contextmanager
+    def _states_kept(self):
+        """A step that is being captured runs twice, once launched to warm up and once replayed.  Keys and values
+        land in the same places both times; a request's fixed-size state would advance twice, so it is put back
+        after the first."""
+        saved = [state.clone() for state in self.cache.states]
+        try:
+            yield
+        finally:
+            for state, before in zip(self.cache.states, saved):
+                state.copy_(before)
 
     def _forward_batch(self, batch: StepBatch) -> torch.Tensor | None:
         if batch.num_logit_rows == 0:
@@ -547,7 +559,7 @@ class ModelRunner:
         batch = _view_step(static, sizes, widths, facts, chunks, self.cache.page_size)
         stream = torch.cuda.Stream(self.device)
         stream.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(stream), self._stream_scope():
+        with torch.cuda.stream(stream), self._stream_scope(), self._states_kept():
             self.model.forward(batch, self.cells)  # loads libraries, builds the work lists kept on `batch`
         torch.cuda.current_stream(self.device).wait_stream(stream)
         torch.cuda.synchronize(self.device)

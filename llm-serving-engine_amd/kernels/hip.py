@@ -56,7 +56,7 @@ _SIGNATURES = {
     "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
     "llmserve_gemm_wide": "pppipiiiiiip",
-    "llmserve_attention_generic": "pipipppippiiiiifip",
+    "llmserve_attention_generic": "pipipppippiiiiifipfp",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
     "llmserve_attention_portions": "pippppippiiiiifip",
     "llmserve_attention_can_fuse": "i",
@@ -540,21 +540,32 @@ class HipKernels:
             padded[: len(work)] = work
             tensor.copy_(torch.from_numpy(padded), non_blocking=False)
 
-    def paged_attention(self, qkv, layout, batch, cell, scale: float, window: int | None) -> torch.Tensor:
+    def paged_attention(
+        self, qkv, layout, batch, cell, scale: float, window: int | None, *,
+        score_slopes: torch.Tensor | None = None, soft_cap: float | None = None,
+    ) -> torch.Tensor:
+        """`score_slopes` (float32 [heads]) and `soft_cap` change the scores before the softmax: cap * tanh(score /
+        cap), then minus slope * distance.  Only the generic kernel takes them: the matrix-core kernels are
+        passed by when either is given."""
         tokens = qkv.shape[0]
         group = batch.groups[cell.group]
         if cell.keys.dtype != qkv.dtype:
             raise KernelError("paged_attention: queries and pages differ in type")
+        if score_slopes is not None and (score_slopes.dtype != torch.float32 or score_slopes.shape != (layout.num_heads,)):
+            raise KernelError("paged_attention: score_slopes is one float32 per query head")
+        if soft_cap is not None and not soft_cap > 0:
+            raise KernelError("paged_attention: soft_cap must be positive")
         out = self._empty((tokens, layout.num_heads * layout.head_dim), qkv.dtype)
         dim = layout.head_dim
-        if qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
+        plain_scores = score_slopes is None and soft_cap is None
+        if plain_scores and qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
             self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0))
             return out
         status = self._attention_generic.llmserve_attention_generic(
             _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
             _pointer(group.block_tables), group.width, _pointer(batch.token_sequence), _pointer(batch.positions),
             tokens, layout.num_heads, layout.num_kv_heads, dim, group.page_size,
-            scale, int(window or 0), self._stream,
+            scale, int(window or 0), _pointer(score_slopes), float(soft_cap or 0.0), self._stream,
         )
         _check(status, "paged_attention")
         return out

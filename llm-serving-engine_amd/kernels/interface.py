@@ -49,9 +49,14 @@ class Kernels(Protocol):
         """Rotary on the q and k heads of `qkv` in place; k and v into the cell's pages if it is writable."""
 
     def paged_attention(
-        self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any, scale: float, window: int | None
+        self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any, scale: float, window: int | None, *,
+        score_slopes: torch.Tensor | None = None, soft_cap: float | None = None,
     ) -> torch.Tensor:
-        """Attention of the q heads of `qkv` over the cell's pages -> [T, heads * head_dim]."""
+        """Attention of the q heads of `qkv` over the cell's pages -> [T, heads * head_dim].
+        Before the softmax a score s of a query at position p for a key at position k may be changed,
+        for encodings and models that want it (Qwen2 wants neither): with `soft_cap`, to
+        soft_cap * tanh(s / soft_cap); with `score_slopes` (float32, one per query head), by
+        - slope * (p - k) after that.  A library refuses what it cannot compute."""
 
     def rotate_store_attend(
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any,

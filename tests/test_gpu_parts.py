@@ -141,6 +141,44 @@ def test_toy_architecture_on_the_gpu(tmp_path, kernels):
         toy.unregister_toy()
 
 
+def test_a_stateful_architecture_is_captured_and_replayed(tmp_path, kernels):
+    """The toy architecture whose mixer keeps a state slot per request and runs on the device alone, with
+    attention whose scores carry a distance bias and a soft cap: its decode steps and its mixed steps are
+    replayed from graphs (the requests that pad a captured step write to a spare state slot, not to a
+    request's), a request that ends hands its slot to the next with the state zeroed, and every logit is the
+    plain forward's, in float32 and in bfloat16."""
+    toy.register_toy()
+    try:
+        folder = toy.write_toy_folder(tmp_path / "sum", config=toy.SUM)
+        sequences = [random_tokens(n, toy.SUM.vocab_size, seed=40 + n) for n in (33, 18, 26)]
+        expected = [toy.plain_toy_forward(folder, tokens) for tokens in sequences]
+        for dtype in DTYPES:
+            loaded = load_model_folder(folder, "float32" if dtype == torch.float32 else "bfloat16")
+            runner = ModelRunner(loaded, kernels[dtype], CacheConfig(block_size=4, num_blocks=40, max_sequences=3))
+            assert runner.use_graphs and runner.cache.states
+            bound = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=0.06 * float(expected[0].std()), rtol=3e-2)
+            fed = [0, 0, 0]
+            for turn in range(12):
+                # request 0 decodes from the start; 1 and 2 bring portions of three tokens, then decode
+                entries = []
+                for index, tokens in enumerate(sequences):
+                    count = 1 if index == 0 or turn >= 5 else 3
+                    if fed[index] + count <= len(tokens):
+                        entries.append((index, StepEntry(f"r{index}", tokens[fed[index] : fed[index] + count], [count - 1])))
+                logits = runner.step([entry for _, entry in entries], create_missing=True).clone()
+                for row, (index, entry) in enumerate(entries):
+                    fed[index] += len(entry.tokens)
+                    torch.testing.assert_close(logits[row].cpu().double(), expected[index][fed[index] - 1], **bound,
+                                               msg=lambda m: f"{dtype} turn {turn} request {index}: {m}")
+            assert runner.step_counts["replayed"] >= 4 and runner.step_counts["captured"] >= 2, runner.step_counts  # mixed and decode steps came from graphs
+            runner.end_request("r1")  # its slot, state zeroed, goes to a new request
+            again = runner.step([StepEntry("new", sequences[1], [len(sequences[1]) - 1])], create_missing=True)
+            torch.testing.assert_close(again[0].cpu().double(), expected[1][-1], **bound)
+            runner.close()
+    finally:
+        toy.unregister_toy()
+
+
 # ------------------------------------------------------------------------------- entry points
 
 

@@ -29,8 +29,8 @@ def test_toy_architecture_steps_like_its_plain_forward(toy_folder):
     cache = runner.cache
     # two state cells (layer 0 runs twice), two paged groups (rotated and unrotated attention need the same pages:
     # one group), the last run owns nothing and reads run 1's pages
-    assert [type(cell.need) for cell in runner.cells] == [FixedState, PagedKeyValue, PagedKeyValue, FixedState, PagedKeyValue]
-    assert len(cache.states) == 2 and len(cache.groups) == 1 and cache.groups[0].cells == [1, 2]
+    assert [type(cell.need) for cell in runner.cells] == [FixedState, PagedKeyValue, PagedKeyValue, FixedState, PagedKeyValue, PagedKeyValue]
+    assert len(cache.states) == 2 and len(cache.groups) == 1 and cache.groups[0].cells == [1, 2, 5]
     # the routed feed-forward and the decaying mixer look at values on the host: no step of this model is replayed from a graph
     assert not runner.model.replayable and not runner.use_graphs
     assert "layers.0.mlp.router.weight" in loaded.tensors and "layers.2.mixer.position.table" in loaded.tensors
@@ -60,6 +60,39 @@ def test_toy_architecture_steps_like_its_plain_forward(toy_folder):
     again = runner.step([StepEntry("b2", prompts["b"], range(9))], create_missing=True)
     torch.testing.assert_close(again.double(), expected["b"], atol=1e-5, rtol=1e-5)
     cache.check_invariants()
+
+
+def test_an_architecture_whose_state_runs_on_the_device_alone(toy_folder, tmp_path):
+    """The second toy architecture: a mixer with a state slot per request that nothing on the host looks at, and
+    attention whose scores carry a distance bias and a soft cap.  It is replayable (on the GPU its steps are
+    captured; tests/test_gpu_parts.py), and steps like its plain forward whatever the cut."""
+    folder = toy.write_toy_folder(tmp_path / "sum", config=toy.SUM)
+    loaded = load_model_folder(folder, "float32")
+    assert loaded.architecture.name == "ToySumForCausalLM"
+    runner = ModelRunner(loaded, TorchKernels(torch.float32), CacheConfig(block_size=4, num_blocks=40, max_sequences=3))
+    assert runner.model.replayable and len(runner.cache.states) == 2 and runner.cache.states[0].shape[0] == 4  # a spare slot
+    prompts = {name: random_tokens(n, toy.SUM.vocab_size, seed=n) for name, n in (("a", 30), ("b", 11))}
+    expected = {name: toy.plain_toy_forward(folder, tokens) for name, tokens in prompts.items()}
+    got = {name: [] for name in prompts}
+    fed = {name: 0 for name in prompts}
+    sizes = {"a": [5, 1, 1, 9, 14], "b": [2, 1, 8]}
+    for turn in range(5):
+        entries = []
+        for name, tokens in prompts.items():
+            if turn < len(sizes[name]):
+                count = sizes[name][turn]
+                entries.append(StepEntry(name, tokens[fed[name] : fed[name] + count], range(count)))
+                fed[name] += count
+        logits = runner.step(entries, create_missing=True)
+        at = 0
+        for entry in entries:
+            got[entry.request_id].append(logits[at : at + len(entry.tokens)])
+            at += len(entry.tokens)
+    for name in prompts:
+        torch.testing.assert_close(torch.cat(got[name]).double(), expected[name], atol=1e-5, rtol=1e-5)
+    runner.end_request("b")
+    again = runner.step([StepEntry("b2", prompts["b"], range(11))], create_missing=True)
+    torch.testing.assert_close(again.double(), expected["b"], atol=1e-5, rtol=1e-5)
 
 
 def test_unregistered_parts_are_refused(tmp_path):

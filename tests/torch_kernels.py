@@ -81,7 +81,7 @@ class TorchKernels:
             cell.keys[pages, :, offsets] = view[:, heads : heads + kv_heads]
             cell.values[pages, :, :, offsets] = view[:, heads + kv_heads :]  # pages are [kv, dim, offset]
 
-    def paged_attention(self, qkv, layout, batch, cell, scale, window):
+    def paged_attention(self, qkv, layout, batch, cell, scale, window, *, score_slopes=None, soft_cap=None):
         tokens = qkv.shape[0]
         heads, kv_heads, dim = layout.num_heads, layout.num_kv_heads, layout.head_dim
         queries = qkv.view(tokens, heads + 2 * kv_heads, dim)[:, :heads].float()
@@ -100,6 +100,10 @@ class TorchKernels:
                 keys = keys.repeat_interleave(heads // kv_heads, dim=1)
                 values = values.repeat_interleave(heads // kv_heads, dim=1)
                 scores = torch.einsum("hd,nhd->hn", queries[row], keys) * scale
+                if soft_cap is not None:
+                    scores = soft_cap * torch.tanh(scores / soft_cap)
+                if score_slopes is not None:
+                    scores = scores - score_slopes.float().view(-1, 1) * (position - where).float()
                 out[row] = torch.einsum("hn,nhd->hd", torch.softmax(scores, dim=-1), values)
                 row += 1
         return out.reshape(tokens, heads * dim).to(self.dtype)

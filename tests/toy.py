@@ -5,7 +5,11 @@ architectures are added by registering them, without a change to the framework's
 - beside attention layers, chosen layer by layer,
 - a feed-forward with routing (a few small experts, the best two per token) in one layer,
 - a position encoding with a tensor of its own (a learned table added to queries and keys) in another,
-- a run order that names one layer twice, and a run that reads another run's cache.
+- a position encoding that acts on the scores, not on queries and keys (a bias that grows with distance, and a
+  soft cap), in a third attention layer,
+- a run order that names one layer twice, and a run that reads another run's cache;
+- and a second architecture all of whose parts are the same kernel launches whatever the data, among them a
+  mixer with state of its own that runs on the device alone: its steps are captured into graphs and replayed.
 
 It is never a model of anyone's: it exists to exercise the interfaces."""
 
@@ -147,6 +151,73 @@ class LearnedPosition(PositionEncoding):
 
 
 @dataclass(frozen=True)
+class DistanceBiasSpec:
+    num_heads: int
+    steepest: float  # head h's slope is steepest / 2^h
+    soft_cap: float
+    kind: str = "toy_distance_bias"
+
+
+class DistanceBias(PositionEncoding):
+    """Nothing is done to queries and keys: a score loses slope[head] * distance after being
+    squashed to soft_cap * tanh(score / soft_cap)."""
+
+    def __init__(self, spec: DistanceBiasSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.slopes = kernels.to_device(torch.tensor([spec.steepest / 2.0 ** head for head in range(spec.num_heads)], dtype=torch.float32))
+
+    def encode_and_store(self, qkv, layout, batch, cell) -> None:
+        self.kernels.rotate_and_store(qkv, layout, batch, cell, None, "none")
+
+    def encode_store_attend(self, qkv, layout, batch, cell, scale, window, project=None):
+        self.encode_and_store(qkv, layout, batch, cell)
+        mixed = self.kernels.paged_attention(qkv, layout, batch, cell, scale, window, score_slopes=self.slopes,
+                                             soft_cap=self.spec.soft_cap)
+        return mixed if project is None else self.kernels.linear(mixed, project, out_dtype=torch.float32, partial=True)
+
+
+@dataclass(frozen=True)
+class RunningSumSpec:
+    hidden_size: int
+    state_size: int
+    kind: str = "toy_running_sum"
+
+
+class RunningSumMixer(Mixer):
+    """state <- state + x W_in;  out = state W_out, token after token in order: the decaying mixer without its
+    decay, so that a request's tokens can be summed by a prefix sum on the device.  Nothing is looked at on the
+    host and every shape depends on the step's shape alone: a step through it may be captured and replayed."""
+
+    @classmethod
+    def tensors(cls, spec: RunningSumSpec) -> dict[str, TensorSpec]:
+        return {
+            "in_proj.weight": TensorSpec((spec.state_size, spec.hidden_size)),
+            "out_proj.weight": TensorSpec((spec.hidden_size, spec.state_size)),
+        }
+
+    @classmethod
+    def cache_need(cls, spec: RunningSumSpec) -> FixedState:
+        return FixedState((spec.state_size,))
+
+    def __init__(self, spec: RunningSumSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.w_in = tensors["in_proj.weight"].float()
+        self.w_out = tensors["out_proj.weight"].float()
+
+    def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
+        pushed = x.float() @ self.w_in.T  # [T, state]
+        request = batch.token_sequence.long()
+        slots = batch.state_slots.long()[request]  # each token's state slot (padding tokens: the spare one)
+        running = torch.cumsum(pushed, dim=0)
+        first = batch.query_start.long()[request]  # row of the token's request's first token
+        before = torch.where((first > 0).unsqueeze(1), running[(first - 1).clamp(min=0)], torch.zeros_like(running))
+        state = cell.state[slots] + (running - before)  # the state after each token
+        if cell.writable:
+            cell.state.index_add_(0, slots, pushed)
+        return state @ self.w_out.T
+
+
+@dataclass(frozen=True)
 class ToyConfig(ArchitectureConfig):
     architecture: ClassVar[str] = "ToyStateForCausalLM"
     vocab_size: int = 0
@@ -195,41 +266,83 @@ def toy_spec(config: ToyConfig) -> ModelSpec:
         LearnedPositionSpec(config.head_dim, config.max_length), qkv_bias=False,
     )
     routed = RoutedSpec(config.hidden_size, config.expert_size, config.experts, config.experts_chosen)
+    biased = AttentionSpec(
+        config.hidden_size, config.num_heads, config.num_heads, config.head_dim, 1.0 / math.sqrt(config.head_dim),
+        DistanceBiasSpec(config.num_heads, BIAS_STEEPEST, BIAS_SOFT_CAP), qkv_bias=False,
+    )
     layers = (
         LayerDefinition("layers.0.", PreNormBlockSpec(norm, decay, norm, routed, mixer_name="mixer.")),
         LayerDefinition("layers.1.", PreNormBlockSpec(norm, attention, norm, ffn, mixer_name="mixer.")),
         LayerDefinition("layers.2.", PreNormBlockSpec(norm, unrotated, norm, ffn, mixer_name="mixer.")),
+        LayerDefinition("layers.3.", PreNormBlockSpec(norm, biased, norm, ffn, mixer_name="mixer.")),
     )
     # layer 0 runs twice (two state cells), layer 1 runs twice, its second run reading the first's pages
-    run_order = (LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(0), LayerRun(1, reads=1))
+    run_order = (LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(0), LayerRun(1, reads=1), LayerRun(3))
     return ModelSpec(
         config.vocab_size, config.hidden_size, layers, run_order, norm, tie_embeddings=True,
         embedding_name="embed.weight", final_norm_name="final_norm.",
     )
 
 
+BIAS_STEEPEST, BIAS_SOFT_CAP = 0.5, 2.0
+
+
+def sum_spec(config: ToyConfig) -> ModelSpec:
+    """The second architecture: a running-sum mixer, then attention whose scores carry a distance bias; every
+    part is the same launches whatever the data."""
+    norm = RMSNormSpec(config.hidden_size, config.eps)
+    ffn = GatedMLPSpec(config.hidden_size, config.ffn_size)
+    summing = RunningSumSpec(config.hidden_size, config.state_size)
+    biased = AttentionSpec(
+        config.hidden_size, config.num_heads, config.num_heads, config.head_dim, 1.0 / math.sqrt(config.head_dim),
+        DistanceBiasSpec(config.num_heads, BIAS_STEEPEST, BIAS_SOFT_CAP), qkv_bias=False,
+    )
+    layers = (
+        LayerDefinition("layers.0.", PreNormBlockSpec(norm, summing, norm, ffn, mixer_name="mixer.")),
+        LayerDefinition("layers.1.", PreNormBlockSpec(norm, biased, norm, ffn, mixer_name="mixer.")),
+    )
+    return ModelSpec(
+        config.vocab_size, config.hidden_size, layers, (LayerRun(0), LayerRun(1), LayerRun(0)), norm, tie_embeddings=True,
+        embedding_name="embed.weight", final_norm_name="final_norm.",
+    )
+
+
+@dataclass(frozen=True)
+class SumConfig(ToyConfig):
+    architecture: ClassVar[str] = "ToySumForCausalLM"
+
+
 TOY = ToyConfig(vocab_size=97, hidden_size=48, state_size=20, decay=0.8, num_heads=3, head_dim=16, ffn_size=64,
                 eps=1e-5, max_length=256, experts=5, experts_chosen=2, expert_size=24)
 
 
+SUM = SumConfig(**TOY.to_dict())
+
+
 def register_toy() -> None:
     MIXERS.register("toy_decay")(DecayMixer)
+    MIXERS.register("toy_running_sum")(RunningSumMixer)
     FEED_FORWARDS.register("toy_routed")(RoutedFeedForward)
     POSITIONS.register("toy_learned")(LearnedPosition)
+    POSITIONS.register("toy_distance_bias")(DistanceBias)
     register_architecture("ToyStateForCausalLM", ToyConfig, toy_spec)
+    register_architecture("ToySumForCausalLM", SumConfig, sum_spec)
 
 
 def unregister_toy() -> None:
     MIXERS.unregister("toy_decay")
+    MIXERS.unregister("toy_running_sum")
     FEED_FORWARDS.unregister("toy_routed")
     POSITIONS.unregister("toy_learned")
+    POSITIONS.unregister("toy_distance_bias")
     unregister_architecture("ToyStateForCausalLM")
+    unregister_architecture("ToySumForCausalLM")
 
 
-def write_toy_folder(folder: Path, seed: int = 3) -> Path:
+def write_toy_folder(folder: Path, seed: int = 3, config: ToyConfig = TOY) -> Path:
     from llmserve_amd.weights import write_model_folder
 
-    return write_model_folder(folder, TOY, seed, dtype=torch.float32, std=0.1, norm_std=0.1)
+    return write_model_folder(folder, config, seed, dtype=torch.float32, std=0.1, norm_std=0.1)
 
 
 # ----------------------------------------------------------------------------- the toy's own plain forward
@@ -272,11 +385,31 @@ def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
         h = h + torch.stack(out)
         return h + routed(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
 
+    def biased_attention(q, k, v, scale):
+        """softmax over keys j <= i of cap * tanh(q_i . k_j * scale / cap) - slope_head * (i - j)"""
+        scores = torch.einsum("ihd,jhd->hij", q, k) * scale
+        scores = BIAS_SOFT_CAP * torch.tanh(scores / BIAS_SOFT_CAP)
+        distance = (torch.arange(length).unsqueeze(1) - torch.arange(length).unsqueeze(0)).double()
+        slopes = torch.tensor([BIAS_STEEPEST / 2.0 ** head for head in range(heads)], dtype=torch.float64)
+        scores = scores - slopes.view(-1, 1, 1) * distance
+        scores = scores.masked_fill(distance < 0, float("-inf"))
+        return torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), v)
+
+    def sum_layer(h, prefix):
+        x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
+        state = torch.cumsum(x @ w[prefix + "mixer.in_proj.weight"].T, dim=0)
+        h = h + state @ w[prefix + "mixer.out_proj.weight"].T
+        return h + ffn(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
+
     def attention_layer(h, prefix, rotate, shared=None):
         x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
         q = (x @ w[prefix + "mixer.q_proj.weight"].T).view(length, heads, dim)
         k = (x @ w[prefix + "mixer.k_proj.weight"].T).view(length, heads, dim)
         v = (x @ w[prefix + "mixer.v_proj.weight"].T).view(length, heads, dim)
+        if rotate == "bias":
+            mixed = biased_attention(q, k, v, 1.0 / math.sqrt(dim)).reshape(length, -1)
+            h = h + mixed @ w[prefix + "mixer.o_proj.weight"].T
+            return h + ffn(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix), (k, v)
         if rotate:
             angles = plain.rope_angles(dim, 100.0, torch.arange(length))
             q, k = plain.rope_half(q, angles), plain.rope_half(k, angles)
@@ -290,9 +423,15 @@ def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
         h = h + ffn(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
         return h, (k, v)
 
+    if config["architectures"] == ["ToySumForCausalLM"]:
+        h = sum_layer(h, "layers.0.")
+        h, _ = attention_layer(h, "layers.1.", "bias")
+        h = sum_layer(h, "layers.0.")
+        return plain.rms_norm(h, w["final_norm.weight"], eps) @ w["embed.weight"].T
     h = decay_layer(h, "layers.0.")
     h, stored = attention_layer(h, "layers.1.", True)
     h, _ = attention_layer(h, "layers.2.", False)
     h = decay_layer(h, "layers.0.")
     h, _ = attention_layer(h, "layers.1.", True, shared=stored)
+    h, _ = attention_layer(h, "layers.3.", "bias")
     return plain.rms_norm(h, w["final_norm.weight"], eps) @ w["embed.weight"].T
