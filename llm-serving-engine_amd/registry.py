@@ -21,6 +21,10 @@ class Architecture:
     config_class: type[ArchitectureConfig]
     build_spec: Callable[[Any], ModelSpec]
     model_types: tuple[str, ...] = ()
+    # The files' tensors, by name, to the model's: for checkpoints whose tensors are named or cut otherwise
+    # than the parts name and cut theirs (projections stored as one fused tensor, another prefix).  Takes and
+    # returns {name: tensor}; called with the configuration before anything is checked.
+    adapt_tensors: Callable[[dict, Any], dict] | None = None
 
 
 ARCHITECTURES: dict[str, Architecture] = {}
@@ -31,8 +35,9 @@ def register_architecture(
     config_class: type[ArchitectureConfig],
     build_spec: Callable[[Any], ModelSpec],
     model_types: tuple[str, ...] = (),
+    adapt_tensors: Callable[[dict, Any], dict] | None = None,
 ) -> Architecture:
-    entry = Architecture(name, config_class, build_spec, model_types)
+    entry = Architecture(name, config_class, build_spec, model_types, adapt_tensors)
     ARCHITECTURES[name] = entry
     return entry
 

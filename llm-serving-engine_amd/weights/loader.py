@@ -144,7 +144,10 @@ def load_model_folder(
     for path in files:
         with safe_open(str(path), framework="pt", device="cpu") as source:
             for source_name in source.keys():
-                found[model_name(source_name)] = source.get_tensor(source_name)
+                found[source_name] = source.get_tensor(source_name)
+    if architecture.adapt_tensors is not None:  # the files name or cut their tensors otherwise than the parts do
+        found = architecture.adapt_tensors(found, config)
+    found = {model_name(name): tensor for name, tensor in found.items()}
 
     # A tied model's file may still carry the head: fine if it is the embedding.
     if spec.tie_embeddings and spec.head_name in found:

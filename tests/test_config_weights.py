@@ -162,3 +162,60 @@ def test_missing_files(tmp_path, model_folders):
     (tmp_path / "config.json").write_text((model_folders["A"] / "config.json").read_text())
     with pytest.raises(FileNotFoundError, match="safetensors"):
         load_model_folder(tmp_path, "float32")  # checkpoint.py:47-48
+
+
+def test_an_architecture_may_adapt_the_files_tensors_to_its_parts(tmp_path):
+    """A checkpoint that stores q, k and v as one fused tensor loads through an architecture registered with
+    `adapt_tensors`, which cuts it where the attention part expects three; the parts and the loader are
+    unchanged, and what does not fit is still reported in one error."""
+    import dataclasses
+    import json
+
+    from safetensors.torch import load_file, save_file
+
+    from llmserve_amd import WeightsError, load_model_folder, write_model_folder
+    from llmserve_amd.models.qwen2 import qwen2_spec
+    from llmserve_amd.registry import register_architecture, unregister_architecture
+    from tests.tiny import TINY_A
+
+    @dataclasses.dataclass(frozen=True)
+    class FusedConfig(type(TINY_A)):
+        architecture = "FusedQwen2ForCausalLM"
+
+    def cut(found, config):
+        adapted = {}
+        q, kv = config.num_attention_heads * config.head_dim, config.num_key_value_heads * config.head_dim
+        for name, tensor in found.items():
+            if ".qkv_proj." in name:
+                for piece, part in zip(("q_proj", "k_proj", "v_proj"), torch.split(tensor, [q, kv, kv])):
+                    adapted[name.replace("qkv_proj", piece)] = part
+            else:
+                adapted[name] = tensor
+        return adapted
+
+    register_architecture("FusedQwen2ForCausalLM", FusedConfig, qwen2_spec, adapt_tensors=cut)
+    try:
+        plain_folder = write_model_folder(tmp_path / "plain", TINY_A, seed=3)
+        tensors = load_file(str(plain_folder / "model.safetensors"))
+        fused = {}
+        for name, tensor in tensors.items():
+            if ".q_proj." in name:
+                k, v = tensors[name.replace("q_proj", "k_proj")], tensors[name.replace("q_proj", "v_proj")]
+                fused[name.replace("q_proj", "qkv_proj")] = torch.cat([tensor, k, v])
+            elif ".k_proj." not in name and ".v_proj." not in name:
+                fused[name] = tensor
+        folder = tmp_path / "fused"
+        folder.mkdir()
+        values = json.loads((plain_folder / "config.json").read_text())
+        values["architectures"] = ["FusedQwen2ForCausalLM"]
+        (folder / "config.json").write_text(json.dumps(values))
+        save_file(fused, str(folder / "model.safetensors"))
+        loaded, reference = load_model_folder(folder, "float32"), load_model_folder(plain_folder, "float32")
+        assert loaded.architecture.name == "FusedQwen2ForCausalLM" and set(loaded.tensors) == set(reference.tensors)
+        assert all(torch.equal(loaded.tensors[name], reference.tensors[name]) for name in reference.tensors)
+        del fused["model.layers.1.self_attn.qkv_proj.bias"]
+        save_file(fused, str(folder / "model.safetensors"))
+        with pytest.raises(WeightsError, match="q_proj.bias"):
+            load_model_folder(folder, "float32")
+    finally:
+        unregister_architecture("FusedQwen2ForCausalLM")
