@@ -494,11 +494,11 @@ class ModelRunner:
             graph.copied[turn].synchronize()  # the staging buffer's last copy has left it
         graph.host[turn].copy_(torch.from_numpy(packed))
         graph.static.copy_(graph.host[turn], non_blocking=True)
+        graph.batch.chunks = chunks
+        self.kernels.refresh_step(graph.batch, turn)
         event = torch.cuda.Event()
         event.record()
         graph.copied[turn] = event
-        graph.batch.chunks = chunks
-        self.kernels.refresh_step(graph.batch)
         graph.graph.replay()
         if wanted == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)

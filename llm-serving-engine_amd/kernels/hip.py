@@ -524,21 +524,29 @@ class HipKernels:
             batch.scratch[key] = (self.to_device(torch.from_numpy(work)) if len(work) else None, len(work), steps)
         return batch.scratch[key]
 
-    def refresh_step(self, batch) -> None:
+    def refresh_step(self, batch, turn: int = 0) -> None:
         """For a batch whose kernels were captured: `batch.chunks` now describes another step of the
         same padded shape; everything this library derived from the chunks on the host (the attention
-        work lists) is made anew, in place, at the addresses the captured kernels read."""
+        work lists) is made anew, in place, at the addresses the captured kernels read.  The lists go
+        through pinned staging buffers, two of each, used in turn (`turn` 0 or 1): the caller does not
+        come back to a turn before the copies it queued in it have left their buffers."""
         import numpy as np
 
-        for key, (tensor, capacity, _) in batch.scratch.items():
-            if key[0] != "attention_work" or tensor is None:
+        for key in [key for key in batch.scratch if key[0] == "attention_work"]:
+            tensor, capacity, _ = batch.scratch[key]
+            if tensor is None:
                 continue
             work, _ = self._work_items(batch.chunks, *key[1:])
             if len(work) > capacity:
                 raise KernelError("a step holds more attention work than the captured step has room for")
-            padded = np.zeros((capacity, 4), np.int32)
-            padded[: len(work)] = work
-            tensor.copy_(torch.from_numpy(padded), non_blocking=False)
+            staging = batch.scratch.get(("staging", key))
+            if staging is None:
+                staging = [torch.zeros((capacity, 4), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+                batch.scratch[("staging", key)] = staging
+            host = staging[turn].numpy()
+            host[: len(work)] = work
+            host[len(work):] = 0
+            tensor.copy_(staging[turn], non_blocking=True)
 
     def paged_attention(
         self, qkv, layout, batch, cell, scale: float, window: int | None, *,
