@@ -337,6 +337,23 @@ class HipKernels:
                 best = splits
         return best
 
+    @staticmethod
+    def _library_splits(rows: int, out_features: int, in_features: int) -> int:
+        """Into how many slices of K a library product is cut when its float32 result may stay partial sums:
+        only where K is long beside N (a down projection).  Measured on torch.mm against torch.bmm over slices:
+        K 8,960 x N 1,536: 2,048 rows 72 -> 53 us in four, 512 rows 42 -> 26, below that nothing gained;
+        K 18,944 x N 3,584: 2,048 rows 342 -> 217 in two, 1,024 rows 189 -> 114 in four, 512 rows 129 -> 68 and
+        136 rows 103 -> 43 in eight."""
+        if in_features < 2 * out_features or in_features < 8192:
+            return 1
+        if in_features < 16384:
+            wanted = 4 if rows >= 512 else 1
+        else:
+            wanted = 2 if rows >= 2048 else 4 if rows >= 1024 else 8
+        while wanted > 1 and in_features % (wanted * 32):
+            wanted //= 2
+        return wanted
+
     def _wide_applies(self, rows: int, out_features: int, in_features: int, splits: int) -> bool:
         """Whether the tiled product would run its 256 x 256 tile: enough tiles for the chip, and
         K a multiple of 32 of at least three steps."""
@@ -390,6 +407,14 @@ class HipKernels:
             streaming = "tiled"
         if streaming is None and self._library(x, weights):
             if (out_dtype or self.dtype) == torch.float32:  # float32 straight from the accumulators
+                cuts = self._library_splits(rows, weights.out_features, inner) if partial and bias is None else 1
+                if cuts > 1:
+                    # The library does not cut a long K over workgroups by itself (the down projection of the 7B
+                    # sizes at 2,048 rows: 342 us in one piece, 217 in two; at 136 rows 103 and 43 in eight).  As a
+                    # strided batch of `cuts` products over slices of K it does, and the batch is the partial sums.
+                    slices = x.view(rows, cuts, inner // cuts).transpose(0, 1)
+                    weight_slices = weights.weight.view(weights.out_features, cuts, inner // cuts).permute(1, 2, 0)
+                    return torch.bmm(slices, weight_slices, out_dtype=torch.float32)
                 out = torch.mm(x, weights.weight.t(), out_dtype=torch.float32)
                 return out if bias is None else out.add_(bias.float())
             if bias is not None and bias.dtype != x.dtype:
@@ -697,6 +722,10 @@ class HipKernels:
                 and rows <= 16
                 and project.weight.dtype == torch.bfloat16
                 and project.in_features == layout.num_heads * dim
+                # every workgroup of the product reads all splits of its K range: rows * splits / 16 times what it
+                # reads of the weights.  Small next to the fixed costs at the 1.5B sizes (4.7 MB of weights), but at
+                # the 7B sizes (25.7 MB) it made a step of 8 rows 3.82 ms against 3.67 with the merging kernel.
+                and project.weight.numel() <= (1 << 22)
             )
             left = self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), fuse=(table, pairing), unmerged=merging)
             if left is None:
