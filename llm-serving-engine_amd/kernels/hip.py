@@ -340,17 +340,17 @@ class HipKernels:
     @staticmethod
     def _library_splits(rows: int, out_features: int, in_features: int) -> int:
         """Into how many slices of K a library product is cut when its float32 result may stay partial sums:
-        only where K is long beside N (a down projection).  Measured on torch.mm against torch.bmm over slices:
-        K 8,960 x N 1,536: 2,048 rows 72 -> 53 us in four, 512 rows 42 -> 26, below that nothing gained;
-        K 18,944 x N 3,584: 2,048 rows 342 -> 217 in two, 1,024 rows 189 -> 114 in four, 512 rows 129 -> 68 and
-        136 rows 103 -> 43 in eight."""
-        if in_features < 2 * out_features or in_features < 8192:
+        only where K is long beside N (a down projection), and as many (a power of two up to eight) as bring
+        the 128 x 128 tiles of the result to about a thousand.  Measured on torch.mm against torch.bmm over
+        slices: K 8,960 x N 1,536: 2,048 rows 72 -> 53 us in four, 512 rows 42 -> 26, below that nothing
+        gained; K 18,944 x N 3,584: 2,048 rows 342 -> 217 in two, 1,024 rows 189 -> 114 in four, 512 rows
+        129 -> 68 and 136 rows 103 -> 43 in eight; K 27,648 x N 5,120: 2,048 rows 453 whole or cut, 512 rows
+        235 -> 130 in four, 136 rows 190 -> 78 in eight."""
+        if in_features < 2 * out_features or in_features < 8192 or (in_features < 16384 and rows < 512):
             return 1
-        if in_features < 16384:
-            wanted = 4 if rows >= 512 else 1
-        else:
-            wanted = 2 if rows >= 2048 else 4 if rows >= 1024 else 8
-        while wanted > 1 and in_features % (wanted * 32):
+        tiles = -(-rows // 128) * -(-out_features // 128)
+        wanted = 8
+        while wanted > 1 and (wanted * tiles > 1000 or in_features % (wanted * 32)):
             wanted //= 2
         return wanted
 

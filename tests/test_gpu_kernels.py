@@ -510,3 +510,29 @@ def test_decode_attention_whose_key_splits_the_output_projection_merges(kernels,
     other = (other if other.ndim == 2 else other.sum(0)).cpu().double()
     torch.testing.assert_close(got, other, atol=1e-2, rtol=1e-2)
     assert float((got - expected).abs().mean()) < 1.5 * float((other - expected).abs().mean()) + 1e-4
+
+
+@pytest.mark.parametrize("rows,inner,outer", [(130, 16384, 72), (600, 8960, 200), (70, 16448, 40)])
+def test_library_products_cut_over_a_long_k(kernels, rows, inner, outer):
+    """A product with a long K beside few weight rows goes to the library as a strided batch over slices of K
+    and comes back as partial sums for the reader to add; the sum is the product."""
+    from llmserve_amd.kernels import HipKernels
+
+    dtype = torch.bfloat16
+    k = kernels[dtype]
+    assert HipKernels._library_splits(rows, outer, inner) > 1
+    x, w = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner)
+    handle = k.prepare_linear([on_gpu(w, dtype)], None)
+    parts = k.linear(on_gpu(x, dtype), handle, out_dtype=torch.float32, partial=True)
+    assert parts.ndim == 3 and parts.shape[1:] == (rows, outer)
+    expected = rounded(x, dtype) @ rounded(w, dtype).T
+    torch.testing.assert_close(parts.sum(0).cpu().double(), expected, atol=1e-3, rtol=1e-3)
+    whole = k.linear(on_gpu(x, dtype), handle, out_dtype=torch.float32)
+    assert whole.ndim == 2
+    torch.testing.assert_close(whole.cpu().double(), expected, atol=1e-3, rtol=1e-3)
+    # the norm that follows adds the parts in order
+    hidden = torch.randn(rows, outer)
+    device_hidden = hidden.cuda()
+    normed = k.add_rms_norm(device_hidden, parts, on_gpu(torch.ones(outer), dtype), 1e-6)
+    torch.testing.assert_close(device_hidden.cpu().double(), hidden.double() + expected, atol=2e-3, rtol=1e-3)
+    torch.testing.assert_close(normed.cpu().double(), plain.rms_norm(hidden.double() + expected, torch.ones(outer).double(), 1e-6), **TOLERANCE[dtype])
