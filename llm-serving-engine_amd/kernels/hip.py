@@ -643,7 +643,10 @@ class HipKernels:
             # two: that pays once the keys no longer fit the chiplets' L2
             # (heads wider than 128 leave no registers for more than one tile)
             wide = 1 if layout.head_dim > 128 else 4 if batch.max_context_length >= 4096 else 2
-            launches.append((wide, *self._attention_work(batch, group_size, wide, per_tile, None)[:2]))
+            # One launch takes the requests of few tokens along (a decoded token fills part of a tile): in a
+            # step of portions beside decoded tokens two launches one after the other cost 11 us each at the
+            # 1.5B sizes, and the walk of a decoded token's keys is the same in either kernel.
+            launches = [(wide, *self._attention_work(batch, group_size, wide, 0, None)[:2])]
         for column_tiles, work, items in launches:
             if items == 0:
                 continue
