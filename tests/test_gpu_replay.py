@@ -249,3 +249,56 @@ def test_captured_mixed_steps_at_benchmark_layer_sizes(wide_models, dtype):
         torch.cuda.synchronize()
     assert any(key[:2] == (64, 8) for key in runner._step_graphs) and runner.step_counts["replayed"] >= 8, runner.step_counts
     runner.close()
+
+
+def test_a_long_context_through_the_whole_engine(wide_models):
+    """Beyond 4,096 keys the bfloat16 attention carries four column tiles a wave for portions and cuts a decoded
+    token's keys into splits (merged by the output projection, or by the merging kernel): the whole engine at
+    the 1.5B widths over 4,400 keys, a prompt in portions of changing size, a portion beside decoded tokens
+    of another long request, then single tokens; against the plain forward."""
+    from llmserve_amd import CacheConfig, ModelRunner, StepEntry
+    from llmserve_amd.kernels import HipKernels
+    from llmserve_amd.weights import load_model_folder
+
+    WIDE = WIDE_CONFIGS["1.5B"][0]
+    folder, plain_config, weights = wide_models("1.5B")
+    config = WIDE
+    sequences = [random_tokens(4400, config.vocab_size, seed=811), random_tokens(4250, config.vocab_size, seed=812)]
+    expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
+    spread = float(expected[0].std())
+    bound = dict(atol=BF16_LARGEST * spread, rtol=3e-2)
+    loaded = load_model_folder(folder, "bfloat16")
+    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(PAGE_WIDE, 2 * 280, 4), max_sequence_length=4608)
+    checked, total = 0, 0.0
+
+    def check(logits, index, positions):
+        nonlocal checked, total
+        for row, position in enumerate(positions):
+            torch.testing.assert_close(logits[row].cpu().double(), expected[index][position], **bound,
+                                       msg=lambda m: f"request {index} position {position}: {m}")
+            total += float((logits[row].cpu().double() - expected[index][position]).abs().mean())
+            checked += 1
+
+    # request 0: 2,048 + 2,000 + 300 tokens; the last portion's queries look back over more than 4,096 keys
+    fed = 0
+    for count in (2048, 2000, 300):
+        want = [0, count // 2, count - 1]
+        logits = runner.step([StepEntry("r0", sequences[0][fed : fed + count], want)], create_missing=True)
+        check(logits, 0, [fed + place for place in want])
+        fed += count
+    # request 1 catches up to 4,200 while request 0 decodes beside its portions
+    at = 0
+    for count in (2048, 2048, 104):
+        entries = [StepEntry("r0", [sequences[0][fed]], [0]), StepEntry("r1", sequences[1][at : at + count], [count - 1])]
+        logits = runner.step(entries, create_missing=True)
+        check(logits[:1], 0, [fed])
+        check(logits[1:], 1, [at + count - 1])
+        fed, at = fed + 1, at + count
+    # both decode: steps of two single tokens over 4,350 and 4,200 keys (captured, keys cut into splits)
+    for _ in range(6):
+        logits = runner.step([StepEntry("r0", [sequences[0][fed]], [0]), StepEntry("r1", [sequences[1][at]], [0])])
+        check(logits[:1], 0, [fed])
+        check(logits[1:], 1, [at])
+        fed, at = fed + 1, at + 1
+    assert checked == 9 + 6 + 12 and total / checked < BF16_MEAN * spread
+    runner.close()
