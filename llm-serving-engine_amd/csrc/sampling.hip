@@ -125,15 +125,24 @@ __global__ void argmax_pick_kernel(const float* __restrict__ piece_values, const
 
 #define ARGMAX_PIECES 64
 
+// Into how many pieces a row is cut: 64 for a few rows (so that they fill the chip), fewer for many (a piece
+// of 2,400 logits leaves a thread of its block two or three of them and the block's reduction dominates:
+// 64 rows of 151,936 took 33 us in 64 pieces each).  About a thousand blocks in all, at least 8 pieces a row.
+static int argmax_pieces(int rows) {
+  int pieces = ARGMAX_PIECES;
+  while (pieces > 8 && rows * pieces > 1024) pieces /= 2;
+  return pieces;
+}
+
 // scratch: at least rows * 64 floats and rows * 64 ints
 extern "C" int llmserve_argmax(const float* logits, float* piece_values, int* piece_indices, int* out, int rows,
                                int vocab, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) return ERR_BAD_ARGUMENT;
-  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(rows, ARGMAX_PIECES), dim3(SAMPLE_THREADS), 0, stream, logits,
-                     piece_values, piece_indices, vocab, ARGMAX_PIECES);
-  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(WAVE), 0, stream, piece_values, piece_indices, out,
-                     ARGMAX_PIECES);
+  const int pieces = argmax_pieces(rows);
+  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(rows, pieces), dim3(SAMPLE_THREADS), 0, stream, logits,
+                     piece_values, piece_indices, vocab, pieces);
+  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(WAVE), 0, stream, piece_values, piece_indices, out, pieces);
   return LAUNCH_STATUS();
 }
 
@@ -172,10 +181,10 @@ extern "C" int llmserve_argmax_static(const float* logits, int* out, int rows, i
   // Nothing has to start at zero: the first kernel writes every slot that the second one reads.
   float* piece_values = (float*)base;
   int* piece_indices = (int*)((unsigned char*)base + ARGMAX_STATIC_SLOTS * sizeof(float));
-  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(rows, ARGMAX_PIECES), dim3(SAMPLE_THREADS), 0, stream, logits,
-                     piece_values, piece_indices, vocab, ARGMAX_PIECES);
-  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(WAVE), 0, stream, piece_values, piece_indices, out,
-                     ARGMAX_PIECES);
+  const int pieces = argmax_pieces(rows);
+  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(rows, pieces), dim3(SAMPLE_THREADS), 0, stream, logits,
+                     piece_values, piece_indices, vocab, pieces);
+  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(WAVE), 0, stream, piece_values, piece_indices, out, pieces);
   return LAUNCH_STATUS();
 }
 

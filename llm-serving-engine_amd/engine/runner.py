@@ -211,6 +211,7 @@ class ModelRunner:
         self.max_step_graphs = 48
         self._step_graphs: dict[tuple, _DecodeGraph] = {}
         self._shape_seen: dict[tuple, int] = {}
+        self._captures_off = False  # set when a capture ran out of memory: graphs that exist are still replayed
         self.step_counts = {"replayed": 0, "captured": 0, "launched": 0}  # how steps reached the device
         self.packing_ms = 0.0  # host time spent on the steps' index arrays
         # What `prepare_decode` has done for the step to come: each request's reservation of one
@@ -476,7 +477,7 @@ class ModelRunner:
         if graph is None:
             seen = self._shape_seen.get(key, 0) + 1
             self._shape_seen[key] = seen
-            if seen < 2:
+            if seen < 2 or self._captures_off:
                 self.step_counts["launched"] += 1
                 return None
         self.step_counts["replayed" if graph is not None else "captured"] += 1
@@ -486,7 +487,16 @@ class ModelRunner:
         chunks = [SequenceChunk(r.request_id, r.slot, r.start, r.count) for r in reservations]
         self.packing_ms += 1000.0 * (time.perf_counter() - started)
         if graph is None:
-            graph = self._capture_step(key, packed, sizes, widths, facts, chunks)
+            try:
+                graph = self._capture_step(key, packed, sizes, widths, facts, chunks)
+            except torch.OutOfMemoryError:
+                # no room for another graph's buffers beside the cache: this shape, and new ones from now on,
+                # are launched kernel by kernel (the step itself has not run yet: nothing is lost)
+                self._captures_off = True
+                self.step_counts["captured"] -= 1
+                self.step_counts["launched"] += 1
+                torch.cuda.empty_cache()
+                return None
         self._step_graphs[key] = graph  # the one used last stands last
         turn = graph.turn
         graph.turn = 1 - turn

@@ -1,6 +1,7 @@
 from .base import (
     BLOCKS,
     FEED_FORWARDS,
+    LOGIT_PARTS,
     MIXERS,
     NORMS,
     POSITIONS,
@@ -8,6 +9,7 @@ from .base import (
     PagedKeyValue,
     Part,
     Registry,
+    STREAM_PARTS,
     TensorSpec,
 )
 from .norm import RMSNorm, RMSNormSpec
@@ -15,6 +17,6 @@ from .position import HeadLayout, NoPositionSpec, PositionEncoding, Rotary, Rota
 from .attention import Attention, AttentionSpec, Mixer
 from .feed_forward import FeedForward, GatedMLP, GatedMLPSpec
 from .block import Block, PreNormBlock, PreNormBlockSpec
-from .model import DecoderModel, LayerDefinition, LayerRun, ModelSpec
+from .model import DecoderModel, LayerDefinition, LayerRun, ModelSpec, NamedPart
 
 __all__ = [name for name in dir() if not name.startswith("_")]

@@ -121,6 +121,12 @@ POSITIONS = Registry("position encoding")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 BLOCKS = Registry("block")
+# What acts on the residual stream between the embedding and the first layer (`forward(hidden, batch)`, in
+# place: a table of absolute positions, a scale), and on the logits after the head (`forward(logits, batch)
+# -> logits`: a bias, a soft cap).  Qwen2 has neither; a model lists them in `ModelSpec.input_parts` and
+# `ModelSpec.output_parts`.
+STREAM_PARTS = Registry("part on the embedded stream")
+LOGIT_PARTS = Registry("part on the logits")
 
 
 def under(tensors: dict[str, Any], prefix: str) -> dict[str, Any]:

@@ -8,7 +8,7 @@ from typing import Any
 
 import torch
 
-from .base import BLOCKS, NORMS, CacheNeed, TensorSpec, prefixed, under
+from .base import BLOCKS, LOGIT_PARTS, NORMS, STREAM_PARTS, CacheNeed, TensorSpec, prefixed, under
 
 
 @dataclass(frozen=True)
@@ -29,6 +29,14 @@ class LayerRun:
 
 
 @dataclass(frozen=True)
+class NamedPart:
+    """A part outside the layers: the prefix of its tensors and its spec."""
+
+    prefix: str
+    spec: Any
+
+
+@dataclass(frozen=True)
 class ModelSpec:
     vocab_size: int
     hidden_size: int
@@ -39,6 +47,10 @@ class ModelSpec:
     embedding_name: str = "model.embed_tokens.weight"
     final_norm_name: str = "model.norm."
     head_name: str = "lm_head.weight"
+    # parts that act on the embedded rows before the first layer (kinds of STREAM_PARTS), and on the
+    # logits after the head (kinds of LOGIT_PARTS), in order; Qwen2 has none
+    input_parts: tuple[NamedPart, ...] = ()
+    output_parts: tuple[NamedPart, ...] = ()
 
     def __post_init__(self) -> None:
         for index, run in enumerate(self.run_order):
@@ -62,6 +74,10 @@ class ModelSpec:
         for layer in self.layers:
             found.update(prefixed(BLOCKS.tensors(layer.block), layer.prefix))
         found.update(prefixed(NORMS.tensors(self.final_norm), self.final_norm_name))
+        for part in self.input_parts:
+            found.update(prefixed(STREAM_PARTS.tensors(part.spec), part.prefix))
+        for part in self.output_parts:
+            found.update(prefixed(LOGIT_PARTS.tensors(part.spec), part.prefix))
         if not self.tie_embeddings:
             found[self.head_name] = TensorSpec((self.vocab_size, self.hidden_size))
         return found
@@ -82,10 +98,15 @@ class DecoderModel:
         self.final_norm = NORMS.build(spec.final_norm, under(tensors, spec.final_norm_name), kernels)
         head = self.embedding if spec.tie_embeddings else tensors[spec.head_name]
         self.head = kernels.prepare_linear([head], None)
-        self.replayable = all(layer.replayable for layer in self.layers) and self.final_norm.replayable
+        self.input_parts = [STREAM_PARTS.build(part.spec, under(tensors, part.prefix), kernels) for part in spec.input_parts]
+        self.output_parts = [LOGIT_PARTS.build(part.spec, under(tensors, part.prefix), kernels) for part in spec.output_parts]
+        every = [*self.layers, self.final_norm, *self.input_parts, *self.output_parts]
+        self.replayable = all(part.replayable for part in every)
 
     def _run_layers(self, batch, cells: list):
         hidden = self.kernels.embedding(self.embedding, batch.token_ids)
+        for part in self.input_parts:
+            part.forward(hidden, batch)
         delta = None
         for run, cell in zip(self.spec.run_order, cells):
             delta = self.layers[run.layer].forward(hidden, delta, batch, cell)
@@ -104,4 +125,7 @@ class DecoderModel:
         else:
             rows = self.kernels.gather_rows(hidden, delta, batch.logit_rows)
             normed = self.final_norm.forward(rows, None)
-        return self.kernels.linear(normed, self.head, out_dtype=torch.float32)
+        logits = self.kernels.linear(normed, self.head, out_dtype=torch.float32)
+        for part in self.output_parts:
+            logits = part.forward(logits, batch)
+        return logits

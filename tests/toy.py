@@ -9,7 +9,9 @@ architectures are added by registering them, without a change to the framework's
   soft cap), in a third attention layer,
 - a run order that names one layer twice, and a run that reads another run's cache;
 - and a second architecture all of whose parts are the same kernel launches whatever the data, among them a
-  mixer with state of its own that runs on the device alone: its steps are captured into graphs and replayed.
+  mixer with state of its own that runs on the device alone: its steps are captured into graphs and replayed;
+  it also has a part between the embedding and the first layer (a learned table of absolute positions, and a
+  scale) and one after the head (a bias and a soft cap on the logits).
 
 It is never a model of anyone's: it exists to exercise the interfaces."""
 
@@ -25,8 +27,9 @@ import torch
 
 from llmserve_amd.config.model import ArchitectureConfig, KeyReader
 from llmserve_amd.parts import (
-    FEED_FORWARDS, MIXERS, POSITIONS, AttentionSpec, FeedForward, FixedState, GatedMLPSpec, LayerDefinition, LayerRun,
-    Mixer, ModelSpec, NoPositionSpec, PositionEncoding, PreNormBlockSpec, RMSNormSpec, RotarySpec, TensorSpec,
+    FEED_FORWARDS, LOGIT_PARTS, MIXERS, POSITIONS, STREAM_PARTS, AttentionSpec, FeedForward, FixedState, GatedMLPSpec,
+    LayerDefinition, LayerRun, Mixer, ModelSpec, NamedPart, NoPositionSpec, Part, PositionEncoding, PreNormBlockSpec,
+    RMSNormSpec, RotarySpec, TensorSpec,
 )
 from llmserve_amd.registry import register_architecture, unregister_architecture
 
@@ -218,6 +221,51 @@ class RunningSumMixer(Mixer):
 
 
 @dataclass(frozen=True)
+class AbsolutePositionsSpec:
+    hidden_size: int
+    max_length: int
+    scale: float
+    kind: str = "toy_absolute_positions"
+
+
+class AbsolutePositions(Part):
+    """h <- h * scale + table[position], on the embedded rows, before the first layer."""
+
+    @classmethod
+    def tensors(cls, spec: AbsolutePositionsSpec) -> dict[str, TensorSpec]:
+        return {"table": TensorSpec((spec.max_length, spec.hidden_size))}
+
+    def __init__(self, spec: AbsolutePositionsSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.table = tensors["table"].float()
+
+    def forward(self, hidden: torch.Tensor, batch) -> None:
+        hidden.mul_(self.spec.scale).add_(self.table[batch.positions.long()])
+
+
+@dataclass(frozen=True)
+class CappedLogitsSpec:
+    vocab_size: int
+    cap: float
+    kind: str = "toy_capped_logits"
+
+
+class CappedLogits(Part):
+    """logits <- cap * tanh((logits + bias) / cap), after the head."""
+
+    @classmethod
+    def tensors(cls, spec: CappedLogitsSpec) -> dict[str, TensorSpec]:
+        return {"bias": TensorSpec((spec.vocab_size,), role="bias")}
+
+    def __init__(self, spec: CappedLogitsSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.bias = tensors["bias"].float()
+
+    def forward(self, logits: torch.Tensor, batch) -> torch.Tensor:
+        return self.spec.cap * torch.tanh((logits + self.bias) / self.spec.cap)
+
+
+@dataclass(frozen=True)
 class ToyConfig(ArchitectureConfig):
     architecture: ClassVar[str] = "ToyStateForCausalLM"
     vocab_size: int = 0
@@ -285,6 +333,7 @@ def toy_spec(config: ToyConfig) -> ModelSpec:
 
 
 BIAS_STEEPEST, BIAS_SOFT_CAP = 0.5, 2.0
+EMBEDDING_SCALE, LOGIT_CAP = 1.5, 3.0
 
 
 def sum_spec(config: ToyConfig) -> ModelSpec:
@@ -304,6 +353,8 @@ def sum_spec(config: ToyConfig) -> ModelSpec:
     return ModelSpec(
         config.vocab_size, config.hidden_size, layers, (LayerRun(0), LayerRun(1), LayerRun(0)), norm, tie_embeddings=True,
         embedding_name="embed.weight", final_norm_name="final_norm.",
+        input_parts=(NamedPart("positions.", AbsolutePositionsSpec(config.hidden_size, config.max_length, EMBEDDING_SCALE)),),
+        output_parts=(NamedPart("logits.", CappedLogitsSpec(config.vocab_size, LOGIT_CAP)),),
     )
 
 
@@ -325,6 +376,8 @@ def register_toy() -> None:
     FEED_FORWARDS.register("toy_routed")(RoutedFeedForward)
     POSITIONS.register("toy_learned")(LearnedPosition)
     POSITIONS.register("toy_distance_bias")(DistanceBias)
+    STREAM_PARTS.register("toy_absolute_positions")(AbsolutePositions)
+    LOGIT_PARTS.register("toy_capped_logits")(CappedLogits)
     register_architecture("ToyStateForCausalLM", ToyConfig, toy_spec)
     register_architecture("ToySumForCausalLM", SumConfig, sum_spec)
 
@@ -335,6 +388,8 @@ def unregister_toy() -> None:
     FEED_FORWARDS.unregister("toy_routed")
     POSITIONS.unregister("toy_learned")
     POSITIONS.unregister("toy_distance_bias")
+    STREAM_PARTS.unregister("toy_absolute_positions")
+    LOGIT_PARTS.unregister("toy_capped_logits")
     unregister_architecture("ToyStateForCausalLM")
     unregister_architecture("ToySumForCausalLM")
 
@@ -424,10 +479,12 @@ def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
         return h, (k, v)
 
     if config["architectures"] == ["ToySumForCausalLM"]:
+        h = h * EMBEDDING_SCALE + w["positions.table"][:length]
         h = sum_layer(h, "layers.0.")
         h, _ = attention_layer(h, "layers.1.", "bias")
         h = sum_layer(h, "layers.0.")
-        return plain.rms_norm(h, w["final_norm.weight"], eps) @ w["embed.weight"].T
+        logits = plain.rms_norm(h, w["final_norm.weight"], eps) @ w["embed.weight"].T
+        return LOGIT_CAP * torch.tanh((logits + w["logits.bias"]) / LOGIT_CAP)
     h = decay_layer(h, "layers.0.")
     h, stored = attention_layer(h, "layers.1.", True)
     h, _ = attention_layer(h, "layers.2.", False)
