@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from ..config.serving import CacheConfig
-from .cell import CacheCell
+from .cell import CacheCell, key_piece_width
 from ..parts.base import FixedState, PagedKeyValue
 from ..parts.model import ModelSpec
 from .pool import CacheFullError, PagePool
@@ -147,7 +147,11 @@ class CacheManager:
                         need=group.need,
                         writable=writable,
                         group=entry[1],
-                        keys=group.storage[entry[2], 0],
+                        keys=group.storage[entry[2], 0].view(
+                            self.config.num_blocks, group.need.num_kv_heads,
+                            group.need.head_dim // key_piece_width(group.need.head_dim), self.page_size,
+                            key_piece_width(group.need.head_dim),
+                        ),
                         values=group.storage[entry[2], 1].view(
                             self.config.num_blocks, group.need.num_kv_heads, group.need.head_dim, self.page_size
                         ),
@@ -307,10 +311,13 @@ class CacheManager:
         for block in range(record.released[group_index], math.ceil(record.length / page_size)):
             held = min(page_size, record.length - block * page_size)
             page = int(table[block])
-            keys = group.storage[cell, 0, page, :, :held]  # [kv_heads, n, head_dim]
+            heads, dim = group.need.num_kv_heads, group.need.head_dim
+            # key pages are kept in pieces, [kv_heads, dim / w, offset, w] (`CacheCell`)
+            width = key_piece_width(dim)
+            keys = group.storage[cell, 0, page].view(heads, dim // width, page_size, width)[:, :, :held]
             # value pages are kept transposed, [kv_heads, head_dim, offset]
-            values = group.storage[cell, 1, page].view(group.need.num_kv_heads, group.need.head_dim, page_size)[:, :, :held]
-            yield block * page_size, keys.transpose(0, 1), values.permute(2, 0, 1)
+            values = group.storage[cell, 1, page].view(heads, dim, page_size)[:, :, :held]
+            yield block * page_size, keys.permute(2, 0, 1, 3).reshape(held, heads, dim), values.permute(2, 0, 1)
 
     def gather(self, request_id: str, run: int) -> tuple[int, torch.Tensor, torch.Tensor]:
         """(first cached position, keys, values) of the request in run `run` as two contiguous tensors

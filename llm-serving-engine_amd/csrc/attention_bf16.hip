@@ -9,7 +9,10 @@
 //   O^T[d][column] += V^T[d][key] * P^T[key][column]      A = rows of the transposed V page
 // so each lane owns one column: its running maximum, its sum and four rows of every 16-row
 // tile of O^T.  Value pages are stored transposed ([page, kv_head, dim, offset]) so that the
-// keys, the contraction index of the second product, are contiguous for the A operand; the
+// keys, the contraction index of the second product, are contiguous for the A operand; key pages
+// are stored in pieces of eight elements, a piece of all the page's keys side by side ([page,
+// kv_head, dim / 8, offset, 8]), so that neighbouring lanes, which hold the same piece of
+// neighbouring keys, read neighbouring bytes (common.h: key_element); the
 // keys of a step are dealt to the rows of the first product in groups of four so that the
 // layout S comes out in is already the layout P goes in with, without a shuffle.
 // The four waves of a workgroup take the steps of the tile's key range in turn and merge
@@ -49,12 +52,15 @@ struct QkOperand {                            // one lane's share of a row for o
 #endif
 };
 
-__device__ __forceinline__ QkOperand load_qk(const bf16_t* row, int step, int q) {
+// `key`: where the key's first piece lies in its page; the pieces are `piece_stride` elements apart
+// (common.h: key_element; KEY_PIECE for a row that is in one piece, as a query's is).  A lane's share of MFMA step `step` is piece 4 step + q, or, with 16-wide
+// steps, half q % 2 of piece 2 step + q / 2.
+__device__ __forceinline__ QkOperand load_qk(const bf16_t* key, unsigned piece_stride, int step, int q) {
   QkOperand r;
 #if HEAD_DIM % 32 == 0
-  r.v = *(const bf16x8*)(row + step * 32 + q * 8);
+  r.v = *(const bf16x8*)(key + (unsigned)(step * 4 + q) * piece_stride);
 #else
-  r.v = *(const s16x4*)(row + step * 16 + q * 4);
+  r.v = *(const s16x4*)(key + (unsigned)(step * 2 + (q >> 1)) * piece_stride + (q & 1) * 4);
 #endif
   return r;
 }
@@ -297,7 +303,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
     column_first[t] = window > 0 ? column_position[t] - window + 1 : 0;
     const bf16_t* q_row = qkv + (size_t)(row0 + safe) * row_width + (size_t)head * D;
 #pragma unroll
-    for (int s = 0; s < QK_STEPS; ++s) query[t][s] = load_qk(q_row, s, q);
+    for (int s = 0; s < QK_STEPS; ++s) query[t][s] = load_qk(q_row, KEY_PIECE, s, q);  // a query's row is in one piece
 #if HEAD_DIM % 32 == 0
     if (FUSED && fused.pairing != 0) {  // the queries come unrotated: rotate them here, in float32
       const float2* angles = fused.table + (size_t)(row0 + safe) * (D / 2);
@@ -358,7 +364,10 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   const bool stores_token = FUSED && step_last >= step_begin && step_last < step_end &&
                             wave == (step_last - step_begin) % WAVES;
   if (stores_token && new_slot >= 0) {
-    bf16_t* k_page = keys + (size_t)(new_slot / page_size) * page_stride + head_offset + (size_t)(new_slot % page_size) * D;
+    // element e of the key: piece e / 8 of the slot's offset, pieces page_size * 8 elements apart
+    bf16_t* k_page = keys + (size_t)(new_slot / page_size) * page_stride + head_offset + (size_t)(new_slot % page_size) * KEY_PIECE;
+    const unsigned piece_stride = (unsigned)page_size * KEY_PIECE;
+    auto k_at = [&](int e) -> bf16_t& { return k_page[(unsigned)(e / KEY_PIECE) * piece_stride + e % KEY_PIECE]; };
     bf16_t* v_page = values + (size_t)(new_slot / page_size) * page_stride + head_offset + new_slot % page_size;
 #pragma unroll
     for (int i = 0; i < PAIR_PIECES; ++i) {
@@ -366,8 +375,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
       if (j < D / 2) {
         float a = (float)new_a[i], b = (float)new_b[i];
         if (fused.pairing != 0) rotate_pair(a, b, new_angle[i]);
-        k_page[fused.pairing == 2 ? j : 2 * j] = (bf16_t)a;
-        k_page[fused.pairing == 2 ? j + D / 2 : 2 * j + 1] = (bf16_t)b;
+        k_at(fused.pairing == 2 ? j : 2 * j) = (bf16_t)a;
+        k_at(fused.pairing == 2 ? j + D / 2 : 2 * j + 1) = (bf16_t)b;
       }
     }
 #pragma unroll
@@ -414,12 +423,13 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   auto fetch_keys = [&](int step, const StepPages& P, StepLoads& L) {
     const StepKeys at = keys_of(step);
     const int offset = at.k - page_index(at.k) * page_size, offset_hi = at.k_hi - page_index(at.k_hi) * page_size;
-    const bf16_t* row_lo = keys + (size_t)(unsigned)P.k * page_stride + (head_offset + (unsigned)offset * D);
-    const bf16_t* row_hi = keys + (size_t)(unsigned)P.k_hi * page_stride + (head_offset + (unsigned)offset_hi * D);
+    const bf16_t* key_lo = keys + (size_t)(unsigned)P.k * page_stride + (head_offset + (unsigned)offset * KEY_PIECE);
+    const bf16_t* key_hi = keys + (size_t)(unsigned)P.k_hi * page_stride + (head_offset + (unsigned)offset_hi * KEY_PIECE);
+    const unsigned piece_stride = (unsigned)page_size * KEY_PIECE;
 #pragma unroll
     for (int s = 0; s < QK_STEPS; ++s) {
-      L.k_lo[s] = load_qk(row_lo, s, q);
-      L.k_hi[s] = load_qk(row_hi, s, q);
+      L.k_lo[s] = load_qk(key_lo, piece_stride, s, q);
+      L.k_hi[s] = load_qk(key_hi, piece_stride, s, q);
     }
   };
   auto fetch_values = [&](int step, const StepPages& P, StepLoads& L) {
@@ -623,7 +633,7 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
     columns.first[t] = window > 0 ? columns.position[t] - window + 1 : 0;
     const bf16_t* q_row = qkv + (size_t)(min(row0, row_first + tokens_all - 1) + safe) * row_width + (size_t)head * D;
 #pragma unroll
-    for (int s = 0; s < QK_STEPS; ++s) columns.query[t][s] = load_qk(q_row, s, q);
+    for (int s = 0; s < QK_STEPS; ++s) columns.query[t][s] = load_qk(q_row, KEY_PIECE, s, q);  // a query's row is in one piece
     columns.running_max[t] = -INFINITY;
     columns.running_sum[t] = 0.f;
 #pragma unroll
@@ -646,12 +656,12 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
     for (int i = 0; i < 4; ++i) pages[i] = table[page_index(min(max(key0 + 8 * i, first_key_all), last_key_all))];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      // K: lane l takes piece l % 16 of row 4 (2 wave + j) + l / 16: 256 bytes of a row from 16 lanes
-      const int row = 4 * (2 * wave + j) + (lane >> 4);
+      // K: lane l takes piece 8 j + l / 8 of row 8 wave + l % 8: eight lanes read 128 bytes in a row
+      const int row = 8 * wave + (lane & 7);
       const int key = min(max(key0 + row, first_key_all), last_key_all);
       const int offset = key - page_index(key) * page_size;
       pieces.k[j] = *(const bf16x8*)(keys + (size_t)(unsigned)pages[wave] * page_stride +
-                                     (head_offset + (unsigned)offset * D) + (lane & 15) * 8);
+                                     (head_offset + ((unsigned)(8 * j + (lane >> 3)) * page_size + offset) * KEY_PIECE));
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -668,8 +678,8 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   auto write_step = [&](const StagedPieces& pieces, bf16_t* stage) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int row = 4 * (2 * wave + j) + (lane >> 4);
-      const int slot = (lane & 15) ^ ((row & 3) | ((row >> 3) << 2));
+      const int row = 8 * wave + (lane & 7);
+      const int slot = (8 * j + (lane >> 3)) ^ ((row & 3) | ((row >> 3) << 2));
       *(bf16x8*)(stage + (size_t)row * D + slot * 8) = pieces.k[j];
       const int d = 16 * (2 * wave + j) + (lane >> 2);
       *(bf16x8*)(stage + KEYS * D + (size_t)d * KEYS + ((lane & 3) ^ ((d >> 1) & 3)) * 8) = pieces.v[j];
@@ -884,10 +894,6 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
                                     scale, window, splits, fused, stream);
   } else if (column_tiles == 2) {
     status = launch_tiles<2, false, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
-                                    table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
-                                    scale, window, splits, fused, stream);
-  } else if (column_tiles == 4) {
-    status = launch_tiles<4, false, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
                                     table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,
                                     scale, window, splits, fused, stream);
   } else {

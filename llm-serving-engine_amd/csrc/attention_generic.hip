@@ -33,6 +33,7 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
 
   const int first = window > 0 ? max(0, position - window + 1) : 0;
   const float slope = slopes ? slopes[head] : 0.f;
+  const int width = key_piece_width(dim);
   const int per_thread = (dim + KEYS_PER_TILE - 1) / KEYS_PER_TILE;  // output dims per thread, <= 4
   float acc[MAX_DIM / KEYS_PER_TILE] = {};
   float running_max = -INFINITY, running_sum = 0.f;
@@ -42,9 +43,13 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
     float score = -INFINITY;
     if (key <= position) {
       const int page = table[key / page_size];
-      const T* k = keys + (((size_t)page * kv_heads + kv_head) * page_size + key % page_size) * dim;
+      // the key's pieces lie page_size * width apart (common.h: key_element)
+      const T* k = keys + ((size_t)page * kv_heads + kv_head) * page_size * dim + (size_t)(key % page_size) * width;
       float dot = 0.f;
-      for (int d = 0; d < dim; ++d) dot = fmaf(query[d], to_float(k[d]), dot);
+      for (int piece = 0; piece < dim / width; ++piece) {
+        const T* part = k + (size_t)piece * page_size * width;
+        for (int e = 0; e < width; ++e) dot = fmaf(query[piece * width + e], to_float(part[e]), dot);
+      }
       score = dot;
       if (soft_cap > 0.f) score = soft_cap * tanhf(score / soft_cap);
       score -= slope * (float)(position - key);

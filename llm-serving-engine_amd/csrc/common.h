@@ -66,3 +66,18 @@ __device__ __forceinline__ float block_max(float v, float* shared /* >= 17 float
   __syncthreads();
   return shared[16];
 }
+
+// Where a key lies in its page.  The keys of one (page, kv head) are kept in pieces of KEY_PIECE
+// elements, the same piece of all the page's keys side by side: [dim / KEY_PIECE][page_size][KEY_PIECE].
+// The matrix cores take a key as a row of their A operand, a lane holding eight elements of one key and
+// its neighbours the same eight of the next keys: laid out like this, four neighbouring lanes read 64
+// bytes in a row and the address unit serves them in one go, where whole rows (256 bytes apart at head
+// size 128) took it four (prefill attention over 2,048 keys: 44 -> 31 us).  A head size that is no
+// multiple of KEY_PIECE has one piece, the whole row.
+#define KEY_PIECE 8
+__device__ __host__ __forceinline__ int key_piece_width(int dim) { return dim % KEY_PIECE == 0 ? KEY_PIECE : dim; }
+// element index of dimension d of the key at `offset`, counted from the start of its (page, kv head)
+__device__ __forceinline__ size_t key_element(int d, int offset, int page_size, int dim) {
+  const int width = key_piece_width(dim);
+  return ((size_t)(d / width) * page_size + offset) * width + d % width;
+}

@@ -223,8 +223,9 @@ extern "C" int llmserve_rotary_table(const int* positions, const float* inverse,
 // becomes (a cos - b sin, b cos + a sin), all in float32.
 // pairing 0: none, 1: adjacent pairs (2j, 2j+1), 2: half pairs (j, j + dim/2).
 // k (after rotation) and v are then written to the pages: slot = page * page_size + offset,
-// key pages laid out [page, kv_head, offset, dim], value pages transposed [page, kv_head,
-// dim, offset] (reference kv_cache.py:249-266 writes both as [page, offset, kv_head, dim]).
+// key pages laid out [page, kv_head, dim / 8, offset, 8] (common.h: key_element), value pages
+// transposed [page, kv_head, dim, offset] (reference kv_cache.py:249-266 writes both as
+// [page, offset, kv_head, dim]).
 // slots may be null (nothing is stored); a negative slot skips the token.
 template <typename T>
 __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const float2* __restrict__ table, int pairing, int heads,
@@ -257,7 +258,7 @@ __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const float2* __res
   for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
     const int head = i / dim, d = i % dim;
     const size_t block = ((size_t)page * kv_heads + head) * page_size * dim;
-    keys[block + (size_t)offset * dim + d] = k_row[i];
+    keys[block + key_element(d, offset, page_size, dim)] = k_row[i];
     values[block + (size_t)d * page_size + offset] = v_row[i];
   }
 }
@@ -310,9 +311,11 @@ __global__ __launch_bounds__(256) void rotate_and_store_vector_kernel(
       *(bf16x8*)(h + ib) = b;
     }
     if (head >= heads && slot >= 0) {
-      bf16_t* k_row = keys + (((size_t)(slot / page_size) * kv_heads + (head - heads)) * page_size + slot % page_size) * dim;
-      *(bf16x8*)(k_row + ia) = a;
-      *(bf16x8*)(k_row + ib) = b;
+      // pieces ia / 8 and ib / 8 of the key at this slot (dim is a multiple of 16 here)
+      bf16_t* k_block = keys + ((size_t)(slot / page_size) * kv_heads + (head - heads)) * page_size * dim;
+      const int offset = slot % page_size;
+      *(bf16x8*)(k_block + ((size_t)(ia / KEY_PIECE) * page_size + offset) * KEY_PIECE) = a;
+      *(bf16x8*)(k_block + ((size_t)(ib / KEY_PIECE) * page_size + offset) * KEY_PIECE) = b;
     }
   } else if (slot >= 0) {
     const int at = piece - rotated, head = at / (dim / 8), d0 = (at % (dim / 8)) * 8;

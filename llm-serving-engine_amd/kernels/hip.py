@@ -224,7 +224,7 @@ class HipKernels:
             raise KernelError("rotate_and_store: qkv does not have the layout's width")
         store = cell is not None and cell.writable
         group = batch.groups[cell.group] if store else None
-        if store and (cell.keys.dtype != qkv.dtype or cell.keys.shape[1:] != (layout.num_kv_heads, group.page_size, layout.head_dim)):
+        if store and (cell.keys.dtype != qkv.dtype or cell.values.shape[1:] != (layout.num_kv_heads, layout.head_dim, group.page_size)):
             raise KernelError("rotate_and_store: the cell's pages do not fit the layout")
         table = self.rotary_table(batch, inverse_frequencies) if pairing != "none" else None
         status = self._elementwise.llmserve_rotate_and_store(
@@ -622,14 +622,15 @@ class HipKernels:
         if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never" and not padded:
             # Prompt portions at this head size may go to the kernel whose waves share each step's K and V
             # through LDS (a quarter of the cache traffic).  Its workgroups walk all their keys step after
-            # step, so it needs several workgroups a CU to be ahead: long prompts, or many of them.
+            # step, 1.2 us a step whatever the arithmetic, so it is ahead where the walks are many and short:
+            # measured at 5 to 7 query heads a kv head over thirty shapes, it wins (by up to a third) where the
+            # steps of all walks together are more than 8 x longest + 110 times the longest walk (sixteen
+            # prompts of 512 tokens, 64 of 128, eight of 1,024 at the 7B sizes), and loses elsewhere (one
+            # prompt of any length, a portion behind a long context, four prompts of 4,096).
             work, items, steps = self._attention_work(batch, group_size, 8, per_tile, None)
-            workgroups = items * kv_heads * head_tiles
-            # measured at 6 and 7 query heads a kv head: it takes 1.2 us for every step of its longest walk
-            # and 0.4 ns for every step of all walks, the other kernel 4 to 6 ns for every step of all walks
             longest = batch.max_context_length / 32
             shared = self.shared_portions == "always" or (
-                workgroups >= 256 and steps * kv_heads * head_tiles > 200 * longest
+                steps * kv_heads * head_tiles >= (8 * longest + 110) * longest
             )
         if shared:
             status = library.llmserve_attention_portions(
@@ -639,10 +640,9 @@ class HipKernels:
             )
             _check(status, "paged_attention")
         elif batch.max_query_length > per_tile:
-            # four column tiles a wave halve the cache traffic of two, at one wave a SIMD instead of
-            # two: that pays once the keys no longer fit the chiplets' L2
-            # (heads wider than 128 leave no registers for more than one tile)
-            wide = 1 if layout.head_dim > 128 else 4 if batch.max_context_length >= 4096 else 2
+            # two column tiles a wave (heads wider than 128 leave no registers for more than one); four, at
+            # one wave a SIMD, were ahead beyond 4,096 keys only while the key pages were whole rows
+            wide = 1 if layout.head_dim > 128 else 2
             # One launch takes the requests of few tokens along (a decoded token fills part of a tile): in a
             # step of portions beside decoded tokens two launches one after the other cost 11 us each at the
             # 1.5B sizes, and the walk of a decoded token's keys is the same in either kernel.

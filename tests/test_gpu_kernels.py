@@ -124,6 +124,21 @@ def test_products_without_the_library(own_kernels, rows, inner, outer):
     torch.testing.assert_close(gated.cpu().double(), want, **TOLERANCE[dtype])
 
 
+def key_pieces(rows):
+    """Key pages written as rows [pages, kv, offset, dim] -> as the cache keeps them, in pieces of eight
+    elements, the same piece of all the keys of a page side by side: [pages, kv, dim / w, offset, w]
+    (a head size that is no multiple of 8 is one piece)."""
+    pages, kv, page, dim = rows.shape
+    width = 8 if dim % 8 == 0 else dim
+    return rows.view(pages, kv, page, dim // width, width).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def key_rows(pieces):
+    """The inverse of `key_pieces`."""
+    pages, kv, count, page, width = pieces.shape
+    return pieces.permute(0, 1, 3, 2, 4).reshape(pages, kv, page, count * width)
+
+
 def paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=0, spare_pages=3):
     """Requests with `lengths[i]` cached tokens of which the last `counts[i]` are this step's.
     Returns the step's batch, the cell with garbage in every unused slot, and per-request q, k, v."""
@@ -166,7 +181,7 @@ def paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=
         state_slots=ints(list(range(len(lengths)))), groups=[group], logit_rows=ints([]), num_logit_rows=0,
         max_query_length=max(counts), max_context_length=max(lengths),
     )
-    cell = CacheCell(PagedKeyValue(kv_heads, dim), True, 0, keys.to("cuda", dtype), values.to("cuda", dtype))
+    cell = CacheCell(PagedKeyValue(kv_heads, dim), True, 0, key_pieces(keys).to("cuda", dtype), values.to("cuda", dtype))
     return batch, cell, per_request, HeadLayout(heads, kv_heads, dim)
 
 
@@ -235,13 +250,13 @@ def test_paged_attention_window_edge(kernels, dtype, window):
 
 
 def _rewrite_cell(batch, cell, per_request, page, dtype):
-    keys, values = cell.keys.cpu().float(), cell.values.cpu().float()
+    keys, values = key_rows(cell.keys.cpu().float()), cell.values.cpu().float()
     tables = batch.groups[0].block_tables.cpu()
     for index, (q, k, v) in enumerate(per_request):
         for position in range(k.shape[0]):
             keys[tables[index, position // page], :, position % page] = k[position]
             values[tables[index, position // page], :, :, position % page] = v[position]
-    cell.keys, cell.values = keys.to("cuda", dtype), values.to("cuda", dtype)
+    cell.keys, cell.values = key_pieces(keys).to("cuda", dtype), values.to("cuda", dtype)
     return batch, cell, per_request, None
 
 
@@ -289,8 +304,8 @@ def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, wind
 
 @pytest.mark.parametrize("window", [None, 1500])
 def test_paged_attention_portion_of_a_long_context(kernels, window):
-    """Beyond 4,096 keys the bfloat16 kernel carries four column tiles a wave: a portion at the end of
-    such a context, with a far key that dominates and, with a window, lies just inside it."""
+    """A portion at the end of a context of more than 4,096 keys (hundreds of steps a wave, many
+    pages), with a far key that dominates and, with a window, lies just inside it."""
     heads, kv_heads, dim, page, dtype = 6, 2, 64, 16, torch.bfloat16
     lengths, counts = [4200, 37], [150, 37]
     batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=3)
@@ -327,14 +342,14 @@ def test_rotate_and_store(kernels, dtype, pairing, heads, kv_heads, dim, page):
     expected = torch.cat([rotate(view[:, : heads + kv_heads], angles), view[:, heads + kv_heads :]], dim=1)
     torch.testing.assert_close(qkv.cpu().double().view_as(expected), expected, **TOLERANCE[dtype])
     slots = batch.groups[0].slot_mapping.cpu().long()
-    stored_k = cell.keys.cpu().double()[slots // page, :, slots % page]
+    stored_k = key_rows(cell.keys.cpu().double())[slots // page, :, slots % page]
     stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
     torch.testing.assert_close(stored_k, expected[:, heads : heads + kv_heads], **TOLERANCE[dtype])
     torch.testing.assert_close(stored_v, expected[:, heads + kv_heads :], atol=0, rtol=0)
     untouched = torch.ones(cell.keys.shape[0], page, dtype=torch.bool)
     untouched[slots // page, slots % page] = False
     same = lambda a, b: torch.equal(torch.nan_to_num(a.float().cpu(), nan=7.0), torch.nan_to_num(b.float().cpu(), nan=7.0))
-    assert same(cell.keys.transpose(1, 2)[untouched], before_keys.transpose(1, 2)[untouched])
+    assert same(key_rows(cell.keys).transpose(1, 2)[untouched], key_rows(before_keys).transpose(1, 2)[untouched])
     assert same(cell.values.permute(0, 3, 1, 2)[untouched], before_values.permute(0, 3, 1, 2)[untouched])
     # a cell that is only read stores nothing
     readonly = types.SimpleNamespace(writable=False)
@@ -431,7 +446,7 @@ def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
         expected.append(full[-1:].flatten(1))
     _rewrite_cell(batch, cell, per_request, page, dtype)
     slots = batch.groups[0].slot_mapping.cpu().long()
-    cell.keys[slots // page, :, slots % page] = float("nan")
+    cell.keys[slots // page, :, :, slots % page] = float("nan")
     cell.values[slots // page, :, :, slots % page] = float("nan")
     rows = []  # the step's rows carry unrotated q and k
     for (q, k, v), original in zip(per_request, [p[1] for p in paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=dim + page)[2]]):
@@ -439,7 +454,7 @@ def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
     qkv = on_gpu(torch.cat(rows), dtype)
     out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None if pairing == "none" else on_gpu(inverse), pairing, 0.2, None)
     torch.testing.assert_close(out.cpu().double(), torch.cat(expected), **TOLERANCE[dtype])
-    stored_k = cell.keys.cpu().double()[slots // page, :, slots % page]
+    stored_k = key_rows(cell.keys.cpu().double())[slots // page, :, slots % page]
     stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
     want_k = torch.stack([p[1][-1].double() for p in per_request])
     want_v = torch.stack([rounded(p[2][-1], dtype) for p in per_request])
@@ -462,7 +477,7 @@ def test_fused_decode_attention_over_long_contexts(kernels, requests):
         k[far] = 3.0 * q[-1, ::6]  # kv head g takes the query of its first head: heads 0 and 6 find this key
     _rewrite_cell(batch, cell, per_request, page, dtype)
     slots = batch.groups[0].slot_mapping.cpu().long()
-    cell.keys[slots // page, :, slots % page] = float("nan")  # the step itself stores the newest key and value
+    cell.keys[slots // page, :, :, slots % page] = float("nan")  # the step itself stores the newest key and value
     cell.values[slots // page, :, :, slots % page] = float("nan")
     qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
     out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None, "none", 1.0, None).cpu().double()

@@ -252,8 +252,8 @@ def test_captured_mixed_steps_at_benchmark_layer_sizes(wide_models, dtype):
 
 
 def test_a_long_context_through_the_whole_engine(wide_models):
-    """Beyond 4,096 keys the bfloat16 attention carries four column tiles a wave for portions and cuts a decoded
-    token's keys into splits (merged by the output projection, or by the merging kernel): the whole engine at
+    """Over thousands of keys a prompt portion's waves walk hundreds of steps and pages, and a decoded token's
+    keys are cut into splits (merged by the output projection, or by the merging kernel): the whole engine at
     the 1.5B widths over 4,400 keys, a prompt in portions of changing size, a portion beside decoded tokens
     of another long request, then single tokens; against the plain forward."""
     from llmserve_amd import CacheConfig, ModelRunner, StepEntry

@@ -78,7 +78,7 @@ class TorchKernels:
             group = batch.groups[cell.group]
             slots = group.slot_mapping.long()
             pages, offsets = slots // group.page_size, slots % group.page_size
-            cell.keys[pages, :, offsets] = view[:, heads : heads + kv_heads]
+            cell.put_key_rows(pages, offsets, view[:, heads : heads + kv_heads])  # pages are [kv, dim / w, offset, w]
             cell.values[pages, :, :, offsets] = view[:, heads + kv_heads :]  # pages are [kv, dim, offset]
 
     def paged_attention(self, qkv, layout, batch, cell, scale, window, *, score_slopes=None, soft_cap=None):
@@ -95,7 +95,7 @@ class TorchKernels:
                 where = torch.arange(first, position + 1)
                 pages = table[where // group.page_size]
                 assert (pages >= 0).all(), "attention reads a page that was given back"
-                keys = cell.keys[pages, :, where % group.page_size].float()  # [n, kv, D]
+                keys = cell.key_rows(pages, where % group.page_size).float()  # [n, kv, D]
                 values = cell.values[pages, :, :, where % group.page_size].float()
                 keys = keys.repeat_interleave(heads // kv_heads, dim=1)
                 values = values.repeat_interleave(heads // kv_heads, dim=1)
