@@ -274,6 +274,199 @@ static int launch_pair(const void* x, const void* w, const void* bias, int bias_
   return LAUNCH_STATUS();
 }
 
+// ---------------------------------------------------------------------------- the streams through LDS
+// gemm_stream: gemm_skinny / gemm_pair for up to 16 rows of x with both operands brought through LDS.
+// The matrix cores take a weight row as a row of the A operand, lane (r, g) holding k = 8g .. 8g+7 of
+// row r, so the four lanes the address unit serves together (r .. r+3 at one g) would read 16 bytes
+// of four different rows, four cache lines, and a load of a wave costs that unit four times what
+// 64 bytes in a row cost it; x is read the same way.  Here lane L instead asks for piece L % 4 of row
+// L / 4 (a quad reads 64 bytes of one row), straight into LDS (global_load_lds_dwordx4: the wave's 1 KB
+// lands in lane order), and lane (r, g) reads its operand back from slot 4 r + g.  The pieces of a
+// row are swizzled by bits 1-2 of the row so that the eight lanes LDS serves together hit all banks.
+// Every wave has STAGES stages of its own, a stage holding one group of G steps of 32 k of its NT
+// weight tiles and of x; nothing is shared between waves before the end, so the only waits are the
+// wave's own: for its loads to land (counted, so that the younger stage may still be under way) and
+// for its reads to come back before the stage is asked for anew.  The reads of LDS are written as
+// instructions: left to the compiler, every read of LDS waits for all loads into LDS under way.
+#define STREAM_STAGES 2
+#define STREAM_CHUNK 1024  // one 32-k step of 16 rows
+
+template <int OFFSET>
+__device__ __forceinline__ void stream_read(bf16x8& operand, unsigned at) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(operand) : "v"(at), "n"(OFFSET) : "memory");
+}
+template <int I, int COUNT>
+struct StreamReads {
+  static __device__ __forceinline__ void run(bf16x8* operands, unsigned at) {
+    stream_read<I * STREAM_CHUNK>(operands[I], at);
+    StreamReads<I + 1, COUNT>::run(operands, at);
+  }
+};
+template <int COUNT>
+struct StreamReads<COUNT, COUNT> {
+  static __device__ __forceinline__ void run(bf16x8*, unsigned) {}
+};
+template <int N>
+__device__ __forceinline__ void stream_wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int WAVES, int NT, int G, typename TO, bool GATED>
+__global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x,
+                                                                 const bf16_t* __restrict__ w,
+                                                                 const void* __restrict__ bias, int bias_is_float,
+                                                                 TO* __restrict__ out, int M, int N, int K,
+                                                                 int k_split) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];
+  constexpr int OPERANDS = (NT + 1) * G;                 // of one group: the weight tiles' steps, then x's
+  constexpr int STAGE_BYTES = OPERANDS * STREAM_CHUNK;
+  constexpr int WAVE_BYTES = STREAM_STAGES * STAGE_BYTES;
+  static_assert(OPERANDS <= 31, "a group's loads are counted in vmcnt beside a second group's");
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int k_first = blockIdx.y * k_split;
+  // what this lane asks for: piece (L % 4) ^ f(row) of row L / 4, and where lane (r, g) finds its own
+  const int load_row = lane >> 2, load_piece = (lane & 3) ^ ((load_row >> 1) & 3);
+  const bf16_t* w_src[NT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s)
+    w_src[s] = w + (size_t)min(((int)blockIdx.x * NT + s) * 16 + load_row, N - 1) * K + k_first + load_piece * 8;
+  // rows of x beyond M are read as row M - 1: their columns of the result are dropped at the end
+  const bf16_t* x_src = x + (size_t)min(load_row, M - 1) * K + k_first + load_piece * 8;
+  unsigned char* mine = stream_lds + (size_t)wave * WAVE_BYTES;
+  const unsigned read_at = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)mine +
+                           (unsigned)(4 * r + (g ^ ((r >> 1) & 3))) * 16;
+
+  // the bias of the four outputs this lane will finish (wave s finishes tile s) is asked for now
+  float bias_here[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias && blockIdx.y == 0 && wave < NT) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      bias_here[i] = load_as_float(bias, bias_is_float, min(((int)blockIdx.x * NT + wave) * 16 + g * 4 + i, N - 1));
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // so that the counts below count the stream alone
+
+  auto request = [&](int group, int stage) {
+    unsigned char* to = mine + (size_t)stage * STAGE_BYTES;
+    const int k = group * G * STEP;
+#pragma unroll
+    for (int u = 0; u < G; ++u) {
+#pragma unroll
+      for (int s = 0; s < NT; ++s)
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(w_src[s] + k + u * STEP),
+                                         (void __attribute__((address_space(3)))*)(to + (s * G + u) * STREAM_CHUNK), 16,
+                                         0, 0);
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(x_src + k + u * STEP),
+                                       (void __attribute__((address_space(3)))*)(to + (NT * G + u) * STREAM_CHUNK), 16, 0,
+                                       0);
+    }
+  };
+
+  f32x4 acc[NT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s) acc[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const int groups = k_split / (STEP * G);
+  int group = wave;
+  if (group < groups) request(group, 0);
+  if (group + WAVES < groups) request(group + WAVES, 1);
+  for (int stage = 0; group < groups; group += WAVES, stage ^= 1) {
+    // this stage has landed once at most the next group's loads are under way
+    if (group + WAVES < groups) stream_wait_loads<OPERANDS>();
+    else stream_wait_loads<0>();
+    bf16x8 operands[OPERANDS];
+    StreamReads<0, OPERANDS>::run(operands, read_at + (unsigned)stage * STAGE_BYTES);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < OPERANDS; ++i) asm volatile("" : "+v"(operands[i]));  // used only after the wait
+    if (group + 2 * WAVES < groups) request(group + 2 * WAVES, stage);       // the stage is read: ask anew
+#pragma unroll
+    for (int u = 0; u < G; ++u)
+#pragma unroll
+      for (int s = 0; s < NT; ++s)
+        acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(operands[s * G + u], operands[NT * G + u], acc[s], 0, 0, 0);
+  }
+
+  __syncthreads();  // every wave is done with its stages: LDS is free for the waves' sums
+  float* partial = (float*)stream_lds;  // [WAVES][NT][64 lanes][4]
+#pragma unroll
+  for (int s = 0; s < NT; ++s) *(f32x4*)(partial + ((wave * NT + s) * 64 + lane) * 4) = acc[s];
+  __syncthreads();
+  if (wave >= NT) return;
+  const int s = wave;
+  f32x4 total = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int v = 0; v < WAVES; ++v) total += *(const f32x4*)(partial + ((v * NT + s) * 64 + lane) * 4);
+  const int m = r;
+  const int n_first = ((int)blockIdx.x * NT + s) * 16 + g * 4;
+  if (m >= M) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) total[i] += bias_here[i];
+  if (GATED) {
+    TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (n_first + 2 * i + 1 < N) {
+        const float gate = total[2 * i], up = total[2 * i + 1];
+        dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+      }
+    }
+  } else {
+    TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n_first + i < N) dst[i] = from_float<TO>(total[i]);
+  }
+}
+
+template <int WAVES, int NT, int G, typename TO, bool GATED>
+static int launch_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
+                         int K, int splits, hipStream_t stream) {
+  const size_t lds = (size_t)WAVES * STREAM_STAGES * (NT + 1) * G * STREAM_CHUNK;
+  if (lds > 64 * 1024) {
+    static bool asked = false;
+    if (!asked) {
+      if (hipFuncSetAttribute((const void*)gemm_stream_kernel<WAVES, NT, G, TO, GATED>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return ERR_BAD_ARGUMENT;
+      asked = true;
+    }
+  }
+  hipLaunchKernelGGL((gemm_stream_kernel<WAVES, NT, G, TO, GATED>), dim3((N + 16 * NT - 1) / (16 * NT), splits),
+                     dim3(WAVES * 64), lds, stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M,
+                     N, K, K / splits);
+  return LAUNCH_STATUS();
+}
+
+// One tile a wave in groups of four steps, or two tiles in groups of two.  Measured at 8 rows against
+// gemm_skinny / gemm_pair, in a captured chain over different weights: 1.5B sizes qkv 4.9 -> 4.1 us,
+// gate/up 15.7 -> 13.0, down 9.5 -> 8.7, o 4.8 -> 3.4; 7B sizes qkv 13.8 -> 10.6 (two tiles), o 9.8 ->
+// 7.9, gate/up 54.7 -> 52.1; 32B sizes qkv 20.9 -> 16.3 (two tiles).  Where a wave walks a long K
+// for four tiles that share its x (the down projections and the 32B sizes' gate/up) gemm_pair's
+// registers stay ahead, and the caller keeps it there.
+// M <= 16, K / splits a multiple of 128.
+template <typename TO, bool GATED>
+static int pick_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
+                       int splits, hipStream_t stream) {
+  const long tiles = (N + 15) / 16;
+  if (tiles >= 256 && tiles < 1024 && tiles * K >= (1L << 20))
+    return launch_stream<4, 2, 2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  return launch_stream<4, 1, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+}
+
+// The same product as llmserve_gemm_skinny, always through gemm_stream (tests and measurements).
+extern "C" int llmserve_gemm_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
+                                    int out_is_float, int gated, int M, int N, int K, int splits,
+                                    hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K <= 0 || splits < 1 || K % splits || (K / splits) % (STEP * GROUP) || (gated && N % 2))
+    return ERR_BAD_ARGUMENT;
+  if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
+  if (gated)
+    return out_is_float ? pick_stream<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                        : pick_stream<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+  return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
+                      : pick_stream<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+}
+
 // ---------------------------------------------------------------------------- key splits merged on the way in
 // gemm_merged: gemm_skinny for up to 16 rows whose x is the output of decode attention that was left in
 // key splits (attention_bf16.hip, `unmerged`): for every (row, head) S results, each divided by its own sum
@@ -1029,6 +1222,14 @@ extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bi
     const int share = (per_wave >= 8 && by_four >= 128 && (M > 2 || tiles <= 1024)) || (tiles >= 4096 && M >= 4) ? 4
                       : (per_wave >= 4 || M > 8 || (tiles >= 4096 && M >= 4)) && by_two * 4 >= TARGET_WAVES ? 2
                                                                                                             : 1;
+    // Two tiles or one: through LDS (gemm_stream), unless many rows of x meet a long walk over K.
+    if (share != 4 && !(share == 2 && M > 8 && per_wave >= 4)) {
+      if (gated)
+        return out_is_float ? pick_stream<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                            : pick_stream<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+      return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
+                          : pick_stream<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+    }
 #define PAIR_CASE(NT)                                                                                              \
   if (share == NT) {                                                                                               \
     if (gated)                                                                                                     \

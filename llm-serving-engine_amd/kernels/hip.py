@@ -52,6 +52,7 @@ _SIGNATURES = {
     "llmserve_gather_rows": "ppiippiip",
     "llmserve_gemm_generic": "pipipipiiiip",
     "llmserve_gemm_skinny": "pppipiiiiiip",
+    "llmserve_gemm_stream": "pppipiiiiiip",
     "llmserve_gemm_medium": "pppipiiiiiip",
     "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",

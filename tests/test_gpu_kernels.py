@@ -551,3 +551,42 @@ def test_library_products_cut_over_a_long_k(kernels, rows, inner, outer):
     normed = k.add_rms_norm(device_hidden, parts, on_gpu(torch.ones(outer), dtype), 1e-6)
     torch.testing.assert_close(device_hidden.cpu().double(), hidden.double() + expected, atol=2e-3, rtol=1e-3)
     torch.testing.assert_close(normed.cpu().double(), plain.rms_norm(hidden.double() + expected, torch.ones(outer).double(), 1e-6), **TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("rows", [1, 7, 16])
+@pytest.mark.parametrize("outer,inner,gated,splits,bias", [
+    (40, 128, False, 1, None), (1000, 384, False, 1, "bfloat16"), (4610, 3584, False, 1, "float32"),  # two tiles a wave
+    (154, 2560, False, 5, None), (318, 256, True, 1, None), (6000, 1536, True, 1, None),
+])
+def test_products_streamed_through_lds(kernels, rows, outer, inner, gated, splits, bias):
+    """The product for up to 16 rows that brings weights and x through LDS, quad by quad, alone: odd
+    numbers of weight rows (the last tile is cut), one and two tiles a wave, a bias of either type,
+    K cut into partial sums, SiLU(gate) * up over interleaved rows; against the plain product."""
+    from llmserve_amd.kernels.hip import _check, _pointer
+
+    k = kernels[torch.bfloat16]
+    x, w = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner)
+    b = None if bias is None else torch.randn(outer)
+    device_x, device_w = on_gpu(x, torch.bfloat16), on_gpu(w, torch.bfloat16)
+    device_b = None if b is None else on_gpu(b, getattr(torch, bias))
+    float_out = splits > 1 or bias == "float32"
+    out = torch.full((splits, rows, outer // 2 if gated else outer), float("nan"), device="cuda",
+                     dtype=torch.float32 if float_out else torch.bfloat16)
+    status = k._gemm_bf16.llmserve_gemm_stream(
+        _pointer(device_x), _pointer(device_w), _pointer(device_b), int(bias == "float32"), _pointer(out), int(float_out),
+        int(gated), rows, outer, inner, splits, k._stream,
+    )
+    _check(status, "gemm_stream")
+    expected = rounded(x, torch.bfloat16) @ rounded(w, torch.bfloat16).T
+    if b is not None:
+        expected = expected + rounded(b, getattr(torch, bias))
+    if gated:
+        expected = torch.nn.functional.silu(expected[:, 0::2]) * expected[:, 1::2]  # weight rows alternate gate, up
+    got = out.sum(0).cpu().double()
+    tolerance = dict(atol=2e-3, rtol=2e-3) if float_out else TOLERANCE[torch.bfloat16]
+    torch.testing.assert_close(got, expected, **tolerance)
+    # and it refuses what it cannot take: more than 16 rows, a K that is no multiple of 128
+    assert k._gemm_bf16.llmserve_gemm_stream(_pointer(device_x), _pointer(device_w), None, 0, _pointer(out), int(float_out),
+                                             0, 17, outer, inner, 1, k._stream) != 0
+    assert k._gemm_bf16.llmserve_gemm_stream(_pointer(device_x), _pointer(device_w), None, 0, _pointer(out), int(float_out),
+                                             0, rows, outer, inner - 32, 1, k._stream) != 0
