@@ -551,18 +551,26 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
       } else {
         const size_t slot = (row * heads + head) * splits + blockIdx.z;
         if (fused.unmerged) {
-          bf16_t* dst = (bf16_t*)partial_acc + slot * D + d4;
+          // for the product that merges: [head][split][piece of 8][16 rows][8], the rows of a piece side by
+          // side, so that the four lanes of its loads that hold four rows' share of a piece read 64 bytes
+          // in a row (the step has at most 16 rows)
+          const size_t of_split = (size_t)head * splits + blockIdx.z;
+          bf16_t* dst = (bf16_t*)partial_acc + ((of_split * (D / 8) + d4 / 8) * 16 + row) * 8 + d4 % 8;
           const float inverse = total > 0.f ? 1.f / total : 0.f;
 #pragma unroll
           for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
+          if (d4 == 0) {
+            partial_ml[(of_split * 16 + row) * 2] = best;
+            partial_ml[(of_split * 16 + row) * 2 + 1] = total;
+          }
         } else {
           float* dst = partial_acc + slot * D + d4;
 #pragma unroll
           for (int i = 0; i < 4; ++i) dst[i] = merged[i];
-        }
-        if (d4 == 0) {
-          partial_ml[slot * 2] = best;
-          partial_ml[slot * 2 + 1] = total;
+          if (d4 == 0) {
+            partial_ml[slot * 2] = best;
+            partial_ml[slot * 2 + 1] = total;
+          }
         }
       }
     }
@@ -862,9 +870,10 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // of the step must lie in one of the tiles: a second kernel merges the splits of all rows.
 // With `fuse` tile i is row i, the one token of request i (`work` is not read), qkv is as the projection left it, and the kernel
 // rotates (table of cos and sin per row, pairing) and stores the token's key and value at slots[row] itself.
-// `fuse` + 2 leaves the key splits unmerged for a reader that merges them itself (gemm_merged): partial_acc is
-// then bfloat16 [rows * heads * splits * D], each split's result divided by its own sum of weights, and
-// partial_ml holds each split's maximum (in units of log2) and sum of weights as before.
+// `fuse` + 2 leaves the key splits unmerged for a reader that merges them itself (gemm_merged; at most 16 rows):
+// partial_acc is then bfloat16 [heads][splits][D / 8][16 rows][8], each split's result divided by its own sum of
+// weights, and partial_ml [heads][splits][16 rows][2] holds each split's maximum (in units of log2) and sum of
+// weights.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
                                         float* partial_ml, void* keys, void* values,
                                         const int* block_tables, int table_width, const int* positions,
@@ -879,6 +888,7 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   const int group = heads / kv_heads;
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
   const bool unmerged = (fuse & 2) != 0 && splits > 1;  // the splits stay as they are: whoever reads them merges them
+  if (unmerged && rows > 16) return ERR_BAD_ARGUMENT;
   fuse &= 1;
   FusedDecode fused = {(const float2*)table, pairing, slots, unmerged ? 1 : 0};
   int status;

@@ -504,14 +504,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_merged_kernel(const bf16_t* _
     bf16x8 a[GROUP];
 #pragma unroll
     for (int u = 0; u < GROUP; ++u) a[u] = load8_stream(w_row + (group * GROUP + u) * STEP);
-    const size_t slot = ((size_t)row * heads + head_first + group) * S;
+    // split_x is [head][split][piece of 8][16 rows][8]: this lane's piece 4 u + g of row `row`, beside the
+    // same piece of the next rows, which the next lanes ask for
+    const size_t slot = (size_t)(head_first + group) * S;
     float2 ml[S];
     bf16x8 piece[S][GROUP];
 #pragma unroll
     for (int s = 0; s < S; ++s) {
-      ml[s] = *(const float2*)(split_ml + (slot + s) * 2);
+      ml[s] = *(const float2*)(split_ml + ((slot + s) * 16 + row) * 2);
 #pragma unroll
-      for (int u = 0; u < GROUP; ++u) piece[s][u] = load8(split_x + (slot + s) * (STEP * GROUP) + u * STEP + g * 8);
+      for (int u = 0; u < GROUP; ++u)
+        piece[s][u] = load8(split_x + (((slot + s) * (STEP * GROUP / 8) + u * 4 + g) * 16 + row) * 8);
     }
     float best = -INFINITY;
 #pragma unroll
@@ -566,7 +569,7 @@ static int launch_merged(const void* split_x, const float* split_ml, const void*
 }
 
 // out [k_splits, M, N] float32 partial sums of x . w^T (+ bias in the first), x [M, K] being the merge of
-// split_x bfloat16 [M, K / 128, splits, 128] with split_ml float32 [M, K / 128, splits, 2] as above.
+// split_x bfloat16 [K / 128, splits, 16, 16 rows, 8] with split_ml float32 [K / 128, splits, 16 rows, 2] as above.
 // M <= 16; K a multiple of 128 * k_splits; splits 2, 3, 4, 6 or 8.
 extern "C" int llmserve_gemm_merged(const void* split_x, const float* split_ml, int splits, const void* w,
                                     const void* bias, int bias_is_float, float* out, int M, int N, int K,

@@ -675,8 +675,9 @@ class HipKernels:
                     else:
                         unmerged = False
                 if splits > 1:
-                    partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), qkv.dtype if unmerged else torch.float32)
-                    partial_ml = self._empty((tokens * heads * splits * 2,), torch.float32)
+                    held = 16 if unmerged else tokens  # the product that merges wants 16 rows side by side
+                    partial_acc = self._empty((held * heads * splits * layout.head_dim,), qkv.dtype if unmerged else torch.float32)
+                    partial_ml = self._empty((held * heads * splits * 2,), torch.float32)
             table, pairing = fuse if fuse is not None else (None, "none")
             status = library.llmserve_attention_tiles(
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
