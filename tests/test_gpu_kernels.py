@@ -590,3 +590,45 @@ def test_products_streamed_through_lds(kernels, rows, outer, inner, gated, split
                                              0, 17, outer, inner, 1, k._stream) != 0
     assert k._gemm_bf16.llmserve_gemm_stream(_pointer(device_x), _pointer(device_w), None, 0, _pointer(out), int(float_out),
                                              0, rows, outer, inner - 32, 1, k._stream) != 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("pairing", ["adjacent", "half"])
+@pytest.mark.parametrize("heads,kv_heads,dim,page,lengths,counts", [
+    (12, 2, 128, 16, [700, 301, 40, 2100], [150, 1, 40, 33]),   # portions beside a decoded token, packed columns
+    (28, 4, 128, 16, [512] * 9, [512] * 9),                     # many whole prompts: the kernel that shares K and V through LDS
+    (6, 1, 64, 8, [90, 17], [90, 2]),
+    (40, 2, 64, 16, [130, 64], [30, 64]),                       # more than 16 query heads a kv head
+    (4, 2, 48, 16, [70, 5], [70, 5]),
+])
+def test_rotation_store_and_attention_of_prompt_portions(kernels, dtype, pairing, heads, kv_heads, dim, page, lengths, counts):
+    """`rotate_store_attend` on steps that are not single tokens (rotation and store, then attention).
+    The step's rows carry unrotated q and k, the pages hold the earlier tokens' rotated keys and garbage
+    where the step's will go; results and pages against the plain implementation."""
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=dim + heads)
+    originals = [(q.clone(), k.clone(), v.clone()) for q, k, v in per_request]
+    theta = 3000.0
+    inverse = 1.0 / (theta ** (torch.arange(0, dim, 2).float() / dim))
+    rotate = {"adjacent": plain.rope_adjacent, "half": plain.rope_half}[pairing]
+    expected, rotated_keys = [], []
+    for index, (q, k, v) in enumerate(per_request):
+        angles = plain.rope_angles(dim, theta, torch.arange(q.shape[0]))
+        k_rot = rotate(rounded(k, dtype), angles).to(dtype).double()
+        q_rot = rotate(rounded(q, dtype), angles).to(dtype).double()
+        per_request[index] = (q, k_rot.float(), v)
+        rotated_keys.append(k_rot)
+        full = plain.causal_attention(q_rot, k_rot, rounded(v, dtype), 0.2)
+        expected.append(full[-counts[index]:].flatten(1))
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    slots = batch.groups[0].slot_mapping.cpu().long()
+    cell.keys[slots // page, :, :, slots % page] = float("nan")  # the step stores these itself
+    cell.values[slots // page, :, :, slots % page] = float("nan")
+    qkv = on_gpu(step_rows(originals, counts, heads, kv_heads, dim), dtype)
+    out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, on_gpu(inverse), pairing, 0.2, None)
+    torch.testing.assert_close(out.cpu().double(), torch.cat(expected), **TOLERANCE[dtype])
+    stored_k = key_rows(cell.keys.cpu().double())[slots // page, :, slots % page]
+    stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
+    want_k = torch.cat([k_rot[-count:] for k_rot, count in zip(rotated_keys, counts)])
+    want_v = torch.cat([rounded(v, dtype)[-count:] for (q, k, v), count in zip(originals, counts)])
+    torch.testing.assert_close(stored_k, want_k, **TOLERANCE[dtype])
+    torch.testing.assert_close(stored_v, want_v, atol=0, rtol=0)
