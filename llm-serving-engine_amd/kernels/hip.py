@@ -311,14 +311,17 @@ class HipKernels:
     def _partial_splits(out_features: int, in_features: int) -> int:
         """Into how many parts of K a weight-streaming product is cut when its float32 result
         may stay in parts: a weight with few rows has too few 16-row tiles to fill the chip, so
-        K is cut (at most 8 ways, parts of at least 512) until about a thousand workgroups run."""
+        K is cut (at most 8 ways) until about a thousand workgroups run.  A part is at least 512 long,
+        and 1,536 where K allows it: shorter walks cost more in waves that start and end than
+        they gain (the 1.5B sizes' down projection at 8 rows: five parts 7.8 us, seven 8.4, two 8.1)."""
         groups = in_features // 128
         if in_features % 128 or groups < 8:
             return 1
         tiles = -(-out_features // 16)
+        shortest = 12 if groups >= 24 else 4
         best = 1
         for splits in range(2, 9):
-            if groups % splits == 0 and groups // splits >= 4 and tiles * splits <= 1024:
+            if groups % splits == 0 and groups // splits >= shortest and tiles * splits <= 1024:
                 best = splits
         return best
 
