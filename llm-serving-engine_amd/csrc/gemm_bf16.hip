@@ -447,7 +447,10 @@ template <typename TO, bool GATED>
 static int pick_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
                        int splits, hipStream_t stream) {
   const long tiles = (N + 15) / 16;
-  if (tiles >= 256 && tiles < 1024 && tiles * K >= (1L << 20))
+  // two tiles a wave for a middling number of weight rows over a K that is not cut (the qkv products of the
+  // 7B and 32B sizes: 11.6 -> 10.6 and 20.0 -> 17.5 us); with K cut over workgroups one tile is as good or
+  // better (the 32B sizes' o in two parts: 13.5 us against 16.9)
+  if (splits == 1 && tiles >= 256 && tiles < 1024 && tiles * K >= 1000000L)
     return launch_stream<4, 2, 2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
   return launch_stream<4, 1, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
 }
