@@ -423,3 +423,41 @@ def test_captured_graphs_are_dropped_by_last_use_and_captured_again(model_folder
     assert seen[3] == [(4, 1), (1, 1)]  # which was captured again when it came back
     assert seen[5][-1] == (2, 1) and seen[-1][-1] == (1, 1)
     runner.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_the_host_reads_the_pages_as_the_kernels_wrote_them(model_folders, dtype, name):
+    """The cache manager's host-side read path (`gather`) and the kernels agree on where a key and a
+    value lie in a page: after a prompt fed in portions and three tokens decoded one by one (these are
+    stored by the fused decode attention in bfloat16), the first layer's pages hold, position by position,
+    the rotated keys and the values the plain implementation computes."""
+    from llmserve_amd.kernels import HipKernels
+
+    config, page = CONFIGS[name]
+    plain_config, weights = plain.PlainConfig.from_folder(model_folders[name]), plain.read_weights(model_folders[name])
+    tokens = random_tokens(3 * page + 8, config.vocab_size, seed=9)
+    loaded = load_model_folder(model_folders[name], dtype)
+    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(page, 16, 2))
+    cut = len(tokens) - 3
+    for start, end in ((0, page + 3), (page + 3, page + 4), (page + 4, cut)):
+        runner.step([StepEntry("r", tokens[start:end], [])], create_missing=True)
+    for token in tokens[cut:]:
+        runner.step([StepEntry("r", [token], [0])])
+    count = len(tokens)
+    hidden = weights["embed_tokens.weight"][torch.tensor(tokens)]
+    normed = plain.rms_norm(hidden, weights["layers.0.input_layernorm.weight"], plain_config.rms_norm_eps)
+    prefix = "layers.0.self_attn."
+    shape = (count, plain_config.num_kv_heads, plain_config.head_dim)
+    bias = lambda which: weights.get(prefix + which + "_proj.bias", 0.0)  # C has no q/k/v biases
+    keys = (normed @ weights[prefix + "k_proj.weight"].T + bias("k")).view(shape)
+    values = (normed @ weights[prefix + "v_proj.weight"].T + bias("v")).view(shape)
+    rotate = plain.rope_half if plain_config.rope_pairing == "half" else plain.rope_adjacent
+    keys = rotate(keys, plain.rope_angles(plain_config.head_dim, plain_config.rope_theta, torch.arange(count)))
+    first, cached_keys, cached_values = runner.cache.gather("r", 0)
+    assert first == 0 and cached_keys.shape == shape
+    tolerance = dict(atol=1e-5, rtol=1e-5) if dtype == "float32" else dict(atol=3e-2, rtol=3e-2)
+    torch.testing.assert_close(cached_keys.cpu().double(), keys, **tolerance)
+    torch.testing.assert_close(cached_values.cpu().double(), values, **tolerance)
+    runner.close()
