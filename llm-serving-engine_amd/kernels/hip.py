@@ -609,11 +609,12 @@ class HipKernels:
 
     def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None, unmerged=False):
         """The MFMA kernel: requests that bring a few tokens (decoding) one column tile per
-        wave, split over the keys when there are few of them; longer portions two or four
-        tiles per wave.  `fuse` = (rotary table, pairing) lets a step of single tokens rotate and
+        wave, split over the keys when there are few of them; longer portions two tiles
+        per wave.  `fuse` = (rotary table, pairing) lets a step of single tokens rotate and
         store inside the same kernel.  With `unmerged` (a step of single tokens whose reader merges
-        key splits itself) the keys are split more finely and the splits are returned as they are,
-        (bfloat16 [T, heads, splits, D], float32 [T, heads, splits, 2], splits), instead of `out`."""
+        key splits itself) the keys are split more finely and the splits are returned as they are
+        (their results in bfloat16, laid out for `gemm_merged`; their maxima and sums in float32; how
+        many), instead of `out`."""
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
         per_tile = max(1, 16 // (heads // kv_heads))
