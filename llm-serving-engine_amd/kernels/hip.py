@@ -63,7 +63,8 @@ _SIGNATURES = {
     "llmserve_attention_can_fuse": "i",
     "llmserve_argmax": "ppppiip",
     "llmserve_argmax_static": "ppiip",
-    "llmserve_sample": "ppppppiip",
+    "llmserve_sample_workspace_kib": "ii",
+    "llmserve_sample": "pppppipiiip",
 }
 _TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 
@@ -176,6 +177,14 @@ class HipKernels:
 
     def to_device(self, tensor: torch.Tensor) -> torch.Tensor:
         return tensor.to(self.device).contiguous()
+
+    def queued_to_device(self, tensor: torch.Tensor) -> torch.Tensor:
+        """A small host tensor's values on the device, by a copy that is only queued: it goes through
+        pinned memory, so the host does not wait for the work queued before it (with a pageable
+        source it would, and a step queued ahead would be waited for)."""
+        pinned = torch.empty(tensor.shape, dtype=tensor.dtype, pin_memory=True)
+        pinned.copy_(tensor)
+        return pinned.to(self.device, non_blocking=True)
 
     def _empty(self, shape, dtype) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype, device=self.device)
@@ -772,13 +781,17 @@ class HipKernels:
         _check(status, "argmax")
         return out
 
-    def sample(self, logits, temperatures, top_ps, uniforms) -> torch.Tensor:
+    def sample(self, logits, temperatures, top_ps, uniforms, with_top_p: bool = True) -> torch.Tensor:
         rows, vocab = logits.shape
         out = self._empty((rows,), torch.int32)
-        scratch = self._empty((rows, vocab), torch.float32)
-        status = self._sampling_library().llmserve_sample(
-            _pointer(logits), _pointer(temperatures), _pointer(top_ps), _pointer(uniforms), _pointer(scratch),
-            _pointer(out), rows, vocab, self._stream,
+        library = self._sampling_library()
+        kib = library.llmserve_sample_workspace_kib(rows, vocab)
+        if kib <= 0:
+            raise KernelError(f"sample: no workspace for {rows} rows of {vocab}")
+        workspace = self._empty((kib * 1024,), torch.uint8)
+        status = library.llmserve_sample(
+            _pointer(logits), _pointer(temperatures), _pointer(top_ps), _pointer(uniforms), _pointer(workspace), kib,
+            _pointer(out), rows, vocab, 1 if with_top_p else 0, self._stream,
         )
         _check(status, "sample")
         return out

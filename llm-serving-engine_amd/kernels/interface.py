@@ -20,6 +20,9 @@ class Kernels(Protocol):
 
     def to_device(self, tensor: torch.Tensor) -> torch.Tensor: ...
 
+    def queued_to_device(self, tensor: torch.Tensor) -> torch.Tensor:
+        """As `to_device`, for small per-step inputs: the host does not wait for work queued before."""
+
     def embedding(self, table: torch.Tensor, token_ids: torch.Tensor) -> torch.Tensor:
         """float32 rows [T, hidden] of `table` at `token_ids`."""
 
@@ -73,5 +76,8 @@ class Kernels(Protocol):
     def argmax(self, logits: torch.Tensor) -> torch.Tensor: ...
 
     def sample(
-        self, logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor, uniforms: torch.Tensor
-    ) -> torch.Tensor: ...
+        self, logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor, uniforms: torch.Tensor,
+        with_top_p: bool = True,
+    ) -> torch.Tensor:
+        """One token per row.  `with_top_p=False` promises that no row with a temperature has top_p < 1
+        (a library may then leave the search for the kept set out)."""

@@ -64,5 +64,6 @@ class Sampler:
             ],
             dtype=torch.float32,
         )
-        values = self.kernels.to_device(values)
-        return self.kernels.sample(logits, values[0], values[1], values[2])
+        values = self.kernels.queued_to_device(values)
+        with_top_p = any(config.temperature > 0 and config.top_p < 1 for config in configs)
+        return self.kernels.sample(logits, values[0], values[1], values[2], with_top_p)

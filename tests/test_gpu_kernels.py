@@ -422,6 +422,48 @@ def test_sampling_edges(kernels):
         assert got == want, (u, got, want)
 
 
+@pytest.mark.parametrize("rows,vocab", [(70, 1025), (300, 130), (3, 40000)])
+def test_sampling_of_many_rows_and_hard_rows(kernels, rows, vocab):
+    """The stages cut a row into fewer pieces when there are many rows; rows whose entries are all
+    equal, tie in groups, underflow to zero or to subnormal numbers, or hold one entry far above the
+    rest must come out as the plain rule says; and leaving the top-p stages out changes nothing for
+    rows without top-p."""
+    k = kernels[torch.float32]
+    torch.manual_seed(rows + vocab)
+    logits = 2.0 * torch.randn(rows, vocab)
+    # all equal, as many as a power of two (the plain rule rounds p = 1 / n to float32 before it adds, the kernel
+    # divides nothing: with every entry tied they agree only where 1 / n is exact); the rest can never come
+    equal = 1 << (vocab.bit_length() - 1)
+    logits[0] = 1.5
+    logits[0, equal:] = -float("inf")
+    if vocab <= 2048:
+        # four values, many ties.  Not at the large size: float32 softmax, which the plain rule starts from, is
+        # off from a sum of 1 by a few parts in a million there, and among ten thousand tied entries that
+        # moves the end of the kept set by an entry; the kernel normalises nothing and has no such error
+        logits[1] = torch.randint(0, 4, (vocab,)).float()
+    logits[2, 1:] -= 200.0  # everything but one entry underflows
+    logits[2, 0] = 3.0
+    if rows > 3:
+        logits[3] = torch.linspace(-180.0, 0.0, vocab)  # the low end is subnormal or zero after exp
+        logits[4, vocab // 3] += 30.0
+    temperatures = [(0.0, 0.6, 1.0, 1.7)[row % 4] for row in range(rows)]
+    temperatures[0], temperatures[1], temperatures[2] = 1.0, 0.9, 1.0
+    top_ps = [(1.0, 0.9, 0.5, 0.05, 0.999)[row % 5] for row in range(rows)]
+    top_ps[0], top_ps[1] = 0.5, 0.7
+    for draw in range(3):
+        uniforms = [plain.uniform_for(draw + 20, row) for row in range(rows)]
+        if draw == 2:
+            uniforms[0], uniforms[1] = 0.0, 0.999999
+        got = k.sample(on_gpu(logits), on_gpu(torch.tensor(temperatures)), on_gpu(torch.tensor(top_ps)), on_gpu(torch.tensor(uniforms))).cpu().tolist()
+        want = [plain.sample(logits[row], temperatures[row], top_ps[row], uniforms[row]) for row in range(rows)]
+        assert got == want, (draw, [(row, a, b) for row, (a, b) in enumerate(zip(got, want)) if a != b])
+        ones = [1.0] * rows
+        got = k.sample(on_gpu(logits), on_gpu(torch.tensor(temperatures)), on_gpu(torch.tensor(ones)), on_gpu(torch.tensor(uniforms)), False).cpu().tolist()
+        want = k.sample(on_gpu(logits), on_gpu(torch.tensor(temperatures)), on_gpu(torch.tensor(ones)), on_gpu(torch.tensor(uniforms))).cpu().tolist()
+        assert got == want
+        assert got == [plain.sample(logits[row], temperatures[row], 1.0, uniforms[row]) for row in range(rows)]
+
+
 @pytest.mark.parametrize("pairing", ["adjacent", "half", "none"])
 @pytest.mark.parametrize("heads,kv_heads,dim,page", [(12, 2, 128, 16), (6, 1, 64, 8), (5, 5, 32, 4), (4, 2, 48, 16), (40, 2, 64, 16), (2, 1, 256, 16), (40, 8, 128, 16), (10, 2, 128, 16), (28, 4, 128, 16)])
 def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):

@@ -29,6 +29,9 @@ class TorchKernels:
     def to_device(self, tensor):
         return tensor
 
+    def queued_to_device(self, tensor):
+        return tensor
+
     def embedding(self, table, token_ids):
         return table[token_ids.long()].float()
 
@@ -122,7 +125,7 @@ class TorchKernels:
     def argmax(self, logits):
         return torch.argmax(logits, dim=-1).to(torch.int32)
 
-    def sample(self, logits, temperatures, top_ps, uniforms):
+    def sample(self, logits, temperatures, top_ps, uniforms, with_top_p=True):
         chosen = []
         for row in range(logits.shape[0]):
             temperature, top_p, u = float(temperatures[row]), float(top_ps[row]), float(uniforms[row])
