@@ -311,16 +311,19 @@ __device__ __forceinline__ void stream_wait_loads() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int WAVES, int NT, int G, typename TO, bool GATED>
+// MT: 16-row tiles of x (up to 16 MT rows).  A stage then holds MT chunks of x beside the NT of the
+// weights for every step, and each weight operand meets MT operands of x.
+template <int WAVES, int NT, int MT, int G, typename TO, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x,
                                                                  const bf16_t* __restrict__ w,
                                                                  const void* __restrict__ bias, int bias_is_float,
                                                                  TO* __restrict__ out, int M, int N, int K,
                                                                  int k_split) {
   extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];
-  constexpr int OPERANDS = (NT + 1) * G;                 // of one group: the weight tiles' steps, then x's
+  constexpr int OPERANDS = (NT + MT) * G;                // of one group: the weight tiles' steps, then x's
   constexpr int STAGE_BYTES = OPERANDS * STREAM_CHUNK;
   constexpr int WAVE_BYTES = STREAM_STAGES * STAGE_BYTES;
+  constexpr int TILES = NT * MT;                         // of the result
   static_assert(OPERANDS <= 31, "a group's loads are counted in vmcnt beside a second group's");
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
@@ -332,17 +335,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
   for (int s = 0; s < NT; ++s)
     w_src[s] = w + (size_t)min(((int)blockIdx.x * NT + s) * 16 + load_row, N - 1) * K + k_first + load_piece * 8;
   // rows of x beyond M are read as row M - 1: their columns of the result are dropped at the end
-  const bf16_t* x_src = x + (size_t)min(load_row, M - 1) * K + k_first + load_piece * 8;
+  const bf16_t* x_src[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) x_src[t] = x + (size_t)min(t * 16 + load_row, M - 1) * K + k_first + load_piece * 8;
   unsigned char* mine = stream_lds + (size_t)wave * WAVE_BYTES;
   const unsigned read_at = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)mine +
                            (unsigned)(4 * r + (g ^ ((r >> 1) & 3))) * 16;
 
-  // the bias of the four outputs this lane will finish (wave s finishes tile s) is asked for now
+  // the bias of the four outputs this lane will finish first (wave v finishes tile v, of weight tile
+  // v / MT) is asked for now
   float bias_here[4] = {0.f, 0.f, 0.f, 0.f};
-  if (bias && blockIdx.y == 0 && wave < NT) {
+  if (bias && blockIdx.y == 0 && wave < TILES) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      bias_here[i] = load_as_float(bias, bias_is_float, min(((int)blockIdx.x * NT + wave) * 16 + g * 4 + i, N - 1));
+      bias_here[i] =
+          load_as_float(bias, bias_is_float, min(((int)blockIdx.x * NT + wave / MT) * 16 + g * 4 + i, N - 1));
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // so that the counts below count the stream alone
 
@@ -356,15 +363,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(w_src[s] + k + u * STEP),
                                          (void __attribute__((address_space(3)))*)(to + (s * G + u) * STREAM_CHUNK), 16,
                                          0, 0);
-      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(x_src + k + u * STEP),
-                                       (void __attribute__((address_space(3)))*)(to + (NT * G + u) * STREAM_CHUNK), 16, 0,
-                                       0);
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(x_src[t] + k + u * STEP),
+                                         (void __attribute__((address_space(3)))*)(to + ((NT + t) * G + u) * STREAM_CHUNK),
+                                         16, 0, 0);
     }
   };
 
-  f32x4 acc[NT];
+  f32x4 acc[NT][MT];
 #pragma unroll
-  for (int s = 0; s < NT; ++s) acc[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < NT; ++s)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[s][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const int groups = k_split / (STEP * G);
   int group = wave;
   if (group < groups) request(group, 0);
@@ -383,54 +394,67 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
     for (int u = 0; u < G; ++u)
 #pragma unroll
       for (int s = 0; s < NT; ++s)
-        acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(operands[s * G + u], operands[NT * G + u], acc[s], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(operands[s * G + u], operands[(NT + t) * G + u],
+                                                              acc[s][t], 0, 0, 0);
   }
 
   __syncthreads();  // every wave is done with its stages: LDS is free for the waves' sums
-  float* partial = (float*)stream_lds;  // [WAVES][NT][64 lanes][4]
+  float* partial = (float*)stream_lds;  // [WAVES][TILES][64 lanes][4]
 #pragma unroll
-  for (int s = 0; s < NT; ++s) *(f32x4*)(partial + ((wave * NT + s) * 64 + lane) * 4) = acc[s];
+  for (int s = 0; s < NT; ++s)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) *(f32x4*)(partial + ((wave * TILES + s * MT + t) * 64 + lane) * 4) = acc[s][t];
   __syncthreads();
-  if (wave >= NT) return;
-  const int s = wave;
-  f32x4 total = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int v = 0; v < WAVES; ++v) total += *(const f32x4*)(partial + ((v * NT + s) * 64 + lane) * 4);
-  const int m = r;
-  const int n_first = ((int)blockIdx.x * NT + s) * 16 + g * 4;
-  if (m >= M) return;
+  for (int tile = wave; tile < TILES; tile += WAVES) {
+    const int s = tile / MT;
+    f32x4 total = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int v = 0; v < WAVES; ++v) total += *(const f32x4*)(partial + ((v * TILES + tile) * 64 + lane) * 4);
+    const int m = (tile % MT) * 16 + r;
+    const int n_first = ((int)blockIdx.x * NT + s) * 16 + g * 4;
+    if (m >= M) continue;
+    if (tile == wave) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) total[i] += bias_here[i];
-  if (GATED) {
-    TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+      for (int i = 0; i < 4; ++i) total[i] += bias_here[i];
+    } else if (bias && blockIdx.y == 0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      if (n_first + 2 * i + 1 < N) {
-        const float gate = total[2 * i], up = total[2 * i + 1];
-        dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
-      }
+      for (int i = 0; i < 4; ++i) total[i] += load_as_float(bias, bias_is_float, min(n_first + i, N - 1));
     }
-  } else {
-    TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
+    if (GATED) {
+      TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (n_first + i < N) dst[i] = from_float<TO>(total[i]);
+      for (int i = 0; i < 2; ++i) {
+        if (n_first + 2 * i + 1 < N) {
+          const float gate = total[2 * i], up = total[2 * i + 1];
+          dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+        }
+      }
+    } else {
+      TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n_first + i < N) dst[i] = from_float<TO>(total[i]);
+    }
   }
 }
 
-template <int WAVES, int NT, int G, typename TO, bool GATED>
+template <int WAVES, int NT, int MT, int G, typename TO, bool GATED>
 static int launch_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
                          int K, int splits, hipStream_t stream) {
-  const size_t lds = (size_t)WAVES * STREAM_STAGES * (NT + 1) * G * STREAM_CHUNK;
+  const size_t stages = (size_t)WAVES * STREAM_STAGES * (NT + MT) * G * STREAM_CHUNK;
+  const size_t sums = (size_t)WAVES * NT * MT * 64 * 4 * sizeof(float);
+  const size_t lds = stages > sums ? stages : sums;
   if (lds > 64 * 1024) {
     static bool asked = false;
     if (!asked) {
-      if (hipFuncSetAttribute((const void*)gemm_stream_kernel<WAVES, NT, G, TO, GATED>,
+      if (hipFuncSetAttribute((const void*)gemm_stream_kernel<WAVES, NT, MT, G, TO, GATED>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return ERR_BAD_ARGUMENT;
       asked = true;
     }
   }
-  hipLaunchKernelGGL((gemm_stream_kernel<WAVES, NT, G, TO, GATED>), dim3((N + 16 * NT - 1) / (16 * NT), splits),
+  hipLaunchKernelGGL((gemm_stream_kernel<WAVES, NT, MT, G, TO, GATED>), dim3((N + 16 * NT - 1) / (16 * NT), splits),
                      dim3(WAVES * 64), lds, stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M,
                      N, K, K / splits);
   return LAUNCH_STATUS();
@@ -445,29 +469,63 @@ static int launch_stream(const void* x, const void* w, const void* bias, int bia
 // M <= 16, K / splits a multiple of 128.
 template <typename TO, bool GATED>
 static int pick_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
-                       int splits, hipStream_t stream) {
+                       int splits, hipStream_t stream, int nt = 0, int g = 0) {
   const long tiles = (N + 15) / 16;
+  if (M > 16) {
+    // 17 to 64 rows: two or four tiles of x.  nt, g: 0 = by the sizes, else as asked (measurements)
+    if (nt == 0) nt = tiles * splits >= 2048 ? 2 : 1;
+    if (g == 0) g = 1;
+#define ROWS_CASE(NT_, MT_, G_)                                                                              \
+  if (nt == NT_ && g == G_ && M <= 16 * MT_)                                                                 \
+    return launch_stream<4, NT_, MT_, G_, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+    ROWS_CASE(1, 2, 1)
+    ROWS_CASE(2, 2, 1)
+    ROWS_CASE(1, 2, 2)
+    ROWS_CASE(2, 2, 2)
+    ROWS_CASE(1, 4, 1)
+    ROWS_CASE(2, 4, 1)
+    ROWS_CASE(1, 4, 2)
+    ROWS_CASE(2, 4, 2)
+    ROWS_CASE(4, 2, 1)
+    ROWS_CASE(4, 4, 1)
+#undef ROWS_CASE
+    return ERR_BAD_ARGUMENT;
+  }
   // two tiles a wave for a middling number of weight rows over a K that is not cut (the qkv products of the
   // 7B and 32B sizes: 11.6 -> 10.6 and 20.0 -> 17.5 us); with K cut over workgroups one tile is as good or
   // better (the 32B sizes' o in two parts: 13.5 us against 16.9)
   if (splits == 1 && tiles >= 256 && tiles < 1024 && tiles * K >= 1000000L)
-    return launch_stream<4, 2, 2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
-  return launch_stream<4, 1, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+    return launch_stream<4, 2, 1, 2, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  return launch_stream<4, 1, 1, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
 }
 
-// The same product as llmserve_gemm_skinny, always through gemm_stream (tests and measurements).
-extern "C" int llmserve_gemm_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
-                                    int out_is_float, int gated, int M, int N, int K, int splits,
-                                    hipStream_t stream) {
+// The same product as llmserve_gemm_skinny, always through gemm_stream (tests and measurements); up to 64 rows.
+static int stream_entry(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int out_is_float,
+                        int gated, int M, int N, int K, int splits, hipStream_t stream, int nt, int g) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 16 || K <= 0 || splits < 1 || K % splits || (K / splits) % (STEP * GROUP) || (gated && N % 2))
+  if (M > 64 || K <= 0 || splits < 1 || K % splits || (K / splits) % (STEP * GROUP) || (gated && N % 2))
     return ERR_BAD_ARGUMENT;
   if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
   if (gated)
-    return out_is_float ? pick_stream<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
-                        : pick_stream<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
-  return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
-                      : pick_stream<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
+    return out_is_float ? pick_stream<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt, g)
+                        : pick_stream<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt, g);
+  return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream, nt, g)
+                      : pick_stream<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt, g);
+}
+
+extern "C" int llmserve_gemm_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
+                                    int out_is_float, int gated, int M, int N, int K, int splits,
+                                    hipStream_t stream) {
+  return stream_entry(x, w, bias, bias_is_float, out, out_is_float, gated, M, N, K, splits, stream, 0, 0);
+}
+
+// The same for 17 to 64 rows with the shape asked for (measurements): nt weight tiles a workgroup (1, 2),
+// groups of g steps (1, 2).
+extern "C" int llmserve_gemm_stream_shaped(const void* x, const void* w, const void* bias, int bias_is_float,
+                                           void* out, int out_is_float, int gated, int M, int N, int K, int splits,
+                                           int nt, int g, hipStream_t stream) {
+  if (M <= 16) return ERR_BAD_ARGUMENT;
+  return stream_entry(x, w, bias, bias_is_float, out, out_is_float, gated, M, N, K, splits, stream, nt, g);
 }
 
 // ---------------------------------------------------------------------------- key splits merged on the way in
@@ -1247,6 +1305,15 @@ extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bi
     PAIR_CASE(2)
     PAIR_CASE(4)
 #undef PAIR_CASE
+  }
+  if (M > 16 && !gated && splits == 1 && K % (STEP * GROUP) == 0 && (long)N * K <= (1L << 22)) {
+    // A small weight at 17 to 64 rows: two or four tiles of x beside one weight tile a workgroup, through
+    // LDS.  In a captured chain over different weights, the 1.5B sizes' qkv and o: 4.8 and 4.0 us at 17
+    // rows, 5.0 and 4.5 at 32, 6.0 and 5.6 at 48, 6.7 and 6.2 at 64 (the library 7.1-7.7 throughout, the
+    // kernel below 5.9 and 4.8 at 17 rows, 6.8 and 5.5 at 32).  Larger weights stay with the library.
+    const int g = M <= 32 ? 2 : 1;
+    return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, 1, g)
+                        : pick_stream<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, 1, g);
   }
   if (gated)
     return out_is_float ? pick_waves<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)

@@ -53,6 +53,7 @@ _SIGNATURES = {
     "llmserve_gemm_generic": "pipipipiiiip",
     "llmserve_gemm_skinny": "pppipiiiiiip",
     "llmserve_gemm_stream": "pppipiiiiiip",
+    "llmserve_gemm_stream_shaped": "pppipiiiiiiiip",
     "llmserve_gemm_medium": "pppipiiiiiip",
     "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
@@ -291,9 +292,11 @@ class HipKernels:
             # On the device the library is ahead of "medium" as it stands, so a captured step (which
             # costs the host nothing per launch) takes the library; a step launched kernel by kernel
             # is bound by the host, where a torch call costs four times one of ours.
-            # Except a small weight at up to 32 rows: there the library's fixed cost shows (qkv and o of
-            # the 1.5B sizes in a captured chain: 7.1 us each, against 5.9 and 4.8 at 17 rows, 6.8 and 5.5 at 32).
-            if not gated and rows <= 32 and inner % 32 == 0 and weights.out_features * inner <= (1 << 22):
+            # Except a small weight: there the library's fixed cost shows (qkv and o of the 1.5B sizes in a
+            # captured chain: 7.1-7.7 us each, against 4.8 and 4.0 at 17 rows, 5.0 and 4.5 at 32, 6.7 and 6.2 at
+            # 64 for the kernel that brings two or four tiles of x through LDS beside a weight tile; where K is
+            # no multiple of 128 an older kernel takes up to 32 rows).
+            if not gated and inner % 32 == 0 and weights.out_features * inner <= (1 << 22) and (rows <= 32 or (rows <= 64 and inner % 128 == 0)):
                 return "skinny"
             return None
         if 16 < rows <= 64 and inner % 128 == 0:

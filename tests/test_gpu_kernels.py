@@ -595,15 +595,16 @@ def test_library_products_cut_over_a_long_k(kernels, rows, inner, outer):
     torch.testing.assert_close(normed.cpu().double(), plain.rms_norm(hidden.double() + expected, torch.ones(outer).double(), 1e-6), **TOLERANCE[dtype])
 
 
-@pytest.mark.parametrize("rows", [1, 7, 16])
+@pytest.mark.parametrize("rows", [1, 7, 16, 17, 40, 64])
 @pytest.mark.parametrize("outer,inner,gated,splits,bias", [
     (40, 128, False, 1, None), (1000, 384, False, 1, "bfloat16"), (4610, 3584, False, 1, "float32"),  # two tiles a wave
     (154, 2560, False, 5, None), (318, 256, True, 1, None), (6000, 1536, True, 1, None),
 ])
 def test_products_streamed_through_lds(kernels, rows, outer, inner, gated, splits, bias):
-    """The product for up to 16 rows that brings weights and x through LDS, quad by quad, alone: odd
-    numbers of weight rows (the last tile is cut), one and two tiles a wave, a bias of either type,
-    K cut into partial sums, SiLU(gate) * up over interleaved rows; against the plain product."""
+    """The product for up to 64 rows that brings weights and x through LDS, quad by quad, alone: odd
+    numbers of weight rows (the last tile is cut), one and two tiles a wave, one, two and four tiles of
+    x (the last one cut), a bias of either type, K cut into partial sums, SiLU(gate) * up over
+    interleaved rows; against the plain product."""
     from llmserve_amd.kernels.hip import _check, _pointer
 
     k = kernels[torch.bfloat16]
@@ -627,11 +628,43 @@ def test_products_streamed_through_lds(kernels, rows, outer, inner, gated, split
     got = out.sum(0).cpu().double()
     tolerance = dict(atol=2e-3, rtol=2e-3) if float_out else TOLERANCE[torch.bfloat16]
     torch.testing.assert_close(got, expected, **tolerance)
-    # and it refuses what it cannot take: more than 16 rows, a K that is no multiple of 128
+    # and it refuses what it cannot take: more than 64 rows, a K that is no multiple of 128
     assert k._gemm_bf16.llmserve_gemm_stream(_pointer(device_x), _pointer(device_w), None, 0, _pointer(out), int(float_out),
-                                             0, 17, outer, inner, 1, k._stream) != 0
+                                             0, 65, outer, inner, 1, k._stream) != 0
     assert k._gemm_bf16.llmserve_gemm_stream(_pointer(device_x), _pointer(device_w), None, 0, _pointer(out), int(float_out),
                                              0, rows, outer, inner - 32, 1, k._stream) != 0
+
+
+@pytest.mark.parametrize("rows", [24, 33, 64])
+@pytest.mark.parametrize("tiles,steps", [(1, 1), (1, 2), (2, 1), (2, 2), (4, 1)])
+def test_streamed_products_of_many_rows_in_every_shape(kernels, rows, tiles, steps):
+    """The same kernel at 17 to 64 rows with every shape it is built in (weight tiles a workgroup, steps
+    a group), plain with a bias and gated, and through the entry point that the engine's small products
+    of such steps take."""
+    from llmserve_amd.kernels.hip import _check, _pointer
+
+    k = kernels[torch.bfloat16]
+    outer, inner = 1210, 640
+    x, w, b = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer)
+    device_x, device_w, device_b = on_gpu(x, torch.bfloat16), on_gpu(w, torch.bfloat16), on_gpu(b, torch.bfloat16)
+    expected = rounded(x, torch.bfloat16) @ rounded(w, torch.bfloat16).T
+    for gated in (False, True):
+        want = expected + rounded(b, torch.bfloat16)
+        if gated:
+            want = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
+        out = torch.full((rows, outer // 2 if gated else outer), float("nan"), device="cuda", dtype=torch.bfloat16)
+        status = k._gemm_bf16.llmserve_gemm_stream_shaped(
+            _pointer(device_x), _pointer(device_w), _pointer(device_b), 0, _pointer(out), 0, int(gated), rows, outer,
+            inner, 1, tiles, steps, k._stream,
+        )
+        _check(status, "gemm_stream_shaped")
+        torch.testing.assert_close(out.cpu().double(), want, **TOLERANCE[torch.bfloat16])
+    out = torch.full((rows, outer), float("nan"), device="cuda", dtype=torch.bfloat16)
+    status = k._gemm_bf16.llmserve_gemm_skinny(
+        _pointer(device_x), _pointer(device_w), _pointer(device_b), 0, _pointer(out), 0, 0, rows, outer, inner, 1, k._stream,
+    )
+    _check(status, "gemm_skinny")
+    torch.testing.assert_close(out.cpu().double(), expected + rounded(b, torch.bfloat16), **TOLERANCE[torch.bfloat16])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
