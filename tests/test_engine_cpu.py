@@ -520,3 +520,27 @@ def test_some_random_workloads_ran_out_of_pages():
     if len(_RANDOM_RUNS) < 12:
         pytest.skip("the random runs did not all run in this process")
     assert sum(1 for evictions in _RANDOM_RUNS.values() if evictions > 0) >= 3, _RANDOM_RUNS
+
+
+def test_the_sampler_says_whether_a_row_has_top_p():
+    """The kernels may leave the top-p stages out when told that no row needs them: the sampler says so
+    only if no row with a temperature has top_p < 1 (a greedy row's top_p does not count)."""
+    from llmserve_amd.sampling.sampler import GenerationConfig, Sampler
+
+    class Recording(TorchKernels):
+        def sample(self, logits, temperatures, top_ps, uniforms, with_top_p=True):
+            self.said = with_top_p
+            return super().sample(logits, temperatures, top_ps, uniforms, with_top_p)
+
+    kernels = Recording(torch.float32)
+    sampler = Sampler(kernels)
+    logits = torch.randn(3, 50)
+    cases = [
+        ([GenerationConfig(4, 0.7, 1.0), GenerationConfig(4, 0.0, 0.5), GenerationConfig(4, 1.2, 1.0)], False),
+        ([GenerationConfig(4, 0.7, 1.0), GenerationConfig(4, 0.0, 1.0), GenerationConfig(4, 1.2, 0.9)], True),
+    ]
+    for configs, expected in cases:
+        tokens = sampler.sample(logits, configs, [0, 1, 2])
+        assert kernels.said is expected
+        want = [plain.sample(logits[row], c.temperature, c.top_p, plain.uniform_for(c.seed, row)) for row, c in enumerate(configs)]
+        assert tokens == want
