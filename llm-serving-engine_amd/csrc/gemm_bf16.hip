@@ -1306,13 +1306,15 @@ extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bi
     PAIR_CASE(4)
 #undef PAIR_CASE
   }
-  if (M > 16 && !gated && splits == 1 && K % (STEP * GROUP) == 0 && (long)N * K <= (1L << 22)) {
+  if (M > 16 && !gated && K % splits == 0 && (K / splits) % (STEP * GROUP) == 0 && (long)N * K <= (1L << 22)) {
     // A small weight at 17 to 64 rows: two or four tiles of x beside one weight tile a workgroup, through
     // LDS.  In a captured chain over different weights, the 1.5B sizes' qkv and o: 4.8 and 4.0 us at 17
     // rows, 5.0 and 4.5 at 32, 6.0 and 5.6 at 48, 6.7 and 6.2 at 64 (the library 7.1-7.7 throughout, the
     // kernel below 5.9 and 4.8 at 17 rows, 6.8 and 5.5 at 32).  Larger weights stay with the library.
-    const int g = M <= 32 ? 2 : 1;
-    return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, 1, g)
+    // With K cut in two (float32 partial sums) o takes 3.5 us at 17 rows, 3.7 at 32, 4.6 at 64 (the kernel
+    // below, in three parts: 4.9, 5.6, 8.0).
+    const int g = M <= 32 && splits == 1 ? 2 : 1;
+    return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream, 1, g)
                         : pick_stream<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, 1, g);
   }
   if (gated)

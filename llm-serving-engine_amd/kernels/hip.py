@@ -444,6 +444,8 @@ class HipKernels:
                     splits = self._tiled_splits(rows, weights.out_features, inner)
                 elif streaming == "medium":
                     splits = self._medium_splits(weights.out_features, inner)
+                elif rows > 16 and weights.out_features * inner <= (1 << 22) and inner % 256 == 0:
+                    splits = 2  # what the kernel for a small weight at 17 to 64 rows does best with
                 else:
                     splits = self._partial_splits(weights.out_features, inner)
             shape = (rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features)

@@ -665,6 +665,14 @@ def test_streamed_products_of_many_rows_in_every_shape(kernels, rows, tiles, ste
     )
     _check(status, "gemm_skinny")
     torch.testing.assert_close(out.cpu().double(), expected + rounded(b, torch.bfloat16), **TOLERANCE[torch.bfloat16])
+    # and with K cut into partial sums (what the output projection of such a step asks for)
+    for splits in (2, 5):
+        parts = torch.full((splits, rows, outer), float("nan"), device="cuda", dtype=torch.float32)
+        status = k._gemm_bf16.llmserve_gemm_skinny(
+            _pointer(device_x), _pointer(device_w), None, 0, _pointer(parts), 1, 0, rows, outer, inner, splits, k._stream,
+        )
+        _check(status, "gemm_skinny in parts")
+        torch.testing.assert_close(parts.sum(0).cpu().double(), expected, atol=2e-3, rtol=2e-3)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
