@@ -422,6 +422,25 @@ def test_sampling_edges(kernels):
         assert got == want, (u, got, want)
 
 
+def test_sampling_refuses_a_workspace_that_is_too_small(kernels):
+    from llmserve_amd.kernels.hip import _pointer
+
+    k = kernels[torch.float32]
+    library = k._sampling_library()
+    rows, vocab = 5, 1000
+    kib = library.llmserve_sample_workspace_kib(rows, vocab)
+    assert kib > rows * vocab * 4 // 1024 and library.llmserve_sample_workspace_kib(0, vocab) < 0
+    logits, values, out = torch.randn(rows, vocab).cuda(), torch.full((rows,), 0.5).cuda(), torch.zeros(rows, dtype=torch.int32).cuda()
+    workspace = torch.empty(kib * 1024, dtype=torch.uint8, device="cuda")
+    arguments = lambda space, size: (_pointer(logits), _pointer(values), _pointer(values), _pointer(values), space, size, _pointer(out), rows, vocab, 1, k._stream)
+    assert library.llmserve_sample(*arguments(_pointer(workspace), kib - 1)) == 1001
+    assert library.llmserve_sample(*arguments(None, kib)) == 1001
+    assert library.llmserve_sample(*arguments(_pointer(workspace) + 16, kib)) == 1001  # not aligned to 256 bytes
+    assert library.llmserve_sample(*arguments(_pointer(workspace), kib)) == 0
+    torch.cuda.synchronize()
+    assert all(0 <= token < vocab for token in out.cpu().tolist())
+
+
 @pytest.mark.parametrize("rows,vocab", [(70, 1025), (300, 130), (3, 40000)])
 def test_sampling_of_many_rows_and_hard_rows(kernels, rows, vocab):
     """The stages cut a row into fewer pieces when there are many rows; rows whose entries are all
