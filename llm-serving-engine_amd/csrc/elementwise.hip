@@ -272,57 +272,91 @@ __global__ __launch_bounds__(256) void rotate_and_store_vector_kernel(
     bf16_t* __restrict__ qkv, const float2* __restrict__ table, int pairing, int heads, int kv_heads, int dim,
     bf16_t* __restrict__ keys, bf16_t* __restrict__ values, const int* __restrict__ slots, int page_size, int tokens) {
   typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+  typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
   const int per_head = dim / 16, half = dim / 2;
-  const int rotated = (heads + kv_heads) * per_head, pieces = rotated + kv_heads * (dim / 8);
-  const size_t id = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const int token = (int)(id / pieces), piece = (int)(id % pieces);
-  if (token >= tokens) return;
-  bf16_t* row = qkv + (size_t)token * (heads + 2 * kv_heads) * dim;
-  const int slot = slots ? slots[token] : -1;
-  if (piece < rotated) {
-    const int head = piece / per_head, p = piece % per_head;
-    bf16_t* h = row + head * dim;
-    const int ia = pairing == 2 ? 8 * p : 16 * p, ib = pairing == 2 ? 8 * p + half : 16 * p + 8;
-    bf16x8 a = *(const bf16x8*)(h + ia), b = *(const bf16x8*)(h + ib);
-    if (pairing != 0) {
-      float2 cs[8];
-      const float2* angles = table + (size_t)token * half + 8 * p;
+  const int rotated = (heads + kv_heads) * per_head;
+  const size_t id = (size_t)blockIdx.x * 256 + threadIdx.x, rotating = (size_t)tokens * rotated;
+  const int row_width = (heads + 2 * kv_heads) * dim;
+  if (id >= rotating) {
+    // The values.  A page keeps them transposed (attention sums over keys), so a token's value row is
+    // `dim` two-byte stores far apart.  A thread therefore takes four dims of eight tokens in a row: its
+    // loads are 8 bytes beside its neighbours', and where the eight tokens lie side by side in a page
+    // (a prompt's portion) it stores 16 bytes a dim.
+    if (slots == nullptr) return;
+    const int quads = dim / 4;
+    const size_t unit = id - rotating;
+    const int quad = (int)(unit % quads), head = (int)(unit / quads % kv_heads);
+    const size_t octet = unit / quads / kv_heads;
+    if (octet * 8 >= (size_t)tokens) return;
+    const int first = (int)octet * 8, count = min(8, tokens - first);
+    int slot[8];
+    bf16x4 v[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) cs[i] = angles[i];
-      if (pairing == 2) {
+    for (int i = 0; i < 8; ++i) {
+      const int token = first + min(i, count - 1);
+      slot[i] = i < count ? slots[token] : -1;
+      v[i] = *(const bf16x4*)(qkv + (size_t)token * row_width + (size_t)(heads + kv_heads + head) * dim + quad * 4);
+    }
+    bool together = count == 8 && slot[0] >= 0 && slot[0] % 8 == 0 && page_size % 8 == 0;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float x = (float)a[i], y = (float)b[i];
-          a[i] = (bf16_t)(x * cs[i].x - y * cs[i].y);
-          b[i] = (bf16_t)(y * cs[i].x + x * cs[i].y);
-        }
-      } else {
+    for (int i = 1; i < 8; ++i) together = together && slot[i] == slot[0] + i;
+    if (together) {
+      bf16_t* v_page = values + ((size_t)(slot[0] / page_size) * kv_heads + head) * page_size * dim + slot[0] % page_size;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float x = (float)a[2 * i], y = (float)a[2 * i + 1];
-          a[2 * i] = (bf16_t)(x * cs[i].x - y * cs[i].y);
-          a[2 * i + 1] = (bf16_t)(y * cs[i].x + x * cs[i].y);
-          const float u = (float)b[2 * i], v = (float)b[2 * i + 1];
-          b[2 * i] = (bf16_t)(u * cs[4 + i].x - v * cs[4 + i].y);
-          b[2 * i + 1] = (bf16_t)(v * cs[4 + i].x + u * cs[4 + i].y);
-        }
+      for (int e = 0; e < 4; ++e) {
+        const bf16x8 run = {v[0][e], v[1][e], v[2][e], v[3][e], v[4][e], v[5][e], v[6][e], v[7][e]};
+        *(bf16x8*)(v_page + (size_t)(quad * 4 + e) * page_size) = run;
       }
-      *(bf16x8*)(h + ia) = a;
-      *(bf16x8*)(h + ib) = b;
-    }
-    if (head >= heads && slot >= 0) {
-      // pieces ia / 8 and ib / 8 of the key at this slot (dim is a multiple of 16 here)
-      bf16_t* k_block = keys + ((size_t)(slot / page_size) * kv_heads + (head - heads)) * page_size * dim;
-      const int offset = slot % page_size;
-      *(bf16x8*)(k_block + ((size_t)(ia / KEY_PIECE) * page_size + offset) * KEY_PIECE) = a;
-      *(bf16x8*)(k_block + ((size_t)(ib / KEY_PIECE) * page_size + offset) * KEY_PIECE) = b;
-    }
-  } else if (slot >= 0) {
-    const int at = piece - rotated, head = at / (dim / 8), d0 = (at % (dim / 8)) * 8;
-    const bf16x8 v = *(const bf16x8*)(row + (size_t)(heads + kv_heads + head) * dim + d0);
-    bf16_t* v_page = values + ((size_t)(slot / page_size) * kv_heads + head) * page_size * dim + slot % page_size;
+    } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v_page[(size_t)(d0 + e) * page_size] = v[e];
+      for (int i = 0; i < 8; ++i) {
+        if (slot[i] < 0) continue;
+        bf16_t* v_page = values + ((size_t)(slot[i] / page_size) * kv_heads + head) * page_size * dim + slot[i] % page_size;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v_page[(size_t)(quad * 4 + e) * page_size] = v[i][e];
+      }
+    }
+    return;
+  }
+  const int token = (int)(id / rotated), piece = (int)(id % rotated);
+  bf16_t* row = qkv + (size_t)token * row_width;
+  const int slot = slots ? slots[token] : -1;
+  const int head = piece / per_head, p = piece % per_head;
+  bf16_t* h = row + head * dim;
+  const int ia = pairing == 2 ? 8 * p : 16 * p, ib = pairing == 2 ? 8 * p + half : 16 * p + 8;
+  bf16x8 a = *(const bf16x8*)(h + ia), b = *(const bf16x8*)(h + ib);
+  if (pairing != 0) {
+    float2 cs[8];
+    const float2* angles = table + (size_t)token * half + 8 * p;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cs[i] = angles[i];
+    if (pairing == 2) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float x = (float)a[i], y = (float)b[i];
+        a[i] = (bf16_t)(x * cs[i].x - y * cs[i].y);
+        b[i] = (bf16_t)(y * cs[i].x + x * cs[i].y);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float x = (float)a[2 * i], y = (float)a[2 * i + 1];
+        a[2 * i] = (bf16_t)(x * cs[i].x - y * cs[i].y);
+        a[2 * i + 1] = (bf16_t)(y * cs[i].x + x * cs[i].y);
+        const float u = (float)b[2 * i], v = (float)b[2 * i + 1];
+        b[2 * i] = (bf16_t)(u * cs[4 + i].x - v * cs[4 + i].y);
+        b[2 * i + 1] = (bf16_t)(v * cs[4 + i].x + u * cs[4 + i].y);
+      }
+    }
+    *(bf16x8*)(h + ia) = a;
+    *(bf16x8*)(h + ib) = b;
+  }
+  if (head >= heads && slot >= 0) {
+    // pieces ia / 8 and ib / 8 of the key at this slot (dim is a multiple of 16 here)
+    bf16_t* k_block = keys + ((size_t)(slot / page_size) * kv_heads + (head - heads)) * page_size * dim;
+    const int offset = slot % page_size;
+    *(bf16x8*)(k_block + ((size_t)(ia / KEY_PIECE) * page_size + offset) * KEY_PIECE) = a;
+    *(bf16x8*)(k_block + ((size_t)(ib / KEY_PIECE) * page_size + offset) * KEY_PIECE) = b;
   }
 }
 
@@ -332,7 +366,9 @@ extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const float* t
   if (tokens <= 0) return 0;
   if (dim % 2 || (pairing != 0 && table == nullptr) || pairing < 0 || pairing > 2) return ERR_BAD_ARGUMENT;
   if (!is_float && dim % 16 == 0) {
-    const size_t threads = (size_t)tokens * ((heads + kv_heads) * (dim / 16) + kv_heads * (dim / 8));
+    // a thread for every 16 elements of a token's q and k heads, then one for every four dims of eight tokens' values
+    const size_t threads = (size_t)tokens * (heads + kv_heads) * (dim / 16) +
+                           (slots ? (size_t)((tokens + 7) / 8) * kv_heads * (dim / 4) : 0);
     hipLaunchKernelGGL(rotate_and_store_vector_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
                        (bf16_t*)qkv, (const float2*)table, pairing, heads, kv_heads, dim, (bf16_t*)keys,
                        (bf16_t*)values, slots, page_size, tokens);
