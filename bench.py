@@ -73,9 +73,23 @@ def main() -> int:
     if not args.skip_points and not args.skip_context_points:
         extra.update({"decode_b8_ctx8k": (8, 8192), "decode_b8_ctx30k": (8, 30000), "decode_b64_ctx4k": (64, 4096)})
     longest = getattr(config, "max_position_embeddings", 32768)
-    extra = {name: shape for name, shape in extra.items() if shape[1] + 300 <= longest}
+    steps = min(args.steps, 250 - args.warmup)
+
+    def budget(batch: int) -> int:
+        return max(2048, batch)  # tokens a step
+
+    def output_tokens(batch: int, prompt: int) -> int:
+        """How many tokens a request of a decode measurement may generate.  Prompts come in portions under
+        the step's token budget, so the requests finish their prompts in different steps and those that
+        finish first decode meanwhile: with this many tokens none of them ends before the timed steps do."""
+        steps_of_prompts = -(-batch * prompt // budget(batch)) + batch
+        return steps_of_prompts + args.warmup + steps + 1
+
+    extra = {name: shape for name, shape in extra.items() if shape[1] + output_tokens(*shape) <= longest}
     most = max(batch for batch, _ in [headline, *extra.values()])
-    pages = max(batch * (-(-(prompt + 256 + page) // page)) for batch, prompt in [headline, *extra.values()])
+    pages = max(
+        batch * (-(-(prompt + output_tokens(batch, prompt) + page) // page)) for batch, prompt in [headline, *extra.values()]
+    )
     pages += args.prefill_len // page + 8
     runner = ModelRunner(loaded, kernels, CacheConfig(block_size=page, num_blocks=pages, max_sequences=most + 1))
     # What a decode step has to read: every weight it uses once (of an untied embedding table only the
@@ -94,9 +108,11 @@ def main() -> int:
         return torch.randint(4, spec.vocab_size, (count,), generator=generator).tolist()
 
     def decode(batch: int, prompt_len: int, steps: int, warmup: int) -> dict:
-        """`steps` timed decode steps of `batch` requests after prompts of `prompt_len` tokens."""
-        core = EngineCore(runner, SchedulerConfig(batch, max(2048, batch)), prefill_chunk_size=min(2048, prompt_len))
-        settings = GenerationConfig(max_new_tokens=warmup + steps + 1)
+        """`steps` timed decode steps of `batch` requests after prompts of `prompt_len` tokens.  Every timed
+        step decodes one token of every request (checked): a request that finished its prompt earlier than
+        the others is further on by then, and the context is the mean over requests and timed steps."""
+        core = EngineCore(runner, SchedulerConfig(batch, budget(batch)), prefill_chunk_size=min(2048, prompt_len))
+        settings = GenerationConfig(max_new_tokens=output_tokens(batch, prompt_len))
         requests = [Request(f"b{batch}-{prompt_len}-{index}", tokens(prompt_len), settings) for index in range(batch)]
         for request in requests:
             core.submit(request)
@@ -104,16 +120,20 @@ def main() -> int:
             core.step()
         for _ in range(warmup):
             core.step()
+        before = [len(request.output) for request in requests]
         torch.cuda.synchronize()
         started = time.perf_counter()
         for _ in range(steps):
-            core.step()
+            produced = core.step()
+            if len(produced) != batch:
+                raise RuntimeError(f"a timed step decoded {len(produced)} tokens, not one of each of the {batch} requests")
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
-        assert all(len(request.output) == 1 + warmup + steps for request in requests)
+        assert all(len(request.output) == had + steps and not request.done for request, had in zip(requests, before))
         for request in requests:
             core.finish(request)
-        context = prompt_len + 1 + warmup + (steps - 1) / 2.0  # mean context length during the timed steps
+        # keys a request's token sees in timed step j: its prompt, what it had generated before, and j
+        context = prompt_len + sum(before) / batch + (steps - 1) / 2.0
         step_bytes = weight_bytes + batch * embedding_row_bytes + batch * context * kv_bytes_per_token
         seconds = elapsed / steps
         return {
@@ -121,7 +141,7 @@ def main() -> int:
             "ms_per_step": 1000 * seconds,
             "context": context,
             "achieved_gbs": step_bytes / seconds / 1e9,
-            "generated": 1 + warmup + steps,
+            "generated": settings.max_new_tokens,
         }
 
     def prefill(length: int, repeats: int = 5) -> float:
@@ -136,7 +156,6 @@ def main() -> int:
             runner.end_request(f"p{repeat}")
         return statistics.median(times[1:])
 
-    steps = min(args.steps, 250 - args.warmup)
     main_run = decode(*headline, steps, args.warmup)
 
     prefill_seconds = prefill(args.prefill_len)

@@ -550,6 +550,43 @@ def test_fused_decode_attention_over_long_contexts(kernels, requests):
             torch.testing.assert_close(got[head], rounded(v, dtype)[far, head // 6], atol=0.05, rtol=0.05)
 
 
+def test_fused_decode_attention_over_tens_of_thousands_of_keys(kernels):
+    """Beyond 8,192 keys a decode step cuts the keys into more parts than the output projection merges
+    (nine to sixty-four) and a kernel of its own merges them.  Two requests of 30,000 and 9,000 keys, a
+    far key planted to dominate heads 0 and 6 of each (deep inside the long one, near the start of the
+    other): the value stored there must come out, and every head must agree with plain attention of the
+    last token over all keys."""
+    dtype, heads, kv_heads, dim, page = torch.bfloat16, 12, 2, 128, 16
+    lengths, counts, places = [30000, 9000] + [30000 - 100 * i for i in range(6)], [1] * 8, [23456, 100] + [29000 - 4000 * i for i in range(6)]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=30)
+    for (q, k, v), far in zip(per_request, places):
+        k[far] = 3.0 * q[-1, ::6]
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None, "none", 1.0, None).cpu().double()
+    for index, ((q, k, v), far) in enumerate(zip(per_request, places)):
+        last = rounded(q, dtype)[-1]  # [heads, dim]
+        all_keys = rounded(k, dtype).repeat_interleave(heads // kv_heads, dim=1)  # [T, heads, dim]
+        all_values = rounded(v, dtype).repeat_interleave(heads // kv_heads, dim=1)
+        weights = torch.softmax(torch.einsum("hd,thd->ht", last, all_keys), dim=-1)
+        want = torch.einsum("ht,thd->hd", weights, all_values)
+        got = out[index].view(heads, dim)
+        torch.testing.assert_close(got, want, **TOLERANCE[dtype])
+        for head in (0, 6):
+            torch.testing.assert_close(got[head], rounded(v, dtype)[far, head // 6], atol=0.05, rtol=0.05)
+    # Keys of zero: every key weighs the same and the result is the mean of all values, which the
+    # kernel's arithmetic gives almost exactly (weights of 1, sums in float32), so that thirty-two keys
+    # left out anywhere would show (a value is of order one, the mean of 30,000 of order 0.006).
+    for q, k, v in per_request:
+        k.zero_()
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None, "none", 1.0, None).cpu().double()
+    for index, (q, k, v) in enumerate(per_request):
+        want = rounded(v, dtype).mean(0).repeat_interleave(heads // kv_heads, dim=0)  # [heads, dim]
+        torch.testing.assert_close(out[index].view(heads, dim), want, atol=6e-5, rtol=5e-3)
+
+
 @pytest.mark.parametrize("heads,kv_heads,outer,requests", [(12, 2, 1536, 8), (40, 8, 272, 16), (28, 4, 1000, 3), (2, 1, 100, 1)])
 def test_decode_attention_whose_key_splits_the_output_projection_merges(kernels, heads, kv_heads, outer, requests):
     """A step of up to 16 single tokens at head size 128 followed by the output projection: the attention
