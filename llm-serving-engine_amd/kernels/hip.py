@@ -683,11 +683,13 @@ class HipKernels:
                     # Attention and product together at 8 rows of the 1.5B sizes, captured, against 15.3 us
                     # unsplit at 530 keys and 22.1 at 1,000: two splits 14.5 and 18.6, four 14.7 and 16.5, eight
                     # 17.0 and 17.8.
-                    # The product takes up to eight splits.  Where the walk is so long that more are wanted
-                    # even at 32 steps a split (beyond 8,192 keys), the kernel that merges is a small share of
-                    # it and that way stays (8 rows of the 1.5B sizes, a whole step: 8,192 keys 2.46 ms with the
-                    # merging kernel, 2.32 with eight splits merged by the product; 30,000 keys 2.62 and 2.92).
-                    if splits <= 8:
+                    # The product takes up to eight splits.  Where the tables reach beyond 4,096 keys the
+                    # kernel that merges (one trip for all splits' maxima and sums) is a small share of the
+                    # walk and that way is taken (8 rows of the 1.5B sizes, a whole step, product against
+                    # kernel: 2,048 keys in tables of 4,096 1.54 and 1.58 ms; 4,096 keys in tables of 8,192
+                    # 1.65 and 1.62; 6,000 keys 1.73 and 1.71; 8,192 keys 1.83 and 1.76; 30,000 keys 2.76 and
+                    # 2.71; 16 rows over 4,096 keys 1.93 and 1.88, one row 1.49 and 1.46).
+                    if splits <= 4:
                         wanted = min(-(-steps // 8), max(1, 1024 // blocks), 8)
                         splits = next(allowed for allowed in (1, 2, 3, 4, 6, 8) if allowed >= wanted)
                     else:

@@ -551,8 +551,8 @@ def test_fused_decode_attention_over_long_contexts(kernels, requests):
 
 
 def test_fused_decode_attention_over_tens_of_thousands_of_keys(kernels):
-    """Beyond 8,192 keys a decode step cuts the keys into more parts than the output projection merges
-    (nine to sixty-four) and a kernel of its own merges them.  Two requests of 30,000 and 9,000 keys, a
+    """Beyond 4,096 keys a decode step cuts the keys into five to sixty-four parts and a kernel of its own
+    merges them (up to there, at up to 16 rows, the output projection does).  Two requests of 30,000 and 9,000 keys, a
     far key planted to dominate heads 0 and 6 of each (deep inside the long one, near the start of the
     other): the value stored there must come out, and every head must agree with plain attention of the
     last token over all keys."""
