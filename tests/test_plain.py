@@ -243,3 +243,35 @@ def test_the_bfloat16_bounds_can_see_a_wrong_rotation_and_a_lost_bias(model_fold
         without = {key: torch.zeros_like(value) if key.endswith("k_proj.bias") else value for key, value in weights.items()}
         lost = torch.cat([plain.forward(without, config, prompt) for prompt in prompts])
         assert float((lost - right).abs().max()) < BF16_LARGEST * float(right.std())
+
+
+def test_the_token_by_token_check_of_a_reduced_precision_run(model_folders):
+    """`unjustified_tokens` is what the GPU tests hold bfloat16 generation against.  It must pass the plain
+    decoder's own tokens even with no allowance at all (greedy, sampled, top-p, stop tokens), and it must see a
+    run whose tokens were drawn with another seed, with the draws of another step, or that went on after a
+    stop token, at the allowance the GPU tests use."""
+    from llmserve_amd import GenerationConfig
+    from tests.tiny import random_tokens, unjustified_tokens
+
+    config, weights = _tiny("B-loud", model_folders)
+    prompt = random_tokens(23, config.vocab_size, seed=3)
+    for chosen in (GenerationConfig(10), GenerationConfig(10, 0.8, 1.0, seed=5), GenerationConfig(10, 0.9, 0.85, seed=6)):
+        own = plain.generate(weights, config, prompt, 10, chosen.temperature, chosen.top_p, chosen.seed)
+        assert not unjustified_tokens(plain, weights, config, prompt, own, chosen, largest=1e-9)
+        assert not unjustified_tokens(plain, weights, config, prompt, own, chosen)
+        if chosen.temperature > 0:  # tokens drawn with another seed are not this request's
+            other = plain.generate(weights, config, prompt, 10, chosen.temperature, chosen.top_p, chosen.seed + 1)
+            assert other != own and unjustified_tokens(plain, weights, config, prompt, other, chosen)
+            shifted = GenerationConfig(10, chosen.temperature, chosen.top_p, seed=chosen.seed)
+            late = own[1:]  # every token one draw too early
+            assert unjustified_tokens(plain, weights, config, prompt, late + own[:1], shifted)
+        else:
+            wrong = list(own)
+            wrong[4] = (own[4] + 1) % config.vocab_size
+            assert [index for index, _, _ in unjustified_tokens(plain, weights, config, prompt, wrong, chosen)][0] == 4
+    own = plain.generate(weights, config, prompt, 10)
+    stopping = GenerationConfig(10, stop_token_ids=(own[3],))
+    first = own.index(own[3])
+    assert not unjustified_tokens(plain, weights, config, prompt, own[: first + 1], stopping)
+    assert unjustified_tokens(plain, weights, config, prompt, own[: first + 2], stopping)  # went on after the stop token
+    assert unjustified_tokens(plain, weights, config, prompt, own[:first], stopping)  # ended early without one

@@ -180,6 +180,59 @@ def unjustified_greedy_tokens(plain, weights, config, prompt: list[int], generat
     return bad
 
 
+def _mass_bounds(mass: float, stretch: float) -> tuple[float, float]:
+    """What the summed probability of a fixed set of tokens can become when every normalised probability moves
+    by a factor between 1 / stretch and stretch (the set's complement moves the same way)."""
+    low = max(mass / stretch, 1.0 - (1.0 - mass) * stretch, 0.0)
+    high = min(mass * stretch, 1.0 - (1.0 - mass) / stretch, 1.0)
+    return low, high
+
+
+def unjustified_tokens(plain, weights, config, prompt: list[int], generated: list[int], settings, largest: float = BF16_LARGEST):
+    """Checks the tokens of a reduced-precision run one by one against the plain implementation fed the run's
+    own prefix.  A greedy token must be the best or within rounding of it (`unjustified_greedy_tokens`).  A
+    sampled token must be one that the plain sampler's rule could give at the request's own draw u =
+    uniform_for(seed, j) once every logit may be off by `largest` of the spread: every probability then moves
+    by a factor of at most exp(2 * that / temperature), and u (times the kept mass, for top-p) must fall into
+    the token's interval of the cumulated probabilities widened by that much; under top-p the token must also
+    be one that can be kept, and tokens whose probabilities are within the factor of the chosen one's may
+    stand before or behind it.  Also: nothing follows a stop token, and a run that ends early ends in one.
+    Returns the offending (index, token, why)."""
+    import math
+
+    bad = []
+    stops = set(settings.stop_token_ids)
+    if len(generated) > settings.max_new_tokens or (len(generated) < settings.max_new_tokens and (not generated or generated[-1] not in stops)):
+        bad.append((len(generated), None, "wrong number of tokens"))
+    for index, token in enumerate(generated):
+        if index < len(generated) - 1 and token in stops:
+            bad.append((index, token, "a stop token is not the last"))
+        logits = plain.forward(weights, config, list(prompt) + list(generated[:index]))[-1].double()
+        off = largest * float(logits.std())
+        if settings.temperature <= 0:
+            if float(logits.max() - logits[token]) > 2 * off:
+                bad.append((index, token, f"{float(logits.max() - logits[token]):.4f} below the best, {2 * off:.4f} allowed"))
+            continue
+        u = plain.uniform_for(settings.seed, index)
+        p = torch.softmax(logits / settings.temperature, dim=-1)
+        stretch = math.exp(2 * off / settings.temperature)
+        if settings.top_p >= 1.0:
+            before, upto = float(p[:token].sum()), float(p[: token + 1].sum())
+            kept_low = kept_high = 1.0
+        else:
+            mine = float(p[token])
+            before = float(p[p > mine * stretch * stretch].sum())  # certainly in front of it in descending order
+            upto = float(p[p >= mine / (stretch * stretch)].sum())  # in front of it at most, itself included
+            kept_low, kept_high = settings.top_p, min(1.0, settings.top_p + float(p.max()) * stretch)
+            if _mass_bounds(before, stretch)[0] >= settings.top_p:
+                bad.append((index, token, f"cannot be kept: mass {before:.4f} lies in front of it, top_p {settings.top_p}"))
+                continue
+        lowest, highest = _mass_bounds(before, stretch)[0], _mass_bounds(upto, stretch)[1]
+        if not (lowest <= u * kept_high and u * kept_low < highest):
+            bad.append((index, token, f"draw {u:.4f} (kept mass {kept_low:.3f}-{kept_high:.3f}) outside [{lowest:.4f}, {highest:.4f})"))
+    return bad
+
+
 def random_tokens(count: int, vocab: int, seed: int) -> list[int]:
     generator = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (count,), generator=generator).tolist()
