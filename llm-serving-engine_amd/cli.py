@@ -115,7 +115,6 @@ async def _benchmark(args) -> None:
     report.cache = engine.cache_stats
     report.metadata["engine"] = engine.iteration_stats
     await engine.close()
-    engine.runner.close()
     output = Path(args.output)
     output.parent.mkdir(parents=True, exist_ok=True)
     report.write_json(output)
@@ -129,10 +128,16 @@ async def _generate(args) -> None:
     loaded, tokenizer = _load_runtime(args)
     engine = _engine(args, loaded, tokenizer, batch_size=1, mode="continuous")
     prompt = [int(t) for t in args.prompt_tokens.split(",")] if args.prompt_tokens else args.prompt
-    settings = GenerationConfig(args.max_tokens, args.temperature, args.top_p, args.seed, tuple(args.stop_token_id or ()))
+    stops = tuple(args.stop_token_id or ())
+    if not stops and args.model and not args.ignore_eos:
+        # as the reference's service does (`service/app.py:88`): generation ends at the model's own
+        # end-of-sequence token unless the caller says where it ends
+        from .engine.tokenizer import folder_eos_token_ids
+
+        stops = folder_eos_token_ids(args.model)
+    settings = GenerationConfig(args.max_tokens, args.temperature, args.top_p, args.seed, stops)
     tokens = await engine.generate(prompt, settings)
     await engine.close()
-    engine.runner.close()
     print(json.dumps({"token_ids": tokens, "text": tokenizer.decode(tokens)}))
 
 
@@ -140,7 +145,8 @@ def _replay(args) -> int:
     import subprocess
 
     command = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", args.model, "--dtype", args.dtype, "--out",
-               args.out, "--max-tokens", str(args.max_tokens), "--block-size", str(args.block_size)]
+               args.out, "--max-tokens", str(args.max_tokens), "--block-size", str(args.block_size),
+               "--max-requests", str(args.max_requests)]
     return subprocess.call(command)
 
 
@@ -188,7 +194,9 @@ def build_parser() -> argparse.ArgumentParser:
     generate.add_argument("--max-tokens", type=int, default=32)
     generate.add_argument("--temperature", type=float, default=0.0)
     generate.add_argument("--top-p", type=float, default=1.0)
-    generate.add_argument("--stop-token-id", type=int, action="append")
+    generate.add_argument("--stop-token-id", type=int, action="append",
+                          help="default: the eos_token_id that the model folder names (generation_config.json, config.json)")
+    generate.add_argument("--ignore-eos", action="store_true", help="run to --max-tokens whatever the model folder names")
     _engine_options(generate)
 
     replay = commands.add_parser("replay", help="feed token ids step by step (stdin) and write logits")
@@ -197,6 +205,7 @@ def build_parser() -> argparse.ArgumentParser:
     replay.add_argument("--out", required=True)
     replay.add_argument("--max-tokens", type=int, required=True)
     replay.add_argument("--block-size", type=int, default=16)
+    replay.add_argument("--max-requests", type=int, default=8, help="most requests alive at a time")
 
     random_model = commands.add_parser("random-model", help="write a model folder with seeded random weights")
     random_model.add_argument("--config", required=True, help="a config.json")

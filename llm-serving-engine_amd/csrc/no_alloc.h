@@ -1,8 +1,9 @@
 // An entry point that allocates nothing.
 //
-// It has no counterpart in the reference, whose sampling goes through torch and allocates freely
-// (engine.py:29-72).  It is for callers that cannot allocate device memory: code under HIP graph
-// capture, tight serving loops, harnesses that forbid hipMalloc.
+// It has no counterpart in the reference.  It is for callers that cannot allocate device memory:
+// code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+// The first call on a device looks up that device's copy of the buffer (hipGetSymbolAddress, under a
+// mutex), which is not a launch: make it outside a capture, any later call is launches only.
 #pragma once
 
 #include <hip/hip_runtime.h>

@@ -364,7 +364,8 @@ class LLMEngine:
         self._wake = asyncio.Event()
         self._server: asyncio.Task | None = None
         self._closed = False
-        self._facts: dict[str, dict[str, float | int | None]] = {}
+        self._facts: dict[str, dict[str, float | int | None]] = {}  # in order of finishing
+        self.facts_kept = 4096
 
     @property
     def scheduler(self) -> Scheduler:
@@ -393,13 +394,14 @@ class LLMEngine:
         request.outcome = asyncio.get_running_loop().create_future()
         self._inbox.append(request)
         self._wake.set()
-        if self._server is None:
+        if self._server is None or self._server.done():  # the first request, or the first after a step failed
             self._server = asyncio.create_task(self._serve())
         return await request.outcome
 
     def request_facts(self, request_id: str) -> dict[str, float | int | None]:
         """What the engine knows about a finished request beside its tokens: when it was first
-        admitted (monotonic seconds), how often it gave way and how many tokens that cost.  Kept until asked for."""
+        admitted (monotonic seconds), how often it gave way and how many tokens that cost.  Kept until
+        asked for, the latest `facts_kept` requests at most."""
         return self._facts.pop(request_id, {})
 
     def _settle(self) -> None:
@@ -410,6 +412,8 @@ class LLMEngine:
                 "preemptions": request.evictions,
                 "recomputed_tokens": request.replayed_tokens,
             }
+            while len(self._facts) > self.facts_kept:  # a caller that never asks does not make it grow
+                del self._facts[next(iter(self._facts))]
             waiter = request.outcome
             if waiter is None or waiter.done():
                 continue
@@ -450,11 +454,13 @@ class LLMEngine:
             self._settle()
 
     async def close(self) -> None:
+        """Stops serving and drops what the runner holds on the device beside the model (captured graphs)."""
         self._closed = True
         server, self._server = self._server, None
         if server is not None:
             server.cancel()
             await asyncio.gather(server, return_exceptions=True)
+        self.runner.close()
 
     @property
     def cache_stats(self) -> dict[str, float]:

@@ -377,6 +377,12 @@ class ModelRunner:
         scope = getattr(self.kernels, "stream_scope", None)
         return scope() if scope is not None else contextlib.nullcontext()
 
+    def _replay_scope(self):
+        """Tells the kernel library that the step it is about to launch is one a graph will replay (its
+        warm-up run and the captured run alike, so that both take the same routes)."""
+        scope = getattr(self.kernels, "replay_scope", None)
+        return scope() if scope is not None else contextlib.nullcontext()
+
     @torch.inference_mode()
     def forward(self, batch: StepBatch) -> torch.Tensor:
         with self._stream_scope():
@@ -526,13 +532,13 @@ class ModelRunner:
         batch = _view_step(static, sizes, widths, facts, chunks, self.cache.page_size, padded_to=(padded_tokens, requests))
         stream = torch.cuda.Stream(self.device)
         stream.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(stream), self._stream_scope(), self._states_kept():
+        with torch.cuda.stream(stream), self._stream_scope(), self._replay_scope(), self._states_kept():
             self._forward_batch(batch)  # loads libraries, builds the work lists kept on `batch`
         torch.cuda.current_stream(self.device).wait_stream(stream)
         torch.cuda.synchronize(self.device)
         batch.computed.clear()  # what kernels computed from the warm-up's values is recorded anew
         captured = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(captured), self._stream_scope():
+        with torch.cuda.graph(captured), self._stream_scope(), self._replay_scope():
             logits = self._forward_batch(batch)
         host = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         return _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)
@@ -569,13 +575,13 @@ class ModelRunner:
         batch = _view_step(static, sizes, widths, facts, chunks, self.cache.page_size)
         stream = torch.cuda.Stream(self.device)
         stream.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(stream), self._stream_scope(), self._states_kept():
+        with torch.cuda.stream(stream), self._stream_scope(), self._replay_scope(), self._states_kept():
             self.model.forward(batch, self.cells)  # loads libraries, builds the work lists kept on `batch`
         torch.cuda.current_stream(self.device).wait_stream(stream)
         torch.cuda.synchronize(self.device)
         batch.computed.clear()  # what kernels computed from the warm-up's values is recorded anew
         captured = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(captured), self._stream_scope():
+        with torch.cuda.graph(captured), self._stream_scope(), self._replay_scope():
             logits = self.model.forward(batch, self.cells)
         host = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         return _DecodeGraph(requests, width, captured, static, host, [None, None], logits, batch)

@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import json
 from pathlib import Path
 from typing import Protocol
 
@@ -33,9 +34,26 @@ class ByteTokenizer:
         return data.decode("utf-8", errors="replace")
 
 
+def folder_eos_token_ids(folder: str | Path) -> tuple[int, ...]:
+    """The end-of-sequence ids a model folder names: `eos_token_id` (a number or a list) of its
+    generation_config.json, else of its config.json; none if neither file has the key."""
+    for name in ("generation_config.json", "config.json"):
+        path = Path(folder) / name
+        if not path.is_file():
+            continue
+        found = json.loads(path.read_text()).get("eos_token_id")
+        if found is None:
+            continue
+        ids = found if isinstance(found, (list, tuple)) else [found]
+        return tuple(int(token) for token in ids)
+    return ()
+
+
 class FileTokenizer:
     """The tokenizer.json of a model folder, through the `tokenizers` library
-    (the reference goes through `transformers.AutoTokenizer`, `tokenizer.py:32-45`)."""
+    (the reference goes through `transformers.AutoTokenizer`, `tokenizer.py:32-45`).
+    `eos_token_id` is the folder's own (generation_config.json, else config.json) unless
+    one is given; -1 where the folder names none."""
 
     def __init__(self, folder: str | Path, eos_token_id: int | None = None) -> None:
         try:
@@ -47,7 +65,10 @@ class FileTokenizer:
             raise FileNotFoundError(f"no tokenizer.json under {folder}")
         self.inner = Inner.from_file(str(path))
         self.vocab_size = self.inner.get_vocab_size()
-        self.eos_token_id = -1 if eos_token_id is None else int(eos_token_id)
+        if eos_token_id is None:
+            named = folder_eos_token_ids(folder)
+            eos_token_id = named[0] if named else -1
+        self.eos_token_id = int(eos_token_id)
 
     def encode(self, text: str) -> list[int]:
         return list(self.inner.encode(text, add_special_tokens=False).ids)

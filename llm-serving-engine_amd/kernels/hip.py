@@ -15,7 +15,7 @@ from typing import Any
 
 import torch
 
-from .build import load_module
+from .build import _say, load_module
 
 _PAIRINGS = {"none": 0, "adjacent": 1, "half": 2}
 
@@ -146,6 +146,8 @@ class HipKernels:
         self._attention_generic = _declared(load_module("attention_generic"))
         self._gemm_bf16 = _declared(load_module("gemm_bf16")) if dtype == torch.bfloat16 else None
         self._pinned_stream: int | None = None
+        self._for_replay = False  # inside `replay_scope`: the step being launched is one that a graph will replay
+        self._told: set[str] = set()
         if self._gemm_bf16 is not None and library_products:
             # The BLAS library sets itself up at its first product, which it cannot do while a stream is
             # being captured; a step of 17 to 64 rows meets the library only inside a capture.
@@ -175,6 +177,23 @@ class HipKernels:
             yield
         finally:
             self._pinned_stream = previous
+
+    @contextlib.contextmanager
+    def replay_scope(self):
+        """Within the scope the step is launched for a graph: its warm-up run and the run that is captured.
+        Such a step costs the host nothing per launch when it is replayed, so products may go where the
+        device is fastest rather than where a launch is cheapest; both runs take the same routes, so the
+        library meets each of the capture's shapes before the capture begins."""
+        previous, self._for_replay = self._for_replay, True
+        try:
+            yield
+        finally:
+            self._for_replay = previous
+
+    def _tell_once(self, key: str, message: str) -> None:
+        if key not in self._told:
+            self._told.add(key)
+            _say(message)
 
     def to_device(self, tensor: torch.Tensor) -> torch.Tensor:
         return tensor.to(self.device).contiguous()
@@ -288,7 +307,7 @@ class HipKernels:
         rows, inner = x.shape[0], weights.in_features
         if 0 < rows <= 16 and inner % 32 == 0:
             return "skinny"
-        if self.library_products and (rows > 64 or torch.cuda.is_current_stream_capturing()):
+        if self.library_products and (rows > 64 or self._for_replay):
             # On the device the library is ahead of "medium" as it stands, so a captured step (which
             # costs the host nothing per launch) takes the library; a step launched kernel by kernel
             # is bound by the host, where a torch call costs four times one of ours.
@@ -612,6 +631,9 @@ class HipKernels:
         if plain_scores and qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
             self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0))
             return out
+        if qkv.dtype == torch.bfloat16:
+            why = "its scores carry a bias or a soft cap" if not plain_scores else f"head size {dim} and pages of {group.page_size}"
+            self._tell_once(f"generic attention: {why}", f"bfloat16 attention runs on the generic kernel, not on the matrix cores: {why}")
         status = self._attention_generic.llmserve_attention_generic(
             _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
             _pointer(group.block_tables), group.width, _pointer(batch.token_sequence), _pointer(batch.positions),

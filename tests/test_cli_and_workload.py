@@ -138,3 +138,28 @@ def test_workload_groups_arrive_in_order_and_fit_the_context():
         LoadProfile(requests=7, groups=(short, long))
     mix = LoadProfile.from_yaml(ROOT / "configs" / "workload-long-context-mix.yaml")
     assert mix.requests == 64 and [group.requests for group in mix.groups] == [48, 16]
+
+
+def test_the_end_of_sequence_ids_a_model_folder_names(tmp_path):
+    """generation_config.json first (a number or a list), then config.json, else none: what `llmserve generate
+    --model` stops at unless told otherwise (reference service/app.py:88 stops at the tokenizer's id)."""
+    import json
+
+    from llmserve_amd.engine.tokenizer import folder_eos_token_ids
+
+    assert folder_eos_token_ids(tmp_path) == ()
+    (tmp_path / "config.json").write_text(json.dumps({"eos_token_id": 7}))
+    assert folder_eos_token_ids(tmp_path) == (7,)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [11, 12]}))
+    assert folder_eos_token_ids(tmp_path) == (11, 12)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"temperature": 0.7}))
+    assert folder_eos_token_ids(tmp_path) == (7,)
+
+
+def test_replay_and_generate_options():
+    from llmserve_amd.cli import build_parser
+
+    args = build_parser().parse_args(["replay", "--model", "m", "--out", "o", "--max-tokens", "64", "--max-requests", "3"])
+    assert args.max_requests == 3
+    args = build_parser().parse_args(["generate", "--ignore-eos"])
+    assert args.ignore_eos and args.stop_token_id is None

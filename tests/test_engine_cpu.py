@@ -453,6 +453,42 @@ def test_async_entry_point_streams_each_token_once(model_folders):
     assert streamed == outputs[0]
 
 
+def test_the_entry_point_closes_its_runner_forgets_old_facts_and_serves_again_after_a_failure(model_folders):
+    """`close` drops what the runner holds (a caller of `async with` need not know the runner); the facts of
+    finished requests that nobody asks for are bounded; after a step has failed and everybody was told, the
+    next request is served by a new task rather than waiting for one that has ended."""
+    config, weights = oracle(model_folders, "A")
+
+    async def run():
+        loaded = load_model_folder(model_folders["A"], "float32")
+        engine = LLMEngine(loaded, cache_config=CacheConfig(16, 32, 8), scheduler_config=SchedulerConfig(3, 64),
+                           dtype="float32", kernels=TorchKernels(torch.float32))
+        closed = []
+        engine.runner.close = lambda: closed.append(True)
+        engine.facts_kept = 2
+        for index in range(4):
+            await engine.generate([5 + index, 9], GenerationConfig(max_new_tokens=2), request_id=f"r{index}")
+        assert list(engine._facts) == ["r2", "r3"] and engine.request_facts("r3")["preemptions"] == 0
+        step, failing = engine.runner.step, [True]
+
+        def broken(*args, **kwargs):
+            if failing[0]:
+                raise RuntimeError("the device went away")
+            return step(*args, **kwargs)
+
+        engine.runner.step = broken
+        with pytest.raises(RuntimeError, match="went away"):
+            await engine.generate([1, 2, 3], GenerationConfig(max_new_tokens=2))
+        failing[0] = False
+        again = await asyncio.wait_for(engine.generate([1, 2, 3], GenerationConfig(max_new_tokens=3)), timeout=60)
+        assert engine.cache.used_pages == 0
+        await engine.close()
+        assert closed == [True]
+        return again
+
+    assert asyncio.run(run()) == plain.generate(weights, config, [1, 2, 3], 3)
+
+
 @pytest.mark.parametrize("case", range(12))
 def test_random_workloads_end_as_the_plain_decoder_says(model_folders, case):
     """Whole runs drawn at random: model (A, or B with its windowed layers), pool size, batch size,

@@ -199,7 +199,6 @@ def test_greedy_generation_through_the_entry_point(model_folders, dtype, name):
                 for index, prompt in enumerate(prompts)
             ])
             assert engine.cache.used_pages == 0
-            engine.runner.close()
             return outputs, streamed
 
     outputs, streamed = asyncio.run(run())
@@ -260,7 +259,19 @@ def test_command_line_generates(model_folders, tmp_path):
                            "--max-tokens", "6", *common], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr[-2000:]
     plain_config, weights = plain.PlainConfig.from_folder(model_folders["A"]), plain.read_weights(model_folders["A"])
-    assert json.loads(done.stdout.strip().splitlines()[-1])["token_ids"] == plain.generate(weights, plain_config, [5, 17, 3, 200], 6)
+    expected = plain.generate(weights, plain_config, [5, 17, 3, 200], 6)
+    assert json.loads(done.stdout.strip().splitlines()[-1])["token_ids"] == expected
+    # a folder that names its end-of-sequence token: generation stops there unless told otherwise
+    import shutil
+
+    named = tmp_path / "named"
+    shutil.copytree(model_folders["A"], named)
+    (named / "generation_config.json").write_text(json.dumps({"eos_token_id": [expected[2], 999999]}))
+    for extra, wanted in (([], expected[: expected.index(expected[2]) + 1]), (["--ignore-eos"], expected)):
+        done = subprocess.run([sys.executable, str(ROOT / "bin" / "llmserve"), "generate", "--prompt-tokens", "5,17,3,200",
+                               "--max-tokens", "6", "--model", str(named), *common[2:], *extra], capture_output=True, text=True, timeout=300)
+        assert done.returncode == 0, done.stderr[-2000:]
+        assert json.loads(done.stdout.strip().splitlines()[-1])["token_ids"] == wanted
     output = tmp_path / "bench.json"
     done = subprocess.run([sys.executable, str(ROOT / "bin" / "llmserve"), "benchmark", "--config", "continuous",
                            "--requests", "6", "--arrival-rate", "200", "--batch-size", "4", "--output", str(output),
