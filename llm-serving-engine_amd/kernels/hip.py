@@ -51,6 +51,7 @@ _SIGNATURES = {
     "llmserve_silu_mul": "pipiiip",
     "llmserve_gather_rows": "ppiippiip",
     "llmserve_gemm_generic": "pipipipiiiip",
+    "llmserve_gemm_f32": "ppppiiiiip",
     "llmserve_gemm_skinny": "pppipiiiiiip",
     "llmserve_gemm_stream": "pppipiiiiiip",
     "llmserve_gemm_stream_shaped": "pppipiiiiiiiip",
@@ -59,6 +60,7 @@ _SIGNATURES = {
     "llmserve_gemm_tiled": "pppipiiiiiip",
     "llmserve_gemm_wide": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifipfp",
+    "llmserve_attention_f32": "pippppppippiiiiiifiip",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
     "llmserve_attention_portions": "pippppippiiiiifip",
     "llmserve_attention_can_fuse": "i",
@@ -143,6 +145,7 @@ class HipKernels:
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
         self._elementwise = _declared(load_module("elementwise"))
         self._gemm_generic = _declared(load_module("gemm_generic"))
+        self._gemm_f32 = _declared(load_module("gemm_f32")) if dtype == torch.float32 else None
         self._attention_generic = _declared(load_module("attention_generic"))
         self._gemm_bf16 = _declared(load_module("gemm_bf16")) if dtype == torch.bfloat16 else None
         self._pinned_stream: int | None = None
@@ -157,6 +160,7 @@ class HipKernels:
                 torch.mm(one, one.t(), out_dtype=torch.float32)
                 torch.cuda.synchronize(self.device)
         self._attention_bf16: dict[int, ctypes.CDLL] = {}  # by head size, compiled when a model needs it
+        self._attention_f32: dict[int, ctypes.CDLL] = {}
         self._sampling = None
 
     # ------------------------------------------------------------------ helpers
@@ -482,6 +486,16 @@ class HipKernels:
                 )
             _check(status, "linear")
             return out
+        if self._all_float32(x, weights) and (out_dtype or self.dtype) == torch.float32:
+            splits = self._float32_splits(rows, weights.out_features, inner) if partial and out_dtype == torch.float32 else 1
+            shape = (rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features)
+            out = self._empty(shape, torch.float32)
+            status = self._gemm_f32.llmserve_gemm_f32(
+                _pointer(x), _pointer(weights.weight), _pointer(bias), _pointer(out), 0, rows, weights.out_features,
+                inner, splits, self._stream,
+            )
+            _check(status, "linear")
+            return out
         out = self._empty((rows, weights.out_features), out_dtype or self.dtype)
         status = self._gemm_generic.llmserve_gemm_generic(
             _pointer(x), _is_float(x), _pointer(weights.weight), _is_float(weights.weight), _pointer(bias),
@@ -490,8 +504,41 @@ class HipKernels:
         _check(status, "linear")
         return out
 
+    def _all_float32(self, x: torch.Tensor, weights: LinearWeights) -> bool:
+        """Whether the product is the true 32-bit path's: every operand float32 and a K that its 16-byte
+        loads can take (the generic kernel takes the rest: mixed types, any K)."""
+        return (
+            self._gemm_f32 is not None
+            and x.dtype == torch.float32
+            and weights.weight.dtype == torch.float32
+            and (weights.bias is None or weights.bias.dtype == torch.float32)
+            and weights.in_features % 4 == 0
+        )
+
+    @staticmethod
+    def _float32_splits(rows: int, out_features: int, in_features: int) -> int:
+        """Into how many parts of K a float32 product is cut when its result may stay in parts: up to 16
+        rows (the weight-streaming kernel, workgroups of 16 weight rows) until about a thousand workgroups
+        run, a part at least 512 long; more rows (128 x 128 tiles) until there is one tile for every CU."""
+        if rows <= 16:
+            tiles, least, goal = -(-out_features // 16), 512, 1024
+        else:
+            tiles, least, goal = -(-rows // 128) * -(-out_features // 128), 256, 256
+        best = 1
+        for splits in range(2, 9):
+            if in_features // splits >= least and tiles * splits <= goal:
+                best = splits
+        return best
+
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
         out = self._empty((x.shape[0], weights.width), self.dtype)
+        if self._all_float32(x, weights.both) and self.dtype == torch.float32:
+            status = self._gemm_f32.llmserve_gemm_f32(
+                _pointer(x), _pointer(weights.both.weight), None, _pointer(out), 1, x.shape[0], 2 * weights.width,
+                x.shape[1], 1, self._stream,
+            )
+            _check(status, "gated_linear")
+            return out
         streaming = self._streaming(x, weights.both, gated=True)
         if (
             streaming is None
@@ -531,12 +578,12 @@ class HipKernels:
         return self._attention_bf16[head_dim]
 
     @staticmethod
-    def _work_items(chunks, group: int, column_tiles: int, longer_than: int, up_to: int | None):
+    def _work_items(chunks, group: int, column_tiles: int, longer_than: int, up_to: int | None, packed: bool | None = None):
         """Work items (request, first row, first head, columns), int32 [items, 4], for the requests of
         the step whose token count lies in (longer_than, up_to], and about how many 32-key steps the
-        items walk all together.  With up to 16 query heads a kv head (`group`) an item is a run of
-        `column_tiles` * 16 (token, head) pairs of a request, token by token and head by head, wherever
-        in a token it begins; with more, `column_tiles` tokens (and "columns" counts tokens)."""
+        items walk all together.  With up to 16 query heads a kv head (`group`), or `packed` set, an item is
+        a run of `column_tiles` * 16 (token, head) pairs of a request, token by token and head by head,
+        wherever in a token it begins; else `column_tiles` tokens (and "columns" counts tokens)."""
         import numpy as np
 
         counts = np.array([chunk.count for chunk in chunks], dtype=np.int64)
@@ -545,7 +592,7 @@ class HipKernels:
         if up_to is not None:
             chosen &= counts <= up_to
         which = np.nonzero(chosen)[0]
-        packed = group <= 16
+        packed = group <= 16 if packed is None else packed
         per_token = group if packed else 1
         per_item = column_tiles * (16 if packed else 1)
         totals = counts[which] * per_token
@@ -560,26 +607,27 @@ class HipKernels:
         return work, steps
 
     @staticmethod
-    def _work_capacity(padded_to: tuple[int, int], group: int, column_tiles: int) -> int:
+    def _work_capacity(padded_to: tuple[int, int], group: int, column_tiles: int, packed: bool | None = None) -> int:
         """The most items a work list can have in a step of `padded_to` = (tokens, requests)."""
         tokens, requests = padded_to
-        per_token = group if group <= 16 else 1
-        per_item = column_tiles * (16 if group <= 16 else 1)
+        packed = group <= 16 if packed is None else packed
+        per_token = group if packed else 1
+        per_item = column_tiles * (16 if packed else 1)
         return -(-tokens * per_token // per_item) + requests
 
-    def _attention_work(self, batch, group: int, column_tiles: int, longer_than: int, up_to: int | None):
+    def _attention_work(self, batch, group: int, column_tiles: int, longer_than: int, up_to: int | None, packed: bool | None = None):
         """The work list of `_work_items` on the device, built once per step and kept on the batch:
         (tensor or None, items, steps).  A batch that is `padded_to` (tokens, requests) for a captured
         step gets a list of the most items such a step can have, the unused ones of no columns: the
         captured launch covers whatever step is replayed, once `refresh_step` has filled in its items."""
-        key = ("attention_work", group, column_tiles, longer_than, up_to)
+        key = ("attention_work", group, column_tiles, longer_than, up_to, packed)
         if key not in batch.scratch:
-            work, steps = self._work_items(batch.chunks, group, column_tiles, longer_than, up_to)
+            work, steps = self._work_items(batch.chunks, group, column_tiles, longer_than, up_to, packed)
             padded_to = getattr(batch, "padded_to", None)
             if padded_to is not None:
                 import numpy as np
 
-                capacity = self._work_capacity(padded_to, group, column_tiles)
+                capacity = self._work_capacity(padded_to, group, column_tiles, packed)
                 if len(work) > capacity:
                     raise KernelError("a step holds more attention work than its padded shape allows")
                 work = np.concatenate([work, np.zeros((capacity - len(work), 4), np.int32)])
@@ -631,6 +679,9 @@ class HipKernels:
         if plain_scores and qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
             self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0))
             return out
+        if plain_scores and qkv.dtype == torch.float32 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
+            self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0))
+            return out
         if qkv.dtype == torch.bfloat16:
             why = "its scores carry a bias or a soft cap" if not plain_scores else f"head size {dim} and pages of {group.page_size}"
             self._tell_once(f"generic attention: {why}", f"bfloat16 attention runs on the generic kernel, not on the matrix cores: {why}")
@@ -642,6 +693,35 @@ class HipKernels:
         )
         _check(status, "paged_attention")
         return out
+
+    def _attention_float32(self, qkv, out, layout, batch, cell, group, scale: float, window: int) -> None:
+        """The 32-bit path's attention on the matrix cores: an item is 16 (decoding) or 32 columns of one
+        request, (token, head) pairs running through the tokens head by head whatever the number of heads; few
+        items over long contexts are cut into key splits that a second kernel merges."""
+        dim = layout.head_dim
+        if dim not in self._attention_f32:
+            self._attention_f32[dim] = _declared(load_module("attention_f32", {"HEAD_DIM": dim}))
+        heads, kv_heads = layout.num_heads, layout.num_kv_heads
+        group_size = heads // kv_heads
+        column_tiles = 2 if batch.max_query_length * group_size > 16 else 1
+        work, items, _ = self._attention_work(batch, group_size, column_tiles, 0, None, True)
+        if items == 0:
+            return
+        tokens = qkv.shape[0]
+        # a wave walks its share of the keys 16 at a time: split where a workgroup would walk more than 32 steps
+        # a wave and the chip has room for more workgroups
+        steps = -(-batch.max_context_length // 16)
+        splits = max(1, min(32, 1024 // (items * kv_heads), steps // 128))
+        partial_acc = partial_ml = None
+        if splits > 1:
+            partial_acc = self._empty((splits, tokens * heads, dim), torch.float32)
+            partial_ml = self._empty((splits, tokens * heads, 2), torch.float32)
+        status = self._attention_f32[dim].llmserve_attention_f32(
+            _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml), _pointer(cell.keys),
+            _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work),
+            items, column_tiles, tokens, heads, kv_heads, group.page_size, scale, window, splits, self._stream,
+        )
+        _check(status, "paged_attention")
 
     def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None, unmerged=False):
         """The MFMA kernel: requests that bring a few tokens (decoding) one column tile per

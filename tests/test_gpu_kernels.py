@@ -302,11 +302,13 @@ def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, wind
     torch.testing.assert_close(out, other, **TOLERANCE[dtype])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("window", [None, 1500])
-def test_paged_attention_portion_of_a_long_context(kernels, window):
+def test_paged_attention_portion_of_a_long_context(kernels, window, dtype):
     """A portion at the end of a context of more than 4,096 keys (hundreds of steps a wave, many
-    pages), with a far key that dominates and, with a window, lies just inside it."""
-    heads, kv_heads, dim, page, dtype = 6, 2, 64, 16, torch.bfloat16
+    pages; in float32 the keys are cut into splits that a second kernel merges), with a far key that
+    dominates and, with a window, lies just inside it."""
+    heads, kv_heads, dim, page = 6, 2, 64, 16
     lengths, counts = [4200, 37], [150, 37]
     batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=3)
     q, k, v = per_request[0]
@@ -321,6 +323,51 @@ def test_paged_attention_portion_of_a_long_context(kernels, window):
         expected.append(full[-count:].flatten(1))
     torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
     torch.testing.assert_close(out[149].view(heads, dim)[0], rounded(per_request[0][2], dtype)[far, 0], atol=5e-2, rtol=0)
+
+
+@pytest.mark.parametrize("window", [None, 3000])
+def test_float32_decode_attention_over_many_key_splits(kernels, window):
+    """Two requests decode over 9,000 and 5,003 keys in float32: few items, so each is cut into several key
+    splits (some of them empty for the shorter request, some wholly outside the window) that the merging
+    kernel adds up; a far key per request dominates one head."""
+    heads, kv_heads, dim, page, dtype = 10, 2, 128, 16, torch.float32
+    lengths, counts = [9000, 5003], [1, 1]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=11)
+    fars = [6500, 2100]
+    for (q, k, v), far in zip(per_request, fars):
+        k[far] = 2.0 * q[-1, ::5]  # heads 0 and 5 share kv heads 0 and 1
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    out = kernels[dtype].paged_attention(qkv, layout, batch, cell, 0.5, window).cpu().double()
+    for row, ((q, k, v), far) in enumerate(zip(per_request, fars)):
+        full = plain.causal_attention(q.double(), k.double(), v.double(), 0.5, window)[-1]
+        torch.testing.assert_close(out[row].view(heads, dim), full, **TOLERANCE[dtype])
+        torch.testing.assert_close(out[row].view(heads, dim)[0], v.double()[far, 0], atol=5e-2, rtol=0)
+
+
+@pytest.mark.parametrize("rows,inner,outer", [(3, 100, 77), (8, 8960, 1536), (16, 1536, 48), (11, 2052, 130),
+                                              (40, 8960, 200), (200, 4480, 130), (130, 100, 77), (2048, 264, 384),
+                                              (129, 2048, 1030)])
+def test_float32_products_in_parts_and_at_odd_sizes(kernels, rows, inner, outer):
+    """The 32-bit path's products on the matrix cores: K that is a multiple of 4 but not of 16 or 64, rows and
+    weight rows that fill no tile, and K cut into partial sums where the result may stay in parts (up to 16 rows:
+    the weight-streaming kernel; more: the tiled one), with bias, and with SiLU(gate) * up over interleaved rows.
+    The bound is that of a float32 sum of K terms in any order: a few times sqrt(K) * 2^-24 of its size."""
+    k = kernels[torch.float32]
+    x, w, b = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer)
+    expected = x.double() @ w.double().T + b.double()
+    bound = dict(atol=8 * math.sqrt(inner) * 2.0 ** -24, rtol=1e-5)
+    handle = k.prepare_linear([on_gpu(w)], [on_gpu(b)])
+    torch.testing.assert_close(k.linear(on_gpu(x), handle).cpu().double(), expected, **bound)
+    parts = k.linear(on_gpu(x), handle, out_dtype=torch.float32, partial=True)
+    cut = k._float32_splits(rows, outer, inner)
+    assert parts.shape == ((cut, rows, outer) if cut > 1 else (rows, outer)) and (cut > 1 or inner < 2048 or rows > 200)
+    summed = parts if parts.ndim == 2 else parts.double().sum(0)
+    torch.testing.assert_close(summed.cpu().double(), expected, **bound)
+    up = torch.randn(outer, inner) / math.sqrt(inner)
+    gated = k.gated_linear(on_gpu(x), k.prepare_gated_linear(on_gpu(w), on_gpu(up)))
+    want = F.silu(x.double() @ w.double().T) * (x.double() @ up.double().T)
+    torch.testing.assert_close(gated.cpu().double(), want, **bound)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
