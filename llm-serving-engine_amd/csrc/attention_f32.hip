@@ -98,20 +98,33 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
   const size_t page_elements = (size_t)page_size * D;
   const int piece_stride = page_size * KEY_PIECE;  // between the pieces of a key (common.h: key_element)
 
+  // Which key a lane reads for the first product (key0 + i) and which four for the second (key0 + 4 g .. + 3, one
+  // page: pages are multiples of 4).  A key outside the item's range is masked, and its page may have been given
+  // back: the nearest inside is read instead.  The pages of a wave's next step are looked up a step ahead.
+  auto key_of = [&](int step) { return max(min(step * KEYS + i, end - 1), begin); };
+  auto value_key_of = [&](int step) { return max(min(step * KEYS + 4 * g, (end - 1) & ~3), begin & ~3); };
+  int next_key_page = 0, next_value_page = 0;
+  if (my_first + wave < my_end) {
+    next_key_page = table[key_of(my_first + wave) / page_size];
+    next_value_page = table[value_key_of(my_first + wave) / page_size];
+  }
   for (int step = my_first + wave; step < my_end; step += WAVES) {
     const int key0 = step * KEYS;
-    // K: lane (i, g) reads d = 16 s + 4 g .. + 3 of key key0 + i (a key outside the item's range is masked, and
-    // its page may have been given back: the nearest key inside is read instead)
-    const int key_mine = max(min(key0 + i, end - 1), begin);
-    const int key_page = table[key_mine / page_size];
+    // K: lane (i, g) reads d = 16 s + 4 g .. + 3 of its key
+    const int key_mine = key_of(step);
+    const int key_page = next_key_page;
     const float* k_at = keys + ((size_t)key_page * kv_heads + kv_head) * page_elements +
                         (size_t)(key_mine % page_size) * KEY_PIECE + (g >> 1) * piece_stride + (g & 1) * 4;
     f32x4 k[D_STEPS];
 #pragma unroll
     for (int s = 0; s < D_STEPS; ++s) k[s] = load4(k_at + (size_t)(2 * s) * piece_stride);
-    // V^T: lane (i, g) reads keys key0 + 4 g .. + 3 (one page: pages are multiples of 4) of row d = 16 s + i
-    const int value_key = max(min(key0 + 4 * g, (end - 1) & ~3), begin & ~3);
-    const int value_page = table[value_key / page_size];
+    // V^T: lane (i, g) reads its four keys of row d = 16 s + i
+    const int value_key = value_key_of(step);
+    const int value_page = next_value_page;
+    if (step + WAVES < my_end) {
+      next_key_page = table[key_of(step + WAVES) / page_size];
+      next_value_page = table[value_key_of(step + WAVES) / page_size];
+    }
     const float* v_at = values + ((size_t)value_page * kv_heads + kv_head) * page_elements + (size_t)i * page_size +
                         value_key % page_size;
     f32x4 v[D_STEPS];

@@ -5,7 +5,7 @@
 // model.py:60-66 via nn.Linear); gemm_generic.hip remains for operands of mixed types and for a K
 // that is no multiple of 4.
 //
-// gemm_f32_stream (M <= 16, decoding): the product is a stream of the weight matrix from HBM.  A
+// gemm_f32_stream (M <= 64, decoding): the product is a stream of the weight matrix from HBM.  A
 // workgroup owns 16 weight rows and its waves split K between them; lane (r, g) keeps groups of four
 // 16-byte loads of weight row r in flight, k = 16 s + 4 g .. + 3 of every 16-wide step s.  An MFMA
 // takes a 16 x 4 piece of the weights as its A operand (lane (r, g) gives A[r][g]) and 4 x 16 of x^T as
@@ -32,23 +32,32 @@ __device__ __forceinline__ f32x4 load4(const float* p) { return *(const f32x4*)p
 
 __device__ __forceinline__ float silu(float gate) { return gate / (1.f + expf(-gate)); }
 
-template <int WAVES, bool GATED>
+// MT: 16-row tiles of x (up to 16 MT rows): every weight operand meets MT operands of x, which each wave
+// reads for itself (M / 16 of what it reads of the weights, from L2).
+template <int WAVES, int MT, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_f32_stream_kernel(const float* __restrict__ x,
                                                                      const float* __restrict__ w,
                                                                      const float* __restrict__ bias,
                                                                      float* __restrict__ out, int M, int N, int K,
                                                                      int k_split) {
-  extern __shared__ float partial[];  // [WAVES][64 lanes][4]
+  extern __shared__ float partial[];  // [WAVES][MT][64 lanes][4]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
   const int n = min((int)blockIdx.x * 16 + r, N - 1);
   const int k_first = blockIdx.y * k_split;
   const int k_count = min(k_split, K - k_first);  // the last slice may be shorter
   const float* w_row = w + (size_t)n * K + k_first + g * 4;
-  const bool x_live = r < M;
-  const float* x_row = x + (size_t)min(r, M - 1) * K + k_first + g * 4;
+  bool x_live[MT];
+  const float* x_row[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    x_live[t] = t * 16 + r < M;
+    x_row[t] = x + (size_t)min(t * 16 + r, M - 1) * K + k_first + g * 4;
+  }
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-  f32x4 acc = zero;
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = zero;
 
   const int groups = k_count / (16 * STREAM_GROUP);
   f32x4 a[STREAM_GROUP], a_next[STREAM_GROUP];
@@ -61,18 +70,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_f32_stream_kernel(const float
     const int next = group + WAVES;
     // this group's x is asked for before the next group's weights: loads come back in the order
     // they were asked for, and the products below wait for x
-    f32x4 b[STREAM_GROUP];
+    f32x4 b[MT][STREAM_GROUP];
 #pragma unroll
-    for (int u = 0; u < STREAM_GROUP; ++u) b[u] = x_live ? load4(x_row + (group * STREAM_GROUP + u) * 16) : zero;
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int u = 0; u < STREAM_GROUP; ++u) b[t][u] = x_live[t] ? load4(x_row[t] + (group * STREAM_GROUP + u) * 16) : zero;
     asm volatile("" ::: "memory");
     if (next < groups) {
 #pragma unroll
       for (int u = 0; u < STREAM_GROUP; ++u) a_next[u] = load4(w_row + (next * STREAM_GROUP + u) * 16);
     }
 #pragma unroll
-    for (int u = 0; u < STREAM_GROUP; ++u)
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][j], b[u][j], acc, 0, 0, 0);
+      for (int u = 0; u < STREAM_GROUP; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][j], b[t][u][j], acc[t], 0, 0, 0);
 #pragma unroll
     for (int u = 0; u < STREAM_GROUP; ++u) a[u] = a_next[u];
     group = next;
@@ -81,18 +94,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_f32_stream_kernel(const float
   for (int step = groups * STREAM_GROUP + wave; step * 16 < k_count; step += WAVES) {
     const bool inside = step * 16 + g * 4 < k_count;
     const f32x4 a_tail = inside ? load4(w_row + step * 16) : zero;
-    const f32x4 b_tail = inside && x_live ? load4(x_row + step * 16) : zero;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a_tail[j], b_tail[j], acc, 0, 0, 0);
+    for (int t = 0; t < MT; ++t) {
+      const f32x4 b_tail = inside && x_live[t] ? load4(x_row[t] + step * 16) : zero;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_tail[j], b_tail[j], acc[t], 0, 0, 0);
+    }
   }
 
-  *(f32x4*)(partial + (wave * 64 + lane) * 4) = acc;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) *(f32x4*)(partial + ((wave * MT + t) * 64 + lane) * 4) = acc[t];
   __syncthreads();
-  if (wave != 0) return;
-  // D[n][m]: the lane holds token m = r and rows n0 + 4 g .. + 3
+  if (wave >= MT) return;
+  // wave t finishes tile t of x.  D[n][m]: the lane holds token m = 16 t + r and rows n0 + 4 g .. + 3
+  const int t = wave;
   f32x4 total = zero;
-  for (int v = 0; v < WAVES; ++v) total += *(const f32x4*)(partial + (v * 64 + lane) * 4);
-  const int m = r;
+  for (int v = 0; v < WAVES; ++v) total += *(const f32x4*)(partial + ((v * MT + t) * 64 + lane) * 4);
+  const int m = t * 16 + r;
   const int n_first = blockIdx.x * 16 + g * 4;
   if (m >= M) return;
   if (bias && blockIdx.y == 0) {
@@ -112,13 +130,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_f32_stream_kernel(const float
   }
 }
 
-template <int WAVES, bool GATED>
+template <int WAVES, int MT, bool GATED>
 static int launch_stream(const float* x, const float* w, const float* bias, float* out, int M, int N, int K, int splits,
                          int k_split, hipStream_t stream) {
-  const size_t lds = (size_t)WAVES * 64 * 4 * sizeof(float);
-  hipLaunchKernelGGL((gemm_f32_stream_kernel<WAVES, GATED>), dim3((N + 15) / 16, splits), dim3(WAVES * 64), lds, stream,
-                     x, w, bias, out, M, N, K, k_split);
+  const size_t lds = (size_t)WAVES * MT * 64 * 4 * sizeof(float);
+  hipLaunchKernelGGL((gemm_f32_stream_kernel<WAVES, MT, GATED>), dim3((N + 15) / 16, splits), dim3(WAVES * 64), lds,
+                     stream, x, w, bias, out, M, N, K, k_split);
   return LAUNCH_STATUS();
+}
+
+template <int WAVES, bool GATED>
+static int pick_tiles(const float* x, const float* w, const float* bias, float* out, int M, int N, int K, int splits,
+                      int k_split, hipStream_t stream) {
+  if (M <= 16) return launch_stream<WAVES, 1, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
+  if (M <= 32) return launch_stream<WAVES, 2, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
+  return launch_stream<WAVES, 4, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
 }
 
 template <bool GATED>
@@ -131,9 +157,9 @@ static int pick_stream(const float* x, const float* w, const float* bias, float*
   const int tiles = (N + 15) / 16 * splits, groups = max(1, k_split / (16 * STREAM_GROUP));
   int waves = 4;
   while (waves < 16 && waves * tiles < 2048 && waves * 2 <= groups) waves *= 2;
-  if (waves == 4) return launch_stream<4, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
-  if (waves == 8) return launch_stream<8, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
-  return launch_stream<16, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
+  if (waves == 4) return pick_tiles<4, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
+  if (waves == 8) return pick_tiles<8, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
+  return pick_tiles<16, GATED>(x, w, bias, out, M, N, K, splits, k_split, stream);
 }
 
 // ---------------------------------------------------------------------------- many rows
@@ -288,12 +314,12 @@ static int launch_tiled(const float* x, const float* w, const float* bias, float
 
 // out [M, N] (or [splits, M, N] partial sums) = x [M, K] . w [N, K]^T (+ bias [N]); all float32, K a multiple
 // of 4.  gated: w's rows alternate gate and up (N even), out is [M, N / 2] = silu(gate) * up, no splits.
-// Up to 16 rows of x go to the weight-streaming kernel, more to the tiled one.
+// Up to 64 rows of x go to the weight-streaming kernel, more to the tiled one.
 extern "C" int llmserve_gemm_f32(const float* x, const float* w, const float* bias, float* out, int gated, int M, int N,
                                  int K, int splits, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 4 || splits < 1 || (gated && (splits != 1 || N % 2))) return ERR_BAD_ARGUMENT;
-  if (M <= 16)
+  if (M <= 64)
     return gated ? pick_stream<true>(x, w, bias, out, M, N, K, splits, stream)
                  : pick_stream<false>(x, w, bias, out, M, N, K, splits, stream);
   return gated ? launch_tiled<true>(x, w, bias, out, M, N, K, splits, stream)

@@ -517,10 +517,10 @@ class HipKernels:
 
     @staticmethod
     def _float32_splits(rows: int, out_features: int, in_features: int) -> int:
-        """Into how many parts of K a float32 product is cut when its result may stay in parts: up to 16
+        """Into how many parts of K a float32 product is cut when its result may stay in parts: up to 64
         rows (the weight-streaming kernel, workgroups of 16 weight rows) until about a thousand workgroups
         run, a part at least 512 long; more rows (128 x 128 tiles) until there is one tile for every CU."""
-        if rows <= 16:
+        if rows <= 64:
             tiles, least, goal = -(-out_features // 16), 512, 1024
         else:
             tiles, least, goal = -(-rows // 128) * -(-out_features // 128), 256, 256
@@ -708,10 +708,12 @@ class HipKernels:
         if items == 0:
             return
         tokens = qkv.shape[0]
-        # a wave walks its share of the keys 16 at a time: split where a workgroup would walk more than 32 steps
-        # a wave and the chip has room for more workgroups
+        # A wave walks its share of the keys 16 at a time, a trip to memory and sixty-four products a step, so a
+        # walk is as long as its steps are many: where the chip has room for more workgroups the keys are split
+        # until a wave has two steps or so (a decode step of 8 requests over 530 keys: 61 us unsplit; the merge
+        # kernel costs about 5).
         steps = -(-batch.max_context_length // 16)
-        splits = max(1, min(32, 1024 // (items * kv_heads), steps // 128))
+        splits = max(1, min(32, 1024 // (items * kv_heads), steps // 8))
         partial_acc = partial_ml = None
         if splits > 1:
             partial_acc = self._empty((splits, tokens * heads, dim), torch.float32)
