@@ -2,41 +2,60 @@
 
 from __future__ import annotations
 
-from dataclasses import dataclass
 from typing import Any
 
 import torch
 
-
-KEY_PIECE = 8  # elements of a key that stay together in a page (csrc/common.h has the same number)
-
-
-def key_piece_width(head_dim: int) -> int:
-    """A key is kept in pieces of KEY_PIECE elements; a head size that is no multiple of it in one piece."""
-    return KEY_PIECE if head_dim % KEY_PIECE == 0 else head_dim
+from ..parts.base import KEY_PIECE, key_piece_width  # noqa: F401  (kernel libraries and tests find them here)
 
 
-@dataclass
 class CacheCell:
-    """What one run of a layer sees of the cache.
+    """What one run of a layer sees of the cache, for one of its needs.
 
-    For a paged need: `keys` is [pages, kv_heads, head_dim / w, page_size, w] with w =
-    `key_piece_width(head_dim)`: a key lies in pieces of w elements, the same piece of all
-    the keys of a page side by side (the matrix cores take keys as rows, a lane holding one
-    piece of one key and its neighbours that piece of the next keys, and neighbouring lanes
-    should read neighbouring bytes).  `values` is stored transposed, [pages, kv_heads,
-    head_dim, page_size] (attention sums over keys, and the matrix cores want the summed
-    index contiguous).  `group` indexes `StepBatch.groups`.  For a fixed state: `state` is
-    [slots, *shape] float32, indexed by `StepBatch.state_slots`.  `writable` is False when
-    the run reads a cell that another run owns.
+    For a paged need: `fields` holds, by the names the need gave in `page_fields`, the tensors
+    [pages, *page shape] of this run, and `group` indexes `StepBatch.groups` (where the step's tokens
+    go, and the requests' block tables).  For keys and values (`PagedKeyValue`): `keys` is [pages,
+    kv_heads, head_dim / w, page_size, w] with w = `key_piece_width(head_dim)`, `values` is stored
+    transposed, [pages, kv_heads, head_dim, page_size]; both are also attributes of the cell.
+    For a per-request need: `state` is [slots, *shape] float32, indexed by `StepBatch.state_slots`.
+    `writable` is False when the run reads a cell that another run owns.
     """
 
-    need: Any
-    writable: bool = True
-    group: int = -1
-    keys: torch.Tensor | None = None
-    values: torch.Tensor | None = None
-    state: torch.Tensor | None = None
+    def __init__(
+        self,
+        need: Any,
+        writable: bool = True,
+        group: int = -1,
+        keys: torch.Tensor | None = None,
+        values: torch.Tensor | None = None,
+        state: torch.Tensor | None = None,
+        fields: dict[str, torch.Tensor] | None = None,
+    ) -> None:
+        self.need = need
+        self.writable = writable
+        self.group = group
+        self.state = state
+        self.fields: dict[str, torch.Tensor] = dict(fields or {})
+        if keys is not None:
+            self.fields["keys"] = keys
+        if values is not None:
+            self.fields["values"] = values
+
+    @property
+    def keys(self) -> torch.Tensor | None:
+        return self.fields.get("keys")
+
+    @keys.setter
+    def keys(self, tensor: torch.Tensor) -> None:
+        self.fields["keys"] = tensor
+
+    @property
+    def values(self) -> torch.Tensor | None:
+        return self.fields.get("values")
+
+    @values.setter
+    def values(self, tensor: torch.Tensor) -> None:
+        self.fields["values"] = tensor
 
     def key_rows(self, pages: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
         """The keys at (pages[i], offsets[i]) as whole rows, [n, kv_heads, head_dim]."""

@@ -1,14 +1,17 @@
-"""The cache manager: pages of keys and values with a block table per request,
-one pool per group of layers with the same need, and slots of fixed-size state.
+"""The cache manager: pages with a block table per request, one pool per group of
+layers with the same need, and slots of fixed-size state.
 
 The reference keeps one tensor [L, 2, NB, P, Hkv, D] for all layers, one block
 table per sequence and a metadata row per sequence (`kv_cache.py:91-179`).  Here
-the layers that run are first sorted into groups by what their mixer needs
-(all keys, a window of keys, a fixed state, nothing); every paged group has its
-own pool, storage [cells, 2, NB, Hkv, P, D] and block tables, and a windowed
-group gives a page back as soon as no later query can read it.  A request's
-slot (the reference's metadata row) is its block-table row in every group and
-its index into every fixed-state tensor.
+the layers that run are first sorted into groups by what their parts need: an
+entry per token (`PagedNeed`: all of them, or a window) or an entry per request
+(`SlotNeed`); a run may need several things at once.  Every paged group has its
+own pool, block tables and, for each field its need names, a tensor [cells, NB,
+*page shape]: what a page holds is the need's business (keys and values for
+attention), the manager only hands pages out and takes them back, and a windowed
+group gives a page back as soon as no later query can read it.  A request's slot
+(the reference's metadata row) is its block-table row in every group and its
+index into every per-request tensor.
 """
 
 from __future__ import annotations
@@ -21,26 +24,25 @@ import numpy as np
 import torch
 
 from ..config.serving import CacheConfig
-from .cell import CacheCell, key_piece_width
-from ..parts.base import FixedState, PagedKeyValue
+from .cell import CacheCell
+from ..parts.base import CacheNeed, PagedNeed, SlotNeed
 from ..parts.model import ModelSpec
 from .pool import CacheFullError, PagePool
 
 
 @dataclass
 class PageGroup:
-    need: PagedKeyValue
-    cells: list[int]  # runs of the run order that own a cell in this group
+    need: PagedNeed
+    cells: list[tuple[int, str | None]]  # (run of the run order, name of the need in that run) of every cell here
     pool: PagePool
-    storage: torch.Tensor | None  # [len(cells), 2, NB, Hkv, P, D]
+    storage: dict[str, torch.Tensor]  # by field of the need: [len(cells), NB, *page shape]
     tables: np.ndarray  # int32 [max_sequences, max_blocks]; -1 where no page is held
     peak_pages: int = 0
 
     @property
     def bytes_per_page(self) -> int:
-        if self.storage is None:
-            return 0
-        return self.storage[:, :, 0].numel() * self.storage.element_size()
+        """What one page takes over all cells and fields of the group."""
+        return sum(tensor[:, 0].numel() * tensor.element_size() for tensor in self.storage.values())
 
 
 @dataclass
@@ -88,79 +90,73 @@ class CacheManager:
         self._high_water = {"pages": 0, "used_tokens": 0, "sequences": 0}
 
         self.groups: list[PageGroup] = []
-        self._cell_of_run: list[tuple[str, int, int] | None] = []  # (kind, group or state index, index inside)
+        # per run: by name of the need (None for a run with one need) -> (kind, group or state index, index inside)
+        self._cell_of_run: list[dict[str | None, tuple[str, int, int]]] = []
         self.states: list[torch.Tensor] = []
-        self._state_needs: list[FixedState] = []
-        by_need: dict[PagedKeyValue, int] = {}
-        owners: dict[int, tuple[str, int, int]] = {}
+        self._state_needs: list[SlotNeed] = []
+        by_need: dict[PagedNeed, int] = {}
         for index, run in enumerate(spec.run_order):
             if run.reads is not None:
-                self._cell_of_run.append(owners[run.reads])
+                self._cell_of_run.append(self._cell_of_run[run.reads])
                 continue
-            need = spec.cell_need(index)
-            if need is None:
-                entry = None
-            elif isinstance(need, PagedKeyValue):
-                if need not in by_need:
-                    by_need[need] = len(self.groups)
-                    self.groups.append(
-                        PageGroup(
-                            need,
-                            [],
-                            PagePool(config.num_blocks),
-                            None,
-                            np.full((config.max_sequences, self.max_blocks_per_sequence), -1, np.int32),
-                        )
+            entries: dict[str | None, tuple[str, int, int]] = {}
+            for name, need in self._named(spec.cell_need(index), index).items():
+                if isinstance(need, PagedNeed):
+                    if need not in by_need:
+                        by_need[need] = len(self.groups)
+                        tables = np.full((config.max_sequences, self.max_blocks_per_sequence), -1, np.int32)
+                        self.groups.append(PageGroup(need, [], PagePool(config.num_blocks), {}, tables))
+                    group = by_need[need]
+                    self.groups[group].cells.append((index, name))
+                    entries[name] = ("pages", group, len(self.groups[group].cells) - 1)
+                elif isinstance(need, SlotNeed):
+                    self._state_needs.append(need)
+                    # one slot more than there are requests: the state of the requests that pad a captured step
+                    self.states.append(
+                        torch.zeros((config.max_sequences + 1, *need.shape), dtype=torch.float32, device=self.device)
                     )
-                group = by_need[need]
-                self.groups[group].cells.append(index)
-                entry = ("pages", group, len(self.groups[group].cells) - 1)
-            elif isinstance(need, FixedState):
-                self._state_needs.append(need)
-                # one slot more than there are requests: the state of the requests that pad a captured step
-                self.states.append(
-                    torch.zeros((config.max_sequences + 1, *need.shape), dtype=torch.float32, device=self.device)
-                )
-                entry = ("state", len(self.states) - 1, 0)
-            else:
-                raise TypeError(f"run {index}: unknown cache need {need!r}")
-            owners[index] = entry
-            self._cell_of_run.append(entry)
+                    entries[name] = ("state", len(self.states) - 1, 0)
+                else:
+                    raise TypeError(f"run {index}: a cache need is a PagedNeed or a SlotNeed, not {need!r}")
+            self._cell_of_run.append(entries)
         for group in self.groups:
-            need = group.need
-            shape = (len(group.cells), 2, config.num_blocks, need.num_kv_heads, self.page_size, need.head_dim)
-            group.storage = torch.zeros(shape, dtype=dtype, device=self.device)
+            for field_name, shape in group.need.page_fields(self.page_size).items():
+                group.storage[field_name] = torch.zeros(
+                    (len(group.cells), config.num_blocks, *shape), dtype=dtype, device=self.device
+                )
+
+    @staticmethod
+    def _named(need: "CacheNeed | dict[str, CacheNeed] | None", run: int) -> dict[str | None, CacheNeed]:
+        """A run's needs by name: none, one (under None), or the several its block named."""
+        if need is None:
+            return {}
+        if isinstance(need, dict):
+            if any(not isinstance(name, str) for name in need):
+                raise TypeError(f"run {run}: several cache needs are named by strings")
+            return {name: value for name, value in need.items() if value is not None}
+        return {None: need}
 
     # ------------------------------------------------------------------ views
 
-    def cells(self) -> list[CacheCell | None]:
-        """One cell per entry of the run order, in order."""
-        views: list[CacheCell | None] = []
-        for index, entry in enumerate(self._cell_of_run):
+    def _cell(self, entry: tuple[str, int, int], writable: bool) -> CacheCell:
+        if entry[0] == "pages":
+            group = self.groups[entry[1]]
+            fields = {name: tensor[entry[2]] for name, tensor in group.storage.items()}
+            return CacheCell(need=group.need, writable=writable, group=entry[1], fields=fields)
+        return CacheCell(need=self._state_needs[entry[1]], writable=writable, state=self.states[entry[1]])
+
+    def cells(self) -> list["CacheCell | dict[str, CacheCell] | None"]:
+        """One entry per entry of the run order, in order: the run's cell, None for a run that keeps
+        nothing, or the cells by name for a run whose block named several needs."""
+        views: list[CacheCell | dict[str, CacheCell] | None] = []
+        for index, entries in enumerate(self._cell_of_run):
             writable = self.spec.run_order[index].reads is None
-            if entry is None:
+            if not entries:
                 views.append(None)
-            elif entry[0] == "pages":
-                group = self.groups[entry[1]]
-                views.append(
-                    CacheCell(
-                        need=group.need,
-                        writable=writable,
-                        group=entry[1],
-                        keys=group.storage[entry[2], 0].view(
-                            self.config.num_blocks, group.need.num_kv_heads,
-                            group.need.head_dim // key_piece_width(group.need.head_dim), self.page_size,
-                            key_piece_width(group.need.head_dim),
-                        ),
-                        values=group.storage[entry[2], 1].view(
-                            self.config.num_blocks, group.need.num_kv_heads, group.need.head_dim, self.page_size
-                        ),
-                    )
-                )
+            elif None in entries:
+                views.append(self._cell(entries[None], writable))
             else:
-                views.append(
-                    CacheCell(need=self._state_needs[entry[1]], writable=writable, state=self.states[entry[1]])
-                )
+                views.append({name: self._cell(entry, writable) for name, entry in entries.items()})
         return views
 
     # ------------------------------------------------------------------ requests
@@ -292,42 +288,52 @@ class CacheManager:
 
     # ------------------------------------------------------------------ host-side read paths
 
-    def _paged_cell(self, run: int) -> tuple[PageGroup, int, int]:
-        entry = self._cell_of_run[run] if 0 <= run < len(self._cell_of_run) else None
+    def _paged_cell(self, run: int, name: str | None = None) -> tuple[PageGroup, int, int]:
+        entries = self._cell_of_run[run] if 0 <= run < len(self._cell_of_run) else {}
+        entry = entries.get(name)
         if entry is None or entry[0] != "pages":
-            raise ValueError(f"run {run} of the run order keeps no pages")
+            raise ValueError(f"run {run} of the run order keeps no pages" + (f" under {name!r}" if name else ""))
         return self.groups[entry[1]], entry[1], entry[2]
 
-    def iter_pages(self, request_id: str, run: int):
-        """Walks what run `run` of the run order has cached for the request, page by page in logical
-        order: yields (first position, keys [n, kv_heads, head_dim], values [n, kv_heads, head_dim]),
-        the last page cut at the request's length, pages that a window has given back left out.  A
-        debugging and testing aid, as the reference's `iter_kv_blocks` (`kv_cache.py:268-296`): the
-        kernels read through the block tables themselves."""
-        group, group_index, cell = self._paged_cell(run)
+    def iter_page_fields(self, request_id: str, run: int, name: str | None = None):
+        """Walks what run `run` of the run order has cached for the request (under `name`, for a run with
+        several needs), page by page in logical order: yields (first position, {field: [n, ...]}), the
+        token's place in the page leading (the need's `token_rows`), the last page cut at the request's
+        length, pages that a window has given back left out.  A debugging and testing aid, as the
+        reference's `iter_kv_blocks` (`kv_cache.py:268-296`): the kernels read through the block tables
+        themselves."""
+        group, group_index, cell = self._paged_cell(run, name)
         record = self.sequences[request_id]
         table = group.tables[record.slot]
         page_size = self.page_size
         for block in range(record.released[group_index], math.ceil(record.length / page_size)):
             held = min(page_size, record.length - block * page_size)
-            page = int(table[block])
-            heads, dim = group.need.num_kv_heads, group.need.head_dim
-            # key pages are kept in pieces, [kv_heads, dim / w, offset, w] (`CacheCell`)
-            width = key_piece_width(dim)
-            keys = group.storage[cell, 0, page].view(heads, dim // width, page_size, width)[:, :, :held]
-            # value pages are kept transposed, [kv_heads, head_dim, offset]
-            values = group.storage[cell, 1, page].view(heads, dim, page_size)[:, :, :held]
-            yield block * page_size, keys.permute(2, 0, 1, 3).reshape(held, heads, dim), values.permute(2, 0, 1)
+            page = {field: tensor[cell, int(table[block])] for field, tensor in group.storage.items()}
+            rows = group.need.token_rows(page, page_size)
+            yield block * page_size, {field: tensor[:held] for field, tensor in rows.items()}
 
-    def gather(self, request_id: str, run: int) -> tuple[int, torch.Tensor, torch.Tensor]:
+    def iter_pages(self, request_id: str, run: int, name: str | None = None):
+        """`iter_page_fields` for keys and values: yields (first position, keys [n, kv_heads, head_dim],
+        values [n, kv_heads, head_dim])."""
+        for first, rows in self.iter_page_fields(request_id, run, name):
+            yield first, rows["keys"], rows["values"]
+
+    def gather_fields(self, request_id: str, run: int, name: str | None = None) -> tuple[int, dict[str, torch.Tensor]]:
+        """(first cached position, {field: [n, ...]}) of the request in run `run`, each field one contiguous tensor."""
+        pages = list(self.iter_page_fields(request_id, run, name))
+        if not pages:
+            return self.sequences[request_id].length, {}
+        return pages[0][0], {field: torch.cat([rows[field] for _, rows in pages]) for field in pages[0][1]}
+
+    def gather(self, request_id: str, run: int, name: str | None = None) -> tuple[int, torch.Tensor, torch.Tensor]:
         """(first cached position, keys, values) of the request in run `run` as two contiguous tensors
         [n, kv_heads, head_dim] (`kv_cache.py:318-342`)."""
-        pages = list(self.iter_pages(request_id, run))
-        if not pages:
-            need = self._paged_cell(run)[0].need
+        first, fields = self.gather_fields(request_id, run, name)
+        if not fields:
+            need = self._paged_cell(run, name)[0].need
             empty = torch.empty((0, need.num_kv_heads, need.head_dim), dtype=self.dtype, device=self.device)
-            return self.sequences[request_id].length, empty, empty.clone()
-        return pages[0][0], torch.cat([keys for _, keys, _ in pages]), torch.cat([values for _, _, values in pages])
+            return first, empty, empty.clone()
+        return first, fields["keys"], fields["values"]
 
     def block_table_tensors(self, request_ids: list[str], group: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
         """A compact [requests, widest] block table (-1 where nothing is held) and the requests'

@@ -385,21 +385,37 @@ extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const float* t
   return LAUNCH_STATUS();
 }
 
-// ---------------------------------------------------------------------------- SiLU(gate) * up
+// ---------------------------------------------------------------------------- act(gate) * up
 // in: [rows, 2 * width] float32 or bfloat16 with gate_j at column 2j and up_j at column 2j + 1 (the
 // product that made it had its weight rows interleaved); out: [rows, width].
-// silu(z) = z * sigmoid(z)  (reference model.py:188).
+// The activation is a parameter: 0 silu(z) = z * sigmoid(z) (reference model.py:188), 1 gelu (the exact one,
+// z * Phi(z)), 2 gelu with tanh, 3 relu.  The products' fused epilogues know silu alone; a feed-forward with
+// another gate activation runs its product plain and this kernel behind it.
+#define ACT_SILU 0
+#define ACT_GELU 1
+#define ACT_GELU_TANH 2
+#define ACT_RELU 3
+
+__device__ __forceinline__ float gate_activation(int activation, float z) {
+  switch (activation) {
+    case ACT_GELU: return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+    case ACT_GELU_TANH: return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    case ACT_RELU: return fmaxf(z, 0.f);
+    default: return z / (1.f + expf(-z));
+  }
+}
+
 template <typename TI, typename TO>
-__global__ void silu_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out, int width) {
+__global__ void gate_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out, int width, int activation) {
   const TI* row = in + (size_t)blockIdx.x * 2 * width;
   TO* dst = out + (size_t)blockIdx.x * width;
   for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x) {
     const float gate = to_float(row[2 * i]), up = to_float(row[2 * i + 1]);
-    dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+    dst[i] = from_float<TO>(gate_activation(activation, gate) * up);
   }
 }
 
-// The same for bfloat16 rows whose width is a multiple of 8: a thread takes eight outputs, 32 bytes in
+// SiLU for bfloat16 rows whose width is a multiple of 8: a thread takes eight outputs, 32 bytes in
 // (two 16-byte loads, both on their way before the first is used) and 16 bytes out.
 __global__ __launch_bounds__(256) void silu_mul_vector_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out,
                                                               size_t octets) {
@@ -418,10 +434,11 @@ __global__ __launch_bounds__(256) void silu_mul_vector_kernel(const bf16_t* __re
   ((bf16x8*)out)[at] = result;
 }
 
-extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
-                                 hipStream_t stream) {
+extern "C" int llmserve_gate_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
+                                 int activation, hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (!in_is_float && !out_is_float && width % 8 == 0) {  // rows are contiguous: the whole is one run of octets
+  if (activation < ACT_SILU || activation > ACT_RELU) return ERR_BAD_ARGUMENT;
+  if (activation == ACT_SILU && !in_is_float && !out_is_float && width % 8 == 0) {  // rows are contiguous: one run of octets
     const size_t octets = (size_t)rows * (width / 8);
     hipLaunchKernelGGL(silu_mul_vector_kernel, dim3((unsigned)((octets + 255) / 256)), dim3(256), 0, stream,
                        (const bf16_t*)in, (bf16_t*)out, octets);
@@ -431,14 +448,19 @@ extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int
   const int pieces = rows >= 1024 ? 1 : max(1, min((width + 255) / 256, 1024 / rows));
   const dim3 grid(rows, pieces), block(256);
   if (in_is_float && out_is_float)
-    hipLaunchKernelGGL((silu_mul_kernel<float, float>), grid, block, 0, stream, (const float*)in, (float*)out, width);
+    hipLaunchKernelGGL((gate_mul_kernel<float, float>), grid, block, 0, stream, (const float*)in, (float*)out, width, activation);
   else if (in_is_float)
-    hipLaunchKernelGGL((silu_mul_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)in, (bf16_t*)out, width);
+    hipLaunchKernelGGL((gate_mul_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)in, (bf16_t*)out, width, activation);
   else if (out_is_float)
-    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)in, (float*)out, width);
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)in, (float*)out, width, activation);
   else
-    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, width);
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, width, activation);
   return LAUNCH_STATUS();
+}
+
+extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
+                                 hipStream_t stream) {
+  return llmserve_gate_mul(in, in_is_float, out, out_is_float, rows, width, ACT_SILU, stream);
 }
 
 // ---------------------------------------------------------------------------- gather rows

@@ -18,6 +18,8 @@ import torch
 from .build import _say, load_module
 
 _PAIRINGS = {"none": 0, "adjacent": 1, "half": 2}
+# gate activations of a gated product (csrc/elementwise.hip: gate_activation); the products' fused epilogues know silu alone
+_ACTIVATIONS = {"silu": 0, "gelu": 1, "gelu_tanh": 2, "relu": 3}
 
 
 class KernelError(RuntimeError):
@@ -49,6 +51,7 @@ _SIGNATURES = {
     "llmserve_rotary_table": "pppiip",
     "llmserve_rotate_and_store": "pipiiiiipppip",
     "llmserve_silu_mul": "pipiiip",
+    "llmserve_gate_mul": "pipiiiip",
     "llmserve_gather_rows": "ppiippiip",
     "llmserve_gemm_generic": "pipipipiiiip",
     "llmserve_gemm_f32": "ppppiiiiip",
@@ -112,6 +115,7 @@ class GatedLinearWeights:
 
     both: LinearWeights
     width: int
+    activation: str = "silu"
 
 
 class HipKernels:
@@ -294,13 +298,17 @@ class HipKernels:
             bias = torch.cat(list(biases), dim=0).contiguous() if len(biases) > 1 else biases[0].contiguous()
         return LinearWeights(weight, bias)
 
-    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor) -> GatedLinearWeights:
+    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu") -> GatedLinearWeights:
+        """`activation` is the gate's: silu is applied in the epilogue of the product itself; the others
+        (gelu, gelu_tanh, relu) by a kernel of their own behind a plain product."""
+        if activation not in _ACTIVATIONS:
+            raise KernelError(f"gated_linear: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
         if gate.shape != up.shape:
             raise KernelError("gated_linear: gate and up differ in shape")
         if gate.dtype != up.dtype:
             gate, up = gate.float(), up.float()
         both = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
-        return GatedLinearWeights(LinearWeights(both, None), gate.shape[0])
+        return GatedLinearWeights(LinearWeights(both, None), gate.shape[0], activation)
 
     def _streaming(self, x: torch.Tensor, weights: LinearWeights, gated: bool = False) -> str | None:
         """Which MFMA kernel takes this product: "skinny" (up to 16 rows of x, weights streamed),
@@ -532,6 +540,14 @@ class HipKernels:
 
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
         out = self._empty((x.shape[0], weights.width), self.dtype)
+        if weights.activation != "silu":  # no fused epilogue: the product plain, the activation behind it
+            both = self.linear(x, weights.both, out_dtype=torch.bfloat16 if self._library(x, weights.both) else torch.float32)
+            status = self._elementwise.llmserve_gate_mul(
+                _pointer(both), _is_float(both), _pointer(out), _is_float(out), x.shape[0], weights.width,
+                _ACTIVATIONS[weights.activation], self._stream,
+            )
+            _check(status, "gate_mul")
+            return out
         if self._all_float32(x, weights.both) and self.dtype == torch.float32:
             status = self._gemm_f32.llmserve_gemm_f32(
                 _pointer(x), _pointer(weights.both.weight), None, _pointer(out), 1, x.shape[0], 2 * weights.width,

@@ -34,7 +34,9 @@ class Kernels(Protocol):
     def prepare_linear(self, weights: list[torch.Tensor], biases: list[torch.Tensor] | None) -> Any:
         """Concatenates [N_i, K] weights (and biases) along N into whatever layout `linear` wants."""
 
-    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor) -> Any: ...
+    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu") -> Any:
+        """Gate and up weights [I, K] in whatever layout `gated_linear` wants; `activation` is the gate's
+        (silu, gelu, gelu_tanh, relu), and one the library has no kernel for is refused here, by name."""
 
     def linear(
         self, x: torch.Tensor, weights: Any, out_dtype: torch.dtype | None = None, *, partial: bool = False
@@ -43,7 +45,7 @@ class Kernels(Protocol):
         `partial`, a float32 result may be [parts, T, N] partial sums for the reader to add."""
 
     def gated_linear(self, x: torch.Tensor, weights: Any) -> torch.Tensor:
-        """silu(x Wg^T) * (x Wu^T) -> [T, I] in the run dtype."""
+        """act(x Wg^T) * (x Wu^T) -> [T, I] in the run dtype."""
 
     def rotate_and_store(
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any,

@@ -5,8 +5,11 @@ from .base import (
     MIXERS,
     NORMS,
     POSITIONS,
+    CacheNeed,
     FixedState,
     PagedKeyValue,
+    PagedNeed,
+    SlotNeed,
     Part,
     Registry,
     STREAM_PARTS,

@@ -31,26 +31,79 @@ class TensorSpec:
     integer: bool = False
 
 
+KEY_PIECE = 8  # elements of a key that stay together in a page (csrc/common.h has the same number)
+
+
+def key_piece_width(head_dim: int) -> int:
+    """A key is kept in pieces of KEY_PIECE elements; a head size that is no multiple of it in one piece."""
+    return KEY_PIECE if head_dim % KEY_PIECE == 0 else head_dim
+
+
+class CacheNeed:
+    """What a part keeps in the cache from one step to the next.  The cache manager knows two ways of
+    giving room, and a need is of one of them: `PagedNeed` (an entry per token, in pages that a request
+    holds through a block table) or `SlotNeed` (one entry of fixed size per request).  What an entry *is*
+    is the need's own business: a new kind of need is a subclass that says what a page of it holds, and
+    nothing in the cache manager, the step function or the scheduler changes.  Needs are compared and
+    hashed (frozen dataclasses): runs with equal paged needs share a pool and a block table per request."""
+
+
+class PagedNeed(CacheNeed):
+    """An entry per token.  A subclass has a field `window` (keys at most that are ever read again, None:
+    all) and says what one page holds."""
+
+    window: int | None = None
+
+    def page_fields(self, page_size: int) -> dict[str, tuple[int, ...]]:
+        """name -> shape of ONE page of that field.  The cache keeps each field as a tensor
+        [pages, *shape] in the run dtype, and a `CacheCell` shows them by these names."""
+        raise NotImplementedError
+
+    def token_rows(self, page: dict[str, torch.Tensor], page_size: int) -> dict[str, torch.Tensor]:
+        """One page's fields rearranged so that the token's offset in the page leads: name ->
+        [page_size, ...].  The host-side read path (tests, debugging) walks pages through it; kernels
+        read the pages as they lie."""
+        raise NotImplementedError
+
+
+class SlotNeed(CacheNeed):
+    """One entry of fixed size per request.  A subclass has a field `shape`: the cache keeps a float32
+    tensor [request slots, *shape], zeroed when a request takes its slot."""
+
+    shape: tuple[int, ...] = ()
+
+
 @dataclass(frozen=True)
-class PagedKeyValue:
-    """Cache need of a mixer that keeps a key and a value per token in pages.
-    Layers with equal needs share a group (one page pool, one block table per
-    request).  `window` keys at most are ever read again; None means all."""
+class PagedKeyValue(PagedNeed):
+    """Cache need of a mixer that keeps a key and a value per token in pages.  Keys lie in pieces of
+    eight elements, the same piece of all the keys of a page side by side ([kv_heads, head_dim / w,
+    page_size, w], w = `key_piece_width(head_dim)`): the matrix cores take keys as rows, a lane holding
+    one piece of one key and its neighbours that piece of the next keys, and neighbouring lanes should
+    read neighbouring bytes.  Values are stored transposed ([kv_heads, head_dim, page_size]): attention
+    sums over keys, and the matrix cores want the summed index contiguous."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
 
+    def page_fields(self, page_size: int) -> dict[str, tuple[int, ...]]:
+        width = key_piece_width(self.head_dim)
+        return {
+            "keys": (self.num_kv_heads, self.head_dim // width, page_size, width),
+            "values": (self.num_kv_heads, self.head_dim, page_size),
+        }
+
+    def token_rows(self, page: dict[str, torch.Tensor], page_size: int) -> dict[str, torch.Tensor]:
+        keys = page["keys"].permute(2, 0, 1, 3).reshape(page_size, self.num_kv_heads, self.head_dim)
+        return {"keys": keys, "values": page["values"].permute(2, 0, 1)}
+
 
 @dataclass(frozen=True)
-class FixedState:
+class FixedState(SlotNeed):
     """Cache need of a mixer that keeps a state of fixed size per request: one
     slot of `shape` float32 values, zeroed when the request is created."""
 
     shape: tuple[int, ...]
-
-
-CacheNeed = PagedKeyValue | FixedState | None
 
 
 class Part:
@@ -68,7 +121,10 @@ class Part:
         return {}
 
     @classmethod
-    def cache_need(cls, spec: Any) -> CacheNeed:
+    def cache_need(cls, spec: Any) -> "CacheNeed | dict[str, CacheNeed] | None":
+        """What the part keeps in the cache: nothing, one need, or several by name (a block with two
+        mixers side by side, one with pages and one with a state): its cell is then a dict of cells
+        by the same names."""
         return None
 
     def __init__(self, spec: Any, tensors: dict[str, torch.Tensor], kernels: Any) -> None:
@@ -106,7 +162,7 @@ class Registry:
     def tensors(self, spec: Any) -> dict[str, TensorSpec]:
         return self.get(spec).tensors(spec)
 
-    def cache_need(self, spec: Any) -> CacheNeed:
+    def cache_need(self, spec: Any) -> "CacheNeed | dict[str, CacheNeed] | None":
         return self.get(spec).cache_need(spec)
 
     def build(self, spec: Any, tensors: dict[str, torch.Tensor], kernels: Any) -> Part:

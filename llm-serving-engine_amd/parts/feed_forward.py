@@ -41,10 +41,9 @@ class GatedMLP(FeedForward):
 
     def __init__(self, spec: GatedMLPSpec, tensors, kernels) -> None:
         super().__init__(spec, tensors, kernels)
-        if spec.activation != "silu":
-            raise ValueError(f"gated_mlp: activation {spec.activation!r} has no kernel")
+        # the kernel library says which activations it has, and refuses another by name
         self.gate_up = kernels.prepare_gated_linear(
-            tensors["gate_proj.weight"], tensors["up_proj.weight"]
+            tensors["gate_proj.weight"], tensors["up_proj.weight"], spec.activation
         )
         self.down = kernels.prepare_linear([tensors["down_proj.weight"]], None)
 

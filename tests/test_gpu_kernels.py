@@ -818,3 +818,22 @@ def test_rotation_store_and_attention_of_prompt_portions(kernels, dtype, pairing
     want_v = torch.cat([rounded(v, dtype)[-count:] for (q, k, v), count in zip(originals, counts)])
     torch.testing.assert_close(stored_k, want_k, **TOLERANCE[dtype])
     torch.testing.assert_close(stored_v, want_v, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("activation", ["silu", "gelu", "gelu_tanh", "relu"])
+@pytest.mark.parametrize("rows,inner,outer", [(5, 96, 200), (70, 64, 333), (300, 128, 1000)])
+def test_gated_products_with_every_gate_activation(kernels, dtype, activation, rows, inner, outer):
+    """The gate's activation is a parameter of the gated product: SiLU is applied in the products' own epilogues,
+    the others by the activation kernel behind a plain product; one that has no kernel is refused by name."""
+    k = kernels[dtype]
+    acts = {"silu": F.silu, "gelu": F.gelu, "gelu_tanh": lambda z: F.gelu(z, approximate="tanh"), "relu": torch.relu}
+    x, gate, up = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer, inner) / math.sqrt(inner)
+    weights = k.prepare_gated_linear(on_gpu(gate, dtype), on_gpu(up, dtype), activation)
+    out = k.gated_linear(on_gpu(x, dtype), weights)
+    want = acts[activation](rounded(x, dtype) @ rounded(gate, dtype).T) * (rounded(x, dtype) @ rounded(up, dtype).T)
+    torch.testing.assert_close(out.cpu().double(), want, **TOLERANCE[dtype])
+    from llmserve_amd.kernels.hip import KernelError
+
+    with pytest.raises(KernelError, match="swish7"):
+        k.prepare_gated_linear(on_gpu(gate, dtype), on_gpu(up, dtype), "swish7")

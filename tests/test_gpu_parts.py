@@ -179,6 +179,40 @@ def test_a_stateful_architecture_is_captured_and_replayed(tmp_path, kernels):
         toy.unregister_toy()
 
 
+def test_cache_needs_of_a_kind_of_their_own_on_the_gpu(tmp_path, kernels):
+    """The third toy architecture on the GPU, in both precisions: pages of a kind of need that the cache manager
+    has never heard of (a narrow key row and a wider value row per token), a run that holds pages and a state
+    slot at once, and a feed-forward whose gate is a gelu (a plain product and the activation kernel behind
+    it); three requests in changing portions against the plain forward, and the pages against its rows."""
+    from tests.test_toy_parts import step_in_portions
+
+    toy.register_toy()
+    try:
+        folder = toy.write_toy_folder(tmp_path / "latent", config=toy.LATENT)
+        prompts = {name: random_tokens(n, toy.LATENT.vocab_size, seed=n) for name, n in (("a", 37), ("b", 9), ("c", 22))}
+        expected = {name: toy.plain_toy_forward(folder, tokens, with_cached_rows=True) for name, tokens in prompts.items()}
+        spread = float(torch.cat([logits for logits, _ in expected.values()]).std())
+        for dtype in DTYPES:
+            loaded = load_model_folder(folder, "float32" if dtype == torch.float32 else "bfloat16")
+            runner = ModelRunner(loaded, kernels[dtype], CacheConfig(block_size=4, num_blocks=20, max_sequences=3))
+            assert not runner.use_graphs and len(runner.cache.groups) == 2 and len(runner.cache.states) == 1
+            got = step_in_portions(runner, prompts, {"a": [5, 1, 1, 9, 2, 19], "b": [2, 7], "c": [1, 1, 1, 1, 18]})
+            bound = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=0.06 * spread, rtol=3e-2)
+            for name in prompts:
+                torch.testing.assert_close(got[name].cpu().double(), expected[name][0], **bound)
+                first, rows = runner.cache.gather_fields(name, 0)
+                stored = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+                torch.testing.assert_close(rows["key_rows"].cpu().double(), expected[name][1][0], **stored)
+                torch.testing.assert_close(rows["value_rows"].cpu().double(), expected[name][1][1], **stored)
+            for name in prompts:
+                runner.end_request(name)
+            runner.cache.check_invariants()
+            assert runner.cache.used_pages == 0
+            runner.close()
+    finally:
+        toy.unregister_toy()
+
+
 # ------------------------------------------------------------------------------- entry points
 
 

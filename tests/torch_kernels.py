@@ -46,8 +46,12 @@ class TorchKernels:
         bias = torch.cat([b.float() for b in biases], dim=0) if biases else None
         return _Linear(weight, bias)
 
-    def prepare_gated_linear(self, gate, up):
-        return (_Linear(gate.float(), None), _Linear(up.float(), None))
+    def prepare_gated_linear(self, gate, up, activation="silu"):
+        acts = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu": torch.relu,
+                "gelu_tanh": lambda z: torch.nn.functional.gelu(z, approximate="tanh")}
+        if activation not in acts:
+            raise ValueError(f"gated_linear: no activation {activation!r}")
+        return (_Linear(gate.float(), None), _Linear(up.float(), None), acts[activation])
 
     def linear(self, x, weights, out_dtype=None, partial=False):
         y = x.float() @ weights.weight.T
@@ -58,7 +62,7 @@ class TorchKernels:
     def gated_linear(self, x, weights):
         gate = x.float() @ weights[0].weight.T
         up = x.float() @ weights[1].weight.T
-        return (gate * torch.sigmoid(gate) * up).to(self.dtype)
+        return (weights[2](gate) * up).to(self.dtype)
 
     def rotate_and_store(self, qkv, layout, batch, cell, inverse_frequencies, pairing):
         tokens = qkv.shape[0]

@@ -11,7 +11,11 @@ architectures are added by registering them, without a change to the framework's
 - and a second architecture all of whose parts are the same kernel launches whatever the data, among them a
   mixer with state of its own that runs on the device alone: its steps are captured into graphs and replayed;
   it also has a part between the embedding and the first layer (a learned table of absolute positions, and a
-  scale) and one after the head (a bias and a soft cap on the logits).
+  scale) and one after the head (a bias and a soft cap on the logits);
+- and a third whose cache needs are its own: a mixer that keeps one narrow key row and one wider value row per
+  token in pages (a kind of need defined here, with its own page layout), a block with attention and the
+  decaying mixer side by side (pages *and* a state slot for one run), and a feed-forward whose gate has
+  another activation.
 
 It is never a model of anyone's: it exists to exercise the interfaces."""
 
@@ -27,10 +31,11 @@ import torch
 
 from llmserve_amd.config.model import ArchitectureConfig, KeyReader
 from llmserve_amd.parts import (
-    FEED_FORWARDS, LOGIT_PARTS, MIXERS, POSITIONS, STREAM_PARTS, AttentionSpec, FeedForward, FixedState, GatedMLPSpec,
-    LayerDefinition, LayerRun, Mixer, ModelSpec, NamedPart, NoPositionSpec, Part, PositionEncoding, PreNormBlockSpec,
-    RMSNormSpec, RotarySpec, TensorSpec,
+    BLOCKS, FEED_FORWARDS, LOGIT_PARTS, MIXERS, NORMS, POSITIONS, STREAM_PARTS, AttentionSpec, Block, FeedForward, FixedState,
+    GatedMLPSpec, LayerDefinition, LayerRun, Mixer, ModelSpec, NamedPart, NoPositionSpec, PagedNeed, Part, PositionEncoding,
+    PreNormBlockSpec, RMSNormSpec, RotarySpec, TensorSpec,
 )
+from llmserve_amd.parts.base import prefixed, under
 from llmserve_amd.registry import register_architecture, unregister_architecture
 
 
@@ -221,6 +226,125 @@ class RunningSumMixer(Mixer):
 
 
 @dataclass(frozen=True)
+class PagedRows(PagedNeed):
+    """A cache need of this file's own: per token one key row and one value row of another width, each page
+    holding its tokens' rows one after the other.  The cache manager has never heard of it."""
+
+    key_width: int
+    value_width: int
+    window: int | None = None
+
+    def page_fields(self, page_size: int) -> dict[str, tuple[int, ...]]:
+        return {"key_rows": (page_size, self.key_width), "value_rows": (page_size, self.value_width)}
+
+    def token_rows(self, page: dict[str, torch.Tensor], page_size: int) -> dict[str, torch.Tensor]:
+        return dict(page)  # the token's place in the page leads already
+
+
+@dataclass(frozen=True)
+class LatentSpec:
+    hidden_size: int
+    key_width: int
+    value_width: int
+    kind: str = "toy_latent"
+
+
+class LatentMixer(Mixer):
+    """One head of attention over narrow keys and wider values: q = x Wq, k = x Wk (key_width), v = x Wv
+    (value_width); softmax(q . k / sqrt(key_width)) over the keys up to the token's own; out = (.) Wo.  What it
+    caches per token is a `PagedRows` entry, written and read here through the step's slot mapping and block
+    tables with plain tensor indexing."""
+
+    replayable = False  # a loop on the host over the step's requests
+
+    @classmethod
+    def tensors(cls, spec: LatentSpec) -> dict[str, TensorSpec]:
+        return {
+            "q_proj.weight": TensorSpec((spec.key_width, spec.hidden_size)),
+            "k_proj.weight": TensorSpec((spec.key_width, spec.hidden_size)),
+            "v_proj.weight": TensorSpec((spec.value_width, spec.hidden_size)),
+            "o_proj.weight": TensorSpec((spec.hidden_size, spec.value_width)),
+        }
+
+    @classmethod
+    def cache_need(cls, spec: LatentSpec) -> PagedRows:
+        return PagedRows(spec.key_width, spec.value_width)
+
+    def __init__(self, spec: LatentSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.w = {name.split(".")[0]: value.float() for name, value in tensors.items()}
+
+    def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
+        x = x.float()
+        q, k, v = x @ self.w["q_proj"].T, x @ self.w["k_proj"].T, x @ self.w["v_proj"].T
+        group = batch.groups[cell.group]
+        key_pages, value_pages = cell.fields["key_rows"], cell.fields["value_rows"]
+        page_size = group.page_size
+        if cell.writable:
+            slots = group.slot_mapping.long()
+            key_pages[slots // page_size, slots % page_size] = k.to(key_pages.dtype)
+            value_pages[slots // page_size, slots % page_size] = v.to(value_pages.dtype)
+        out = torch.empty(x.shape[0], self.spec.hidden_size, dtype=torch.float32, device=x.device)
+        row = 0
+        for index, chunk in enumerate(batch.chunks):
+            context = chunk.start + chunk.count
+            table = group.block_tables[index, : -(-context // page_size)].long()
+            keys = key_pages[table].reshape(-1, self.spec.key_width)[:context].float()
+            values = value_pages[table].reshape(-1, self.spec.value_width)[:context].float()
+            scores = q[row : row + chunk.count] @ keys.T / math.sqrt(self.spec.key_width)
+            position = torch.arange(chunk.start, context, device=x.device).unsqueeze(1)
+            scores = scores.masked_fill(torch.arange(context, device=x.device).unsqueeze(0) > position, float("-inf"))
+            out[row : row + chunk.count] = (torch.softmax(scores, dim=-1) @ values) @ self.w["o_proj"].T
+            row += chunk.count
+        return out
+
+
+@dataclass(frozen=True)
+class SideBySideBlockSpec:
+    """h += attention(norm(h)) + decay(norm(h)); h += feed_forward(norm(h))."""
+
+    norm: Any
+    attention: Any
+    decay: Any
+    feed_forward_norm: Any
+    feed_forward: Any
+    kind: str = "toy_side_by_side"
+
+
+class SideBySideBlock(Block):
+    """Two mixers read the same normed rows and their results are added: one keeps keys and values in pages, the
+    other a state per request, so one run of the layer needs both, by name."""
+
+    _MEMBERS = (("input_layernorm.", NORMS, "norm"), ("attention.", MIXERS, "attention"), ("decay.", MIXERS, "decay"),
+                ("post_attention_layernorm.", NORMS, "feed_forward_norm"), ("mlp.", FEED_FORWARDS, "feed_forward"))
+
+    @classmethod
+    def tensors(cls, spec: SideBySideBlockSpec) -> dict[str, TensorSpec]:
+        found: dict[str, TensorSpec] = {}
+        for name, registry, field in cls._MEMBERS:
+            found.update(prefixed(registry.tensors(getattr(spec, field)), name))
+        return found
+
+    @classmethod
+    def cache_need(cls, spec: SideBySideBlockSpec):
+        return {"attention": MIXERS.cache_need(spec.attention), "decay": MIXERS.cache_need(spec.decay)}
+
+    def __init__(self, spec: SideBySideBlockSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        for name, registry, field in self._MEMBERS:
+            setattr(self, field, registry.build(getattr(spec, field), under(tensors, name), kernels))
+        self.replayable = False
+
+    def forward(self, hidden, delta, batch, cell) -> torch.Tensor:
+        normed = self.norm.forward(hidden, delta)
+        attended = self.attention.forward(normed, batch, cell["attention"])
+        attended = attended if attended.ndim == 2 else attended.sum(0)
+        mixed = attended + self.decay.forward(normed, batch, cell["decay"])
+        normed = self.feed_forward_norm.forward(hidden, mixed)
+        return self.feed_forward.forward(normed, batch)
+
+
+@dataclass(frozen=True)
 class AbsolutePositionsSpec:
     hidden_size: int
     max_length: int
@@ -363,11 +487,42 @@ class SumConfig(ToyConfig):
     architecture: ClassVar[str] = "ToySumForCausalLM"
 
 
+LATENT_KEY_WIDTH, LATENT_VALUE_WIDTH, LATENT_ACTIVATION = 12, 28, "gelu_tanh"
+
+
+def latent_spec(config: ToyConfig) -> ModelSpec:
+    """The third architecture: the latent mixer with a feed-forward whose gate is a gelu, then a block with
+    attention and the decaying mixer side by side, then the first layer again (a second cell in its group)."""
+    norm = RMSNormSpec(config.hidden_size, config.eps)
+    gelu_ffn = GatedMLPSpec(config.hidden_size, config.ffn_size, activation=LATENT_ACTIVATION)
+    ffn = GatedMLPSpec(config.hidden_size, config.ffn_size)
+    latent = LatentSpec(config.hidden_size, LATENT_KEY_WIDTH, LATENT_VALUE_WIDTH)
+    decay = DecaySpec(config.hidden_size, config.state_size, config.decay)
+    attention = AttentionSpec(
+        config.hidden_size, config.num_heads, config.num_heads, config.head_dim, 1.0 / math.sqrt(config.head_dim),
+        RotarySpec(config.head_dim, 100.0, "half"), qkv_bias=False,
+    )
+    layers = (
+        LayerDefinition("layers.0.", PreNormBlockSpec(norm, latent, norm, gelu_ffn, mixer_name="mixer.")),
+        LayerDefinition("layers.1.", SideBySideBlockSpec(norm, attention, decay, norm, ffn)),
+    )
+    return ModelSpec(
+        config.vocab_size, config.hidden_size, layers, (LayerRun(0), LayerRun(1), LayerRun(0)), norm, tie_embeddings=True,
+        embedding_name="embed.weight", final_norm_name="final_norm.",
+    )
+
+
+@dataclass(frozen=True)
+class LatentConfig(ToyConfig):
+    architecture: ClassVar[str] = "ToyLatentForCausalLM"
+
+
 TOY = ToyConfig(vocab_size=97, hidden_size=48, state_size=20, decay=0.8, num_heads=3, head_dim=16, ffn_size=64,
                 eps=1e-5, max_length=256, experts=5, experts_chosen=2, expert_size=24)
 
 
 SUM = SumConfig(**TOY.to_dict())
+LATENT = LatentConfig(**TOY.to_dict())
 
 
 def register_toy() -> None:
@@ -380,6 +535,9 @@ def register_toy() -> None:
     LOGIT_PARTS.register("toy_capped_logits")(CappedLogits)
     register_architecture("ToyStateForCausalLM", ToyConfig, toy_spec)
     register_architecture("ToySumForCausalLM", SumConfig, sum_spec)
+    MIXERS.register("toy_latent")(LatentMixer)
+    BLOCKS.register("toy_side_by_side")(SideBySideBlock)
+    register_architecture("ToyLatentForCausalLM", LatentConfig, latent_spec)
 
 
 def unregister_toy() -> None:
@@ -392,6 +550,9 @@ def unregister_toy() -> None:
     LOGIT_PARTS.unregister("toy_capped_logits")
     unregister_architecture("ToyStateForCausalLM")
     unregister_architecture("ToySumForCausalLM")
+    MIXERS.unregister("toy_latent")
+    BLOCKS.unregister("toy_side_by_side")
+    unregister_architecture("ToyLatentForCausalLM")
 
 
 def write_toy_folder(folder: Path, seed: int = 3, config: ToyConfig = TOY) -> Path:
@@ -403,8 +564,9 @@ def write_toy_folder(folder: Path, seed: int = 3, config: ToyConfig = TOY) -> Pa
 # ----------------------------------------------------------------------------- the toy's own plain forward
 
 
-def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
-    """Whole sequence, no cache, float64; written apart from the parts above."""
+def plain_toy_forward(folder: Path, tokens: list[int], with_cached_rows: bool = False) -> torch.Tensor:
+    """Whole sequence, no cache, float64; written apart from the parts above.  `with_cached_rows` (the third
+    architecture): also the key and value rows that its first run would cache."""
     from safetensors.torch import load_file
 
     from tests.plain import qwen2_plain as plain
@@ -478,6 +640,41 @@ def plain_toy_forward(folder: Path, tokens: list[int]) -> torch.Tensor:
         h = h + ffn(plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps), prefix)
         return h, (k, v)
 
+    def latent_layer(h, prefix):
+        """One head over narrow keys and wider values, then a feed-forward whose gate is a gelu (tanh form).
+        Returns the layer's output and the rows it would cache."""
+        x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
+        q, k, v = (x @ w[prefix + f"mixer.{name}_proj.weight"].T for name in "qkv")
+        scores = (q @ k.T) / math.sqrt(LATENT_KEY_WIDTH)
+        scores = scores.masked_fill(torch.arange(length).unsqueeze(0) > torch.arange(length).unsqueeze(1), float("-inf"))
+        h = h + (torch.softmax(scores, dim=-1) @ v) @ w[prefix + "mixer.o_proj.weight"].T
+        x = plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps)
+        gate = torch.nn.functional.gelu(x @ w[prefix + "mlp.gate_proj.weight"].T, approximate="tanh")
+        return h + (gate * (x @ w[prefix + "mlp.up_proj.weight"].T)) @ w[prefix + "mlp.down_proj.weight"].T, (k, v)
+
+    def side_by_side_layer(h, prefix):
+        x = plain.rms_norm(h, w[prefix + "input_layernorm.weight"], eps)
+        q = (x @ w[prefix + "attention.q_proj.weight"].T).view(length, heads, dim)
+        k = (x @ w[prefix + "attention.k_proj.weight"].T).view(length, heads, dim)
+        v = (x @ w[prefix + "attention.v_proj.weight"].T).view(length, heads, dim)
+        angles = plain.rope_angles(dim, 100.0, torch.arange(length))
+        q, k = plain.rope_half(q, angles), plain.rope_half(k, angles)
+        mixed = plain.causal_attention(q, k, v, 1.0 / math.sqrt(dim)).reshape(length, -1) @ w[prefix + "attention.o_proj.weight"].T
+        state = torch.zeros(config["state_size"], dtype=torch.float64)
+        decayed = []
+        for t in range(length):
+            state = config["decay"] * state + w[prefix + "decay.in_proj.weight"] @ x[t]
+            decayed.append(w[prefix + "decay.out_proj.weight"] @ state)
+        h = h + mixed + torch.stack(decayed)
+        x = plain.rms_norm(h, w[prefix + "post_attention_layernorm.weight"], eps)
+        return h + plain.swiglu(x, w[prefix + "mlp.gate_proj.weight"], w[prefix + "mlp.up_proj.weight"], w[prefix + "mlp.down_proj.weight"])
+
+    if config["architectures"] == ["ToyLatentForCausalLM"]:
+        h, first_rows = latent_layer(h, "layers.0.")
+        h = side_by_side_layer(h, "layers.1.")
+        h, _ = latent_layer(h, "layers.0.")
+        logits = plain.rms_norm(h, w["final_norm.weight"], eps) @ w["embed.weight"].T
+        return (logits, first_rows) if with_cached_rows else logits
     if config["architectures"] == ["ToySumForCausalLM"]:
         h = h * EMBEDDING_SCALE + w["positions.table"][:length]
         h = sum_layer(h, "layers.0.")
