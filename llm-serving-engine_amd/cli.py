@@ -54,6 +54,12 @@ def _engine(args, loaded, tokenizer, *, batch_size: int, mode: str):
     from .config import CacheConfig, SchedulerConfig
     from .engine import LLMEngine
 
+    kernels = None
+    if getattr(args, "own_products", False):  # every product on the hand-written kernels, none sent to the BLAS library
+        from .kernels import HipKernels
+        from .weights import run_dtype
+
+        kernels = HipKernels(run_dtype(args.dtype), args.device if args.device != "auto" else "cuda:0", library_products=False)
     return LLMEngine(
         loaded,
         tokenizer,
@@ -64,6 +70,7 @@ def _engine(args, loaded, tokenizer, *, batch_size: int, mode: str):
         collect_iteration_metrics=True,
         device=args.device if args.device != "auto" else "cuda:0",
         dtype=args.dtype,
+        kernels=kernels,
     )
 
 
@@ -147,6 +154,8 @@ def _replay(args) -> int:
     command = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", args.model, "--dtype", args.dtype, "--out",
                args.out, "--max-tokens", str(args.max_tokens), "--block-size", str(args.block_size),
                "--max-requests", str(args.max_requests)]
+    if args.own_products:
+        command.append("--own-products")
     return subprocess.call(command)
 
 
@@ -173,6 +182,8 @@ def _engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--max-tokens-per-step", type=int, default=2048)
     parser.add_argument("--policy", choices=("fcfs", "sjf", "priority"), default="fcfs")
     parser.add_argument("--seed", type=int, default=7)
+    parser.add_argument("--own-products", action="store_true",
+                        help="every matrix product on the engine's own kernels, none sent to the BLAS library")
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -206,6 +217,8 @@ def build_parser() -> argparse.ArgumentParser:
     replay.add_argument("--max-tokens", type=int, required=True)
     replay.add_argument("--block-size", type=int, default=16)
     replay.add_argument("--max-requests", type=int, default=8, help="most requests alive at a time")
+    replay.add_argument("--own-products", action="store_true",
+                        help="every matrix product on the engine's own kernels, none sent to the BLAS library")
 
     random_model = commands.add_parser("random-model", help="write a model folder with seeded random weights")
     random_model.add_argument("--config", required=True, help="a config.json")

@@ -121,16 +121,13 @@ class GatedLinearWeights:
 class HipKernels:
     def __init__(
         self, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0", *, library_products: bool = True,
-        shared_portions: str = "auto", wide_products: str = "never",
+        shared_portions: str = "auto",
     ) -> None:
-        """`library_products=False` keeps every product on the hand-written kernels.  `wide_products`:
-        which products of more than 64 rows leave the library for the hand-written 256 x 256 tile
-        although `library_products` is set: "never" (the default: inside a step neither is ahead, see
-        below), "partial" (float32 results that may stay partial sums over K, the down projection),
-        "gated" (those and gate/up with its fused SiLU * up).  Alone, the down projection of 2,048 rows
-        at the 1.5B sizes takes 60 us against the library's 67, but its five partial sums cost the
-        norm that adds them more than that; gate/up takes 150 us against the library's 120 + 18 for
-        SiLU * up.
+        """`library_products=False` keeps every product on the hand-written kernels (the command line's and
+        bench.py's --own-products): the weight-streaming ones up to 64 rows, the LDS-tiled ones above, with
+        their fused epilogues.  Inside a whole step the library is ahead for many rows (at 2,048 rows of the
+        1.5B sizes gate/up with its fused SiLU * up takes 150 us against the library's 120 + 18 for SiLU * up),
+        so it is the default there.
         `shared_portions`:
         whether prompt portions at head size 128 go to the attention kernel whose waves share K and V
         through LDS: "auto" (when the step's walks, taken together, are long beside the longest), "always", "never"."""
@@ -142,7 +139,6 @@ class HipKernels:
         self.device = torch.device(device)
         self.library_products = library_products
         self.shared_portions = shared_portions
-        self.wide_products = wide_products
         self.merge_in_product = True  # decode attention leaves its key splits to the product that reads them
         name = torch.cuda.get_device_properties(self.device).gcnArchName
         if not name.startswith("gfx950"):
@@ -401,12 +397,6 @@ class HipKernels:
             wanted //= 2
         return wanted
 
-    def _wide_applies(self, rows: int, out_features: int, in_features: int, splits: int) -> bool:
-        """Whether the tiled product would run its 256 x 256 tile: enough tiles for the chip, and
-        K a multiple of 32 of at least three steps."""
-        tiles = -(-rows // 256) * -(-out_features // 256) * splits
-        return tiles >= 200 and in_features % (32 * splits) == 0 and in_features // splits >= 96
-
     @staticmethod
     def _tiled_splits(rows: int, out_features: int, in_features: int) -> int:
         """Into how many parts of K the tiled product is cut when its float32 result may stay in
@@ -442,16 +432,6 @@ class HipKernels:
             # a long K over few weight rows (the down projection): cut over K into partial sums, the
             # hand-written kernel is ahead of the library (16 against 25 us at 64 rows of the 1.5B sizes)
             streaming = "medium"
-        if (
-            streaming is None
-            and partial
-            and out_dtype == torch.float32
-            and self.wide_products != "never"
-            and self._library(x, weights)
-            and rows > 64
-            and self._wide_applies(rows, weights.out_features, inner, self._tiled_splits(rows, weights.out_features, inner))
-        ):
-            streaming = "tiled"
         if streaming is None and self._library(x, weights):
             if (out_dtype or self.dtype) == torch.float32:  # float32 straight from the accumulators
                 cuts = self._library_splits(rows, weights.out_features, inner) if partial and bias is None else 1
@@ -556,14 +536,6 @@ class HipKernels:
             _check(status, "gated_linear")
             return out
         streaming = self._streaming(x, weights.both, gated=True)
-        if (
-            streaming is None
-            and self.wide_products == "gated"
-            and self._library(x, weights.both)
-            and x.shape[0] > 64
-            and self._wide_applies(x.shape[0], 2 * weights.width, x.shape[1], 1)
-        ):
-            streaming = "tiled"
         if streaming is not None:
             if streaming == "tiled":
                 status = self._gemm_bf16.llmserve_gemm_tiled(

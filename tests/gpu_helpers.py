@@ -14,10 +14,10 @@ ROOT = Path(__file__).resolve().parent.parent
 
 
 def replay(folder: Path, dtype: str, steps: list[dict], out: Path, max_tokens: int, block_size: int,
-           vocab: int) -> dict[int, torch.Tensor]:
+           vocab: int, extra: tuple[str, ...] = ()) -> dict[int, torch.Tensor]:
     """Runs bin/trace_run on `steps` and returns {step: logits [wanted, vocab]}."""
     command = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype, "--out",
-               str(out), "--max-tokens", str(max_tokens), "--block-size", str(block_size)]
+               str(out), "--max-tokens", str(max_tokens), "--block-size", str(block_size), *extra]
     text = "".join(json.dumps(step) + "\n" for step in steps)
     done = subprocess.run(command, input=text, capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, f"trace_run failed:\n{done.stderr[-3000:]}"

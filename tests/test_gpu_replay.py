@@ -129,19 +129,20 @@ def wide_models(tmp_path_factory):
     return get
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("sizes", ["1.5B", "7B", "32B"])
-def test_replay_at_benchmark_layer_sizes(wide_models, tmp_path, sizes, dtype):
+@pytest.mark.parametrize("sizes,dtype,own", [(sizes, dtype, False) for sizes in ("1.5B", "7B", "32B") for dtype in ("float32", "bfloat16")]
+                         + [("1.5B", "bfloat16", True)])
+def test_replay_at_benchmark_layer_sizes(wide_models, tmp_path, sizes, dtype, own):
     """The layer widths of the 1.5B, 7B and 32B configurations (head size 128; six, seven and five query
     heads a kv head), one or two layers of them: the same four ways of cutting, with prompts that cross many
-    pages and a pool that the three do not fit into together."""
+    pages and a pool that the three do not fit into together.  `own`: with every product on the engine's own
+    kernels (--own-products), none sent to the BLAS library."""
     WIDE = WIDE_CONFIGS[sizes][0]
     folder, plain_config, weights = wide_models(sizes)
     prompts = {f"p{n}": random_tokens(n, WIDE.vocab_size, seed=300 + n) for n in (3, 130, 290)}
     expected = {key: plain.forward(weights, plain_config, tokens) for key, tokens in prompts.items()}
     trace = build_trace(prompts, PAGE_WIDE, budget=512)
     results = replay(folder, dtype, trace.steps, tmp_path / "out", max_tokens=512, block_size=PAGE_WIDE,
-                     vocab=WIDE.vocab_size)
+                     vocab=WIDE.vocab_size, extra=("--own-products",) if own else ())
     # These logits spread five to ten times wider than the tiny models' (std 0.78 at width 1536, 1.4 at 5120), so
     # both bounds are stated in units of that spread.  bfloat16: each of the ten or so roundings of an activation
     # between kernels adds about 2^-9 of it, 0.6 % together; the largest of 1.7 million elements lies near five times
