@@ -2,8 +2,10 @@
 // and adds float32 as they stand), float32 pages.  Compiled once per head size (-DHEAD_DIM=..., a
 // multiple of 16).  It is the 32-bit path's attention for prompt portions and decoded tokens alike
 // (reference model.py:140-175 computes the same recurrence page by page); attention_generic.hip
-// remains for head sizes that are no multiple of 16, pages that are no multiple of 4, and scores with a
-// bias or a soft cap.
+// remains for head sizes that are no multiple of 16 and pages that are no multiple of 4.
+// Two things may change a score before the softmax, for position encodings and models that want them
+// (the reference has neither): `soft_cap` > 0 squashes it to cap * tanh(score / cap), and `slopes` (one
+// per query head) then adds -slope * (query position - key position).
 //
 // The unit of work is an item: up to 16 * COLUMN_TILES "columns", the (token, query head) pairs of
 // consecutive tokens of one request that share one kv head, running through the tokens head by head so
@@ -37,13 +39,14 @@ constexpr int WAVES = 4;
 __device__ __forceinline__ f32x4 load4(const float* p) { return *(const f32x4*)p; }
 
 // work[item] = {request index in the step, first token row, first head of that token, columns}
-template <int COLUMN_TILES>
+// CHANGED: the scores carry a soft cap or a distance bias (a variant of its own, so that the plain one pays nothing)
+template <int COLUMN_TILES, bool CHANGED>
 __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
     const float* __restrict__ qkv, int row_width, float* __restrict__ out, float* __restrict__ partial_acc,
     float* __restrict__ partial_ml, const float* __restrict__ keys, const float* __restrict__ values,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ positions,
     const int* __restrict__ work, int heads, int kv_heads, int page_size, float scale_log2, int window, int splits,
-    int columns_total) {
+    int columns_total, const float* __restrict__ slopes, float soft_cap) {
   __shared__ float wave_max[WAVES][COLUMN_TILES][16];
   __shared__ float wave_sum[WAVES][COLUMN_TILES][16];
   __shared__ __attribute__((aligned(16))) float merged[COLUMN_TILES][D_STEPS][64][4];
@@ -58,6 +61,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
 
   // this lane's column in each tile: its token, head, and the keys it sees, [first, position]
   int position[COLUMN_TILES], first[COLUMN_TILES], token_row[COLUMN_TILES], head[COLUMN_TILES];
+  [[maybe_unused]] float slope[COLUMN_TILES];  // of the column's head, in units of log2
   f32x4 query[COLUMN_TILES][D_STEPS];
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
@@ -68,6 +72,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
     head[t] = kv_head * group + flat % group;
     position[t] = live ? positions[token_row[t]] : -1;
     first[t] = window > 0 ? max(0, position[t] - window + 1) : 0;
+    if (CHANGED) slope[t] = slopes ? slopes[head[t]] * 1.4426950408889634f : 0.f;
     const float* q = qkv + (size_t)token_row[t] * row_width + head[t] * D + 4 * g;
 #pragma unroll
     for (int s = 0; s < D_STEPS; ++s) {
@@ -145,6 +150,10 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
       for (int e = 0; e < 4; ++e) {
         const int key = key0 + 4 * g + e;
         const bool seen = key <= position[t] && key >= first[t];
+        if (CHANGED) {  // scores are kept in units of log2: the cap is applied to the score itself
+          if (soft_cap > 0.f) s4[e] = soft_cap * 1.4426950408889634f * tanhf(s4[e] * 0.6931471805599453f / soft_cap);
+          s4[e] -= slope[t] * (float)(position[t] - key);
+        }
         s4[e] = seen ? s4[e] : -INFINITY;
         best = fmaxf(best, s4[e]);
       }
@@ -271,13 +280,13 @@ __global__ __launch_bounds__(64) void attention_f32_merge_kernel(float* __restri
 
 // qkv [tokens, row_width] float32 with the queries in front (heads * D), out [tokens, heads * D]; key pages in
 // pieces ([page, kv_head, D / 8, offset, 8]), value pages transposed ([page, kv_head, D, offset]); work [items, 4].
-// column_tiles 1 or 2; page_size a multiple of 4.  With splits > 1: partial_acc float32 [splits, tokens * heads, D]
+// column_tiles 1 or 2; page_size a multiple of 4; slopes float32 [heads] or null, soft_cap 0 for none.  With splits > 1: partial_acc float32 [splits, tokens * heads, D]
 // and partial_ml [splits, tokens * heads, 2]; every column of the step must belong to an item.
 extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* out, float* partial_acc, float* partial_ml,
                                       const float* keys, const float* values, const int* block_tables, int table_width,
                                       const int* positions, const int* work, int items, int column_tiles, int tokens,
                                       int heads, int kv_heads, int page_size, float scale, int window, int splits,
-                                      hipStream_t stream) {
+                                      const float* slopes, float soft_cap, hipStream_t stream) {
   if (items <= 0 || tokens <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 4 || splits < 1 ||
       (column_tiles != 1 && column_tiles != 2) || (splits > 1 && (!partial_acc || !partial_ml)))
@@ -285,14 +294,16 @@ extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* ou
   const float scale_log2 = scale * 1.4426950408889634f;
   const int columns_total = tokens * heads;
   dim3 grid(items, kv_heads, splits);
-  if (column_tiles == 1)
-    hipLaunchKernelGGL(attention_f32_kernel<1>, grid, dim3(WAVES * 64), 0, stream, qkv, row_width, out, partial_acc,
-                       partial_ml, keys, values, block_tables, table_width, positions, work, heads, kv_heads, page_size,
-                       scale_log2, window, splits, columns_total);
-  else
-    hipLaunchKernelGGL(attention_f32_kernel<2>, grid, dim3(WAVES * 64), 0, stream, qkv, row_width, out, partial_acc,
-                       partial_ml, keys, values, block_tables, table_width, positions, work, heads, kv_heads, page_size,
-                       scale_log2, window, splits, columns_total);
+  const bool changed = slopes != nullptr || soft_cap > 0.f;
+#define LAUNCH_ATTENTION_F32(TILES, CHANGED)                                                                          \
+  hipLaunchKernelGGL((attention_f32_kernel<TILES, CHANGED>), grid, dim3(WAVES * 64), 0, stream, qkv, row_width, out,   \
+                     partial_acc, partial_ml, keys, values, block_tables, table_width, positions, work, heads,        \
+                     kv_heads, page_size, scale_log2, window, splits, columns_total, slopes, soft_cap)
+  if (column_tiles == 1 && !changed) LAUNCH_ATTENTION_F32(1, false);
+  else if (column_tiles == 1) LAUNCH_ATTENTION_F32(1, true);
+  else if (!changed) LAUNCH_ATTENTION_F32(2, false);
+  else LAUNCH_ATTENTION_F32(2, true);
+#undef LAUNCH_ATTENTION_F32
   int status = LAUNCH_STATUS();
   if (status != 0 || splits == 1) return status;
   hipLaunchKernelGGL(attention_f32_merge_kernel, dim3(columns_total), dim3(64), 0, stream, out, partial_acc, partial_ml,

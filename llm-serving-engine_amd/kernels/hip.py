@@ -63,7 +63,7 @@ _SIGNATURES = {
     "llmserve_gemm_tiled": "pppipiiiiiip",
     "llmserve_gemm_wide": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifipfp",
-    "llmserve_attention_f32": "pippppppippiiiiiifiip",
+    "llmserve_attention_f32": "pippppppippiiiiiifiipfp",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
     "llmserve_attention_portions": "pippppippiiiiifip",
     "llmserve_attention_can_fuse": "i",
@@ -651,8 +651,8 @@ class HipKernels:
         score_slopes: torch.Tensor | None = None, soft_cap: float | None = None,
     ) -> torch.Tensor:
         """`score_slopes` (float32 [heads]) and `soft_cap` change the scores before the softmax: cap * tanh(score /
-        cap), then minus slope * distance.  Only the generic kernel takes them: the matrix-core kernels are
-        passed by when either is given."""
+        cap), then minus slope * distance.  The float32 kernels take them; in bfloat16 the matrix-core kernels
+        are passed by when either is given, for the generic kernel."""
         tokens = qkv.shape[0]
         group = batch.groups[cell.group]
         if cell.keys.dtype != qkv.dtype:
@@ -667,8 +667,8 @@ class HipKernels:
         if plain_scores and qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
             self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0))
             return out
-        if plain_scores and qkv.dtype == torch.float32 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
-            self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0))
+        if qkv.dtype == torch.float32 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
+            self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0), score_slopes, soft_cap)
             return out
         if qkv.dtype == torch.bfloat16:
             why = "its scores carry a bias or a soft cap" if not plain_scores else f"head size {dim} and pages of {group.page_size}"
@@ -682,7 +682,7 @@ class HipKernels:
         _check(status, "paged_attention")
         return out
 
-    def _attention_float32(self, qkv, out, layout, batch, cell, group, scale: float, window: int) -> None:
+    def _attention_float32(self, qkv, out, layout, batch, cell, group, scale: float, window: int, score_slopes=None, soft_cap=None) -> None:
         """The 32-bit path's attention on the matrix cores: an item is 16 (decoding) or 32 columns of one
         request, (token, head) pairs running through the tokens head by head whatever the number of heads; few
         items over long contexts are cut into key splits that a second kernel merges."""
@@ -709,7 +709,8 @@ class HipKernels:
         status = self._attention_f32[dim].llmserve_attention_f32(
             _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml), _pointer(cell.keys),
             _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work),
-            items, column_tiles, tokens, heads, kv_heads, group.page_size, scale, window, splits, self._stream,
+            items, column_tiles, tokens, heads, kv_heads, group.page_size, scale, window, splits, _pointer(score_slopes),
+            float(soft_cap or 0.0), self._stream,
         )
         _check(status, "paged_attention")
 

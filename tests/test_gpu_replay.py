@@ -312,3 +312,44 @@ def test_a_long_context_through_the_whole_engine(wide_models, dtype):
         fed, at = fed + 1, at + 1
     assert checked == 9 + 6 + 12 and total / checked < (BF16_MEAN * spread if dtype == "bfloat16" else walk)
     runner.close()
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_nine_thousand_keys_through_the_whole_engine(tmp_path_factory, dtype):
+    """A context of more than 9,000 keys through the step function, in both precisions: a prompt in portions of
+    2,048 tokens (each portion's queries behind thousands of cached keys), then single tokens decoded from captured
+    steps whose keys are cut into splits and merged by the merging kernel, beside a short request; a key planted
+    far back must decide the last logits.  Against the plain forward of a narrow model with the benchmark's head
+    size."""
+    from llmserve_amd import CacheConfig, ModelRunner, StepEntry
+    from llmserve_amd.kernels import HipKernels
+    from llmserve_amd.weights import load_model_folder, write_model_folder
+    from tests.tiny import LONG, LOUD
+
+    folder = write_model_folder(tmp_path_factory.mktemp("long") / "long", LONG, seed=77, norm_std=0.1, **LOUD)
+    plain_config, weights = plain.PlainConfig.from_folder(folder), plain.read_weights(folder)
+    sequences = [random_tokens(9100, LONG.vocab_size, seed=821), random_tokens(40, LONG.vocab_size, seed=822)]
+    expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
+    spread = float(expected[0].std())
+    walk = math.sqrt(9100) * 2.0 ** -24 * spread
+    bound = dict(atol=BF16_LARGEST * spread, rtol=3e-2) if dtype == "bfloat16" else dict(atol=8 * walk, rtol=1e-4)
+    loaded = load_model_folder(folder, dtype)
+    runner = ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(PAGE_WIDE, 600, 4))
+    fed, checked = 0, 0
+    for count in (2048, 2048, 2048, 2048, 900):
+        want = [0, count - 1]
+        logits = runner.step([StepEntry("long", sequences[0][fed : fed + count], want)], create_missing=True)
+        for row, place in enumerate(want):
+            torch.testing.assert_close(logits[row].cpu().double(), expected[0][fed + place], **bound,
+                                       msg=lambda m: f"position {fed + place}: {m}")
+        fed, checked = fed + count, checked + 2
+    runner.step([StepEntry("short", sequences[1][:30], [])], create_missing=True)
+    for step in range(8):  # two requests decode side by side: 9,092 + step keys and 30 + step
+        entries = [StepEntry("long", [sequences[0][fed + step]], [0]), StepEntry("short", [sequences[1][30 + step]], [0])]
+        logits = runner.step(entries)
+        torch.testing.assert_close(logits[0].cpu().double(), expected[0][fed + step], **bound,
+                                   msg=lambda m: f"decoded position {fed + step}: {m}")
+        torch.testing.assert_close(logits[1].cpu().double(), expected[1][30 + step], **bound)
+        checked += 2
+    assert checked == 26 and runner.step_counts["replayed"] >= 6
+    runner.close()

@@ -128,6 +128,25 @@ WIDE_32B = Qwen2Config(
     rope_pairing="half",
 )
 
+# A narrow model with the benchmark's head size, for contexts of thousands of keys through the whole engine: six
+# query heads over one kv head of 128, so that decoding takes the kernels that serving takes there (the fused
+# decode attention, its key splits, the kernel that merges them).
+LONG = Qwen2Config(
+    vocab_size=517,
+    hidden_size=384,
+    intermediate_size=640,
+    num_layers=2,
+    num_attention_heads=6,
+    num_key_value_heads=1,
+    head_dim=128,
+    max_position_embeddings=16384,
+    rope_theta=1e6,
+    rms_norm_eps=1e-6,
+    attention_bias=True,
+    tie_word_embeddings=True,
+    rope_pairing="half",
+)
+
 WIDE_CONFIGS = {"1.5B": (WIDE, 31), "7B": (WIDE_7B, 37), "32B": (WIDE_32B, 41)}
 
 
