@@ -6,7 +6,7 @@ from typing import Any
 
 import torch
 
-from ..parts.base import KEY_PIECE, key_piece_width  # noqa: F401  (kernel libraries and tests find them here)
+from ..parts.base import KEY_PIECE, VALUE_PIECE, key_piece_width, value_piece_width  # noqa: F401  (kernel libraries and tests find them here)
 
 
 class CacheCell:
@@ -16,7 +16,8 @@ class CacheCell:
     [pages, *page shape] of this run, and `group` indexes `StepBatch.groups` (where the step's tokens
     go, and the requests' block tables).  For keys and values (`PagedKeyValue`): `keys` is [pages,
     kv_heads, head_dim / w, page_size, w] with w = `key_piece_width(head_dim)`, `values` is stored
-    transposed, [pages, kv_heads, head_dim, page_size]; both are also attributes of the cell.
+    transposed in pieces of v = `value_piece_width(page_size)` keys, [pages, kv_heads, page_size / v, head_dim,
+    v]; both are also attributes of the cell, and `key_rows` / `value_rows` give whole rows back.
     For a per-request need: `state` is [slots, *shape] float32, indexed by `StepBatch.state_slots`.
     `writable` is False when the run reads a cell that another run owns.
     """
@@ -66,3 +67,13 @@ class CacheCell:
         """Writes whole rows [n, kv_heads, head_dim] as the keys at (pages[i], offsets[i])."""
         pieces, width = self.keys.shape[2], self.keys.shape[4]
         self.keys[pages, :, :, offsets] = rows.reshape(rows.shape[0], rows.shape[1], pieces, width).to(self.keys.dtype)
+
+    def value_rows(self, pages: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
+        """The values at (pages[i], offsets[i]) as whole rows, [n, kv_heads, head_dim]."""
+        width = self.values.shape[4]
+        return self.values[pages, :, offsets // width, :, offsets % width]
+
+    def put_value_rows(self, pages: torch.Tensor, offsets: torch.Tensor, rows: torch.Tensor) -> None:
+        """Writes whole rows [n, kv_heads, head_dim] as the values at (pages[i], offsets[i])."""
+        width = self.values.shape[4]
+        self.values[pages, :, offsets // width, :, offsets % width] = rows.to(self.values.dtype)

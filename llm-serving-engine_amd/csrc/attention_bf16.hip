@@ -8,8 +8,9 @@
 //   P = exp(S * scale - the column's reference maximum), masked per column to the keys (p - window, p]
 //   O^T[d][column] += V^T[d][key] * P^T[key][column]      A = rows of the transposed V page
 // so each lane owns one column: its running maximum, its sum and four rows of every 16-row
-// tile of O^T.  Value pages are stored transposed ([page, kv_head, dim, offset]) so that the
-// keys, the contraction index of the second product, are contiguous for the A operand; key pages
+// tile of O^T.  Value pages are stored transposed, in pieces of eight keys ([page, kv_head, offset / 8,
+// dim, 8]; common.h: value_element), so that the keys, the contraction index of the second product, are
+// contiguous for the A operand and neighbouring lanes, which hold neighbouring rows, read neighbouring bytes; key pages
 // are stored in pieces of eight elements, a piece of all the page's keys side by side ([page,
 // kv_head, dim / 8, offset, 8]), so that neighbouring lanes, which hold the same piece of
 // neighbouring keys, read neighbouring bytes (common.h: key_element); the
@@ -374,7 +375,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
     bf16_t* k_page = keys + (size_t)(new_slot / page_size) * page_stride + head_offset + (size_t)(new_slot % page_size) * KEY_PIECE;
     const unsigned piece_stride = (unsigned)page_size * KEY_PIECE;
     auto k_at = [&](int e) -> bf16_t& { return k_page[(unsigned)(e / KEY_PIECE) * piece_stride + e % KEY_PIECE]; };
-    bf16_t* v_page = values + (size_t)(new_slot / page_size) * page_stride + head_offset + new_slot % page_size;
+    bf16_t* v_page = values + (size_t)(new_slot / page_size) * page_stride + head_offset +
+                     (size_t)(new_slot % page_size / VALUE_PIECE) * (D * VALUE_PIECE) + new_slot % page_size % VALUE_PIECE;
 #pragma unroll
     for (int i = 0; i < PAIR_PIECES; ++i) {
       const int j = lane + i * WAVE;
@@ -388,7 +390,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
 #pragma unroll
     for (int i = 0; i < VALUE_PIECES; ++i) {
       const int d = lane + i * WAVE;
-      if (d < D) v_page[(size_t)d * page_size] = new_v[i];
+      if (d < D) v_page[(size_t)d * VALUE_PIECE] = new_v[i];  // (pages are multiples of eight keys here: common.h, value_element)
     }
     // Other lanes of this wave read these bytes back below.  A wave's accesses to memory are carried
     // out in the order it issues them, so nothing has to be waited for; the fence keeps the compiler
@@ -440,9 +442,11 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   };
   auto fetch_values = [&](int step, const StepPages& P, StepLoads& L) {
     const StepKeys at = keys_of(step);
-    const bf16_t* base = values + (size_t)(unsigned)P.v * page_stride + (head_offset + (unsigned)(at.v - page_index(at.v) * page_size));
+    // the lane's eight keys are one piece of the page: [page_size / 8][D][8], the rows of a piece side by side
+    const bf16_t* base = values + (size_t)(unsigned)P.v * page_stride +
+                         (head_offset + (unsigned)(at.v - page_index(at.v) * page_size) * (unsigned)D);
 #pragma unroll
-    for (int d = 0; d < D_TILES; ++d) L.v[d] = *(const bf16x8*)(base + (unsigned)(d * 16 + c) * page_size);
+    for (int d = 0; d < D_TILES; ++d) L.v[d] = *(const bf16x8*)(base + (unsigned)(d * 16 + c) * VALUE_PIECE);
   };
 
   const float scale_log2 = scale * 1.44269504088896f;
@@ -679,14 +683,15 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      // V^T: lane l takes piece l % 4 (the keys 8 piece .. 8 piece + 7 of the step) of row 16 (2 wave + j) + l / 4
-      const int d = 16 * (2 * wave + j) + (lane >> 2);
-      const int piece = lane & 3;
+      // V^T: lane l takes piece l / 16 (the keys 8 piece .. 8 piece + 7 of the step) of row 16 (2 wave + j) + l % 16:
+      // sixteen lanes read 256 bytes in a row (a page keeps a piece of eight keys of all rows side by side)
+      const int d = 16 * (2 * wave + j) + (lane & 15);
+      const int piece = lane >> 4;
       const int key = min(max(key0 + 8 * piece, low_limit), high_limit);
       const int page = piece == 0 ? pages[0] : piece == 1 ? pages[1] : piece == 2 ? pages[2] : pages[3];
       const int offset = key - page_index(key) * page_size;
       pieces.v[j] = *(const bf16x8*)(values + (size_t)(unsigned)page * page_stride +
-                                     (head_offset + (unsigned)d * page_size + offset));
+                                     (head_offset + ((unsigned)offset * D + (unsigned)d * VALUE_PIECE)));
     }
   };
   auto write_step = [&](const StagedPieces& pieces, bf16_t* stage) {
@@ -695,8 +700,8 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
       const int row = 8 * wave + (lane & 7);
       const int slot = (8 * j + (lane >> 3)) ^ ((row & 3) | ((row >> 3) << 2));
       *(bf16x8*)(stage + (size_t)row * D + slot * 8) = pieces.k[j];
-      const int d = 16 * (2 * wave + j) + (lane >> 2);
-      *(bf16x8*)(stage + KEYS * D + (size_t)d * KEYS + ((lane & 3) ^ ((d >> 1) & 3)) * 8) = pieces.v[j];
+      const int d = 16 * (2 * wave + j) + (lane & 15);
+      *(bf16x8*)(stage + KEYS * D + (size_t)d * KEYS + ((lane >> 4) ^ ((d >> 1) & 3)) * 8) = pieces.v[j];
     }
   };
 

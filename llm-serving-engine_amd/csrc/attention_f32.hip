@@ -130,11 +130,13 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
       next_key_page = table[key_of(step + WAVES) / page_size];
       next_value_page = table[value_key_of(step + WAVES) / page_size];
     }
-    const float* v_at = values + ((size_t)value_page * kv_heads + kv_head) * page_elements + (size_t)i * page_size +
-                        value_key % page_size;
+    // (its four keys are half a piece of eight keys, or lie in the one piece of a page that is no multiple of eight)
+    const float* v_at = values + ((size_t)value_page * kv_heads + kv_head) * page_elements +
+                        value_element(i, value_key % page_size, page_size, D);
+    const int value_width = value_piece_width(page_size);
     f32x4 v[D_STEPS];
 #pragma unroll
-    for (int s = 0; s < D_STEPS; ++s) v[s] = load4(v_at + (size_t)(16 * s) * page_size);
+    for (int s = 0; s < D_STEPS; ++s) v[s] = load4(v_at + (size_t)(16 * s) * value_width);
 
     f32x4 p[COLUMN_TILES];
 #pragma unroll
@@ -279,7 +281,8 @@ __global__ __launch_bounds__(64) void attention_f32_merge_kernel(float* __restri
 }
 
 // qkv [tokens, row_width] float32 with the queries in front (heads * D), out [tokens, heads * D]; key pages in
-// pieces ([page, kv_head, D / 8, offset, 8]), value pages transposed ([page, kv_head, D, offset]); work [items, 4].
+// pieces ([page, kv_head, D / 8, offset, 8]), value pages transposed in pieces of eight keys ([page, kv_head,
+// page_size / 8, D, 8]; common.h: value_element); work [items, 4].
 // column_tiles 1 or 2; page_size a multiple of 4; slopes float32 [heads] or null, soft_cap 0 for none.  With splits > 1: partial_acc float32 [splits, tokens * heads, D]
 // and partial_ml [splits, tokens * heads, 2]; every column of the step must belong to an item.
 extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* out, float* partial_acc, float* partial_ml,

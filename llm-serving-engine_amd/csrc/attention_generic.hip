@@ -70,8 +70,8 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
       for (int j = 0; j < in_tile; ++j) {
         const int at = tile + j;
         const int page = table[at / page_size];
-        const T* v = values + ((size_t)page * kv_heads + kv_head) * page_size * dim + at % page_size;
-        sum = fmaf(weights[j], to_float(v[(size_t)d * page_size]), sum);  // value pages are [dim, offset]
+        const T* v = values + ((size_t)page * kv_heads + kv_head) * page_size * dim;
+        sum = fmaf(weights[j], to_float(v[value_element(d, at % page_size, page_size, dim)]), sum);  // common.h: value_element
       }
       acc[i] = acc[i] * correction + sum;
     }

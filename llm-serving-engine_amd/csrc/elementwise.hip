@@ -224,8 +224,8 @@ extern "C" int llmserve_rotary_table(const int* positions, const float* inverse,
 // pairing 0: none, 1: adjacent pairs (2j, 2j+1), 2: half pairs (j, j + dim/2).
 // k (after rotation) and v are then written to the pages: slot = page * page_size + offset,
 // key pages laid out [page, kv_head, dim / 8, offset, 8] (common.h: key_element), value pages
-// transposed [page, kv_head, dim, offset] (reference kv_cache.py:249-266 writes both as
-// [page, offset, kv_head, dim]).
+// transposed in pieces of eight keys, [page, kv_head, page_size / 8, dim, 8] (common.h: value_element;
+// reference kv_cache.py:249-266 writes both as [page, offset, kv_head, dim]).
 // slots may be null (nothing is stored); a negative slot skips the token.
 template <typename T>
 __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const float2* __restrict__ table, int pairing, int heads,
@@ -259,7 +259,7 @@ __global__ void rotate_and_store_kernel(T* __restrict__ qkv, const float2* __res
     const int head = i / dim, d = i % dim;
     const size_t block = ((size_t)page * kv_heads + head) * page_size * dim;
     keys[block + key_element(d, offset, page_size, dim)] = k_row[i];
-    values[block + (size_t)d * page_size + offset] = v_row[i];
+    values[block + value_element(d, offset, page_size, dim)] = v_row[i];
   }
 }
 
@@ -278,10 +278,10 @@ __global__ __launch_bounds__(256) void rotate_and_store_vector_kernel(
   const size_t id = (size_t)blockIdx.x * 256 + threadIdx.x, rotating = (size_t)tokens * rotated;
   const int row_width = (heads + 2 * kv_heads) * dim;
   if (id >= rotating) {
-    // The values.  A page keeps them transposed (attention sums over keys), so a token's value row is
-    // `dim` two-byte stores far apart.  A thread therefore takes four dims of eight tokens in a row: its
-    // loads are 8 bytes beside its neighbours', and where the eight tokens lie side by side in a page
-    // (a prompt's portion) it stores 16 bytes a dim.
+    // The values.  A page keeps them transposed in pieces of eight keys (attention sums over keys), so a
+    // token's value row is `dim` two-byte stores 16 bytes apart.  A thread therefore takes four dims of eight
+    // tokens in a row: its loads are 8 bytes beside its neighbours', and where the eight tokens are one piece
+    // of a page (a prompt's portion) it stores 16 bytes a dim, 64 bytes in a row.
     if (slots == nullptr) return;
     const int quads = dim / 4;
     const size_t unit = id - rotating;
@@ -301,19 +301,19 @@ __global__ __launch_bounds__(256) void rotate_and_store_vector_kernel(
 #pragma unroll
     for (int i = 1; i < 8; ++i) together = together && slot[i] == slot[0] + i;
     if (together) {
-      bf16_t* v_page = values + ((size_t)(slot[0] / page_size) * kv_heads + head) * page_size * dim + slot[0] % page_size;
+      bf16_t* v_page = values + ((size_t)(slot[0] / page_size) * kv_heads + head) * page_size * dim;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const bf16x8 run = {v[0][e], v[1][e], v[2][e], v[3][e], v[4][e], v[5][e], v[6][e], v[7][e]};
-        *(bf16x8*)(v_page + (size_t)(quad * 4 + e) * page_size) = run;
+        *(bf16x8*)(v_page + value_element(quad * 4 + e, slot[0] % page_size, page_size, dim)) = run;
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if (slot[i] < 0) continue;
-        bf16_t* v_page = values + ((size_t)(slot[i] / page_size) * kv_heads + head) * page_size * dim + slot[i] % page_size;
+        bf16_t* v_page = values + ((size_t)(slot[i] / page_size) * kv_heads + head) * page_size * dim;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v_page[(size_t)(quad * 4 + e) * page_size] = v[i][e];
+        for (int e = 0; e < 4; ++e) v_page[value_element(quad * 4 + e, slot[i] % page_size, page_size, dim)] = v[i][e];
       }
     }
     return;

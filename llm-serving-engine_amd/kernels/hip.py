@@ -258,7 +258,7 @@ class HipKernels:
             raise KernelError("rotate_and_store: qkv does not have the layout's width")
         store = cell is not None and cell.writable
         group = batch.groups[cell.group] if store else None
-        if store and (cell.keys.dtype != qkv.dtype or cell.values.shape[1:] != (layout.num_kv_heads, layout.head_dim, group.page_size)):
+        if store and (cell.keys.dtype != qkv.dtype or cell.values.shape[1:] != cell.need.page_fields(group.page_size)["values"]):
             raise KernelError("rotate_and_store: the cell's pages do not fit the layout")
         table = self.rotary_table(batch, inverse_frequencies) if pairing != "none" else None
         status = self._elementwise.llmserve_rotate_and_store(

@@ -39,6 +39,14 @@ def key_piece_width(head_dim: int) -> int:
     return KEY_PIECE if head_dim % KEY_PIECE == 0 else head_dim
 
 
+VALUE_PIECE = 8  # keys whose values of one dimension stay together in a page (csrc/common.h has the same number)
+
+
+def value_piece_width(page_size: int) -> int:
+    """A page's values are kept in pieces of VALUE_PIECE keys; a page size that is no multiple of it in one piece."""
+    return VALUE_PIECE if page_size % VALUE_PIECE == 0 else page_size
+
+
 class CacheNeed:
     """What a part keeps in the cache from one step to the next.  The cache manager knows two ways of
     giving room, and a need is of one of them: `PagedNeed` (an entry per token, in pages that a request
@@ -79,8 +87,9 @@ class PagedKeyValue(PagedNeed):
     eight elements, the same piece of all the keys of a page side by side ([kv_heads, head_dim / w,
     page_size, w], w = `key_piece_width(head_dim)`): the matrix cores take keys as rows, a lane holding
     one piece of one key and its neighbours that piece of the next keys, and neighbouring lanes should
-    read neighbouring bytes.  Values are stored transposed ([kv_heads, head_dim, page_size]): attention
-    sums over keys, and the matrix cores want the summed index contiguous."""
+    read neighbouring bytes.  Values are stored transposed, in pieces of eight keys ([kv_heads, page_size / v,
+    head_dim, v], v = `value_piece_width(page_size)`): attention sums over keys, the matrix cores want the
+    summed index contiguous, and a lane's neighbours hold the same keys of the next dimensions."""
 
     num_kv_heads: int
     head_dim: int
@@ -90,12 +99,13 @@ class PagedKeyValue(PagedNeed):
         width = key_piece_width(self.head_dim)
         return {
             "keys": (self.num_kv_heads, self.head_dim // width, page_size, width),
-            "values": (self.num_kv_heads, self.head_dim, page_size),
+            "values": (self.num_kv_heads, page_size // value_piece_width(page_size), self.head_dim, value_piece_width(page_size)),
         }
 
     def token_rows(self, page: dict[str, torch.Tensor], page_size: int) -> dict[str, torch.Tensor]:
         keys = page["keys"].permute(2, 0, 1, 3).reshape(page_size, self.num_kv_heads, self.head_dim)
-        return {"keys": keys, "values": page["values"].permute(2, 0, 1)}
+        values = page["values"].permute(1, 3, 0, 2).reshape(page_size, self.num_kv_heads, self.head_dim)
+        return {"keys": keys, "values": values}
 
 
 @dataclass(frozen=True)

@@ -108,7 +108,7 @@ def test_full_cache_raises_and_holds_nothing_new():
 def test_groups_have_pages_of_their_own_and_a_window_gives_them_back():
     cache = manager(TINY_B, 8, 16, length=512)  # layer 0 sees all keys, layers 1 and 2 the last 24
     assert [(g.need.window, g.cells) for g in cache.groups] == [(None, [(0, None)]), (24, [(1, None), (2, None)])]
-    assert cache.groups[1].storage["keys"].shape == (2, 16, 1, 4, 8, 8) and cache.groups[1].storage["values"].shape == (2, 16, 1, 32, 8)
+    assert cache.groups[1].storage["keys"].shape == (2, 16, 1, 4, 8, 8) and cache.groups[1].storage["values"].shape == (2, 16, 1, 1, 32, 8)
     cache.create("r")
     cache.reserve("r", 40)  # nothing to give back yet: the step starts at position 0
     assert [g.pool.used_pages for g in cache.groups] == [5, 5]

@@ -139,6 +139,21 @@ def key_rows(pieces):
     return pieces.permute(0, 1, 3, 2, 4).reshape(pages, kv, page, count * width)
 
 
+def value_pieces(rows):
+    """Value pages written transposed [pages, kv, dim, page] -> as the cache keeps them, in pieces of eight keys,
+    the same piece of all dimensions side by side: [pages, kv, page / v, dim, v] (a page size that is no
+    multiple of 8 is one piece)."""
+    pages, kv, dim, page = rows.shape
+    width = 8 if page % 8 == 0 else page
+    return rows.view(pages, kv, dim, page // width, width).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def value_rows(pieces):
+    """The inverse of `value_pieces`."""
+    pages, kv, count, dim, width = pieces.shape
+    return pieces.permute(0, 1, 3, 2, 4).reshape(pages, kv, dim, count * width)
+
+
 def paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=0, spare_pages=3):
     """Requests with `lengths[i]` cached tokens of which the last `counts[i]` are this step's.
     Returns the step's batch, the cell with garbage in every unused slot, and per-request q, k, v."""
@@ -181,7 +196,7 @@ def paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=
         state_slots=ints(list(range(len(lengths)))), groups=[group], logit_rows=ints([]), num_logit_rows=0,
         max_query_length=max(counts), max_context_length=max(lengths),
     )
-    cell = CacheCell(PagedKeyValue(kv_heads, dim), True, 0, key_pieces(keys).to("cuda", dtype), values.to("cuda", dtype))
+    cell = CacheCell(PagedKeyValue(kv_heads, dim), True, 0, key_pieces(keys).to("cuda", dtype), value_pieces(values).to("cuda", dtype))
     return batch, cell, per_request, HeadLayout(heads, kv_heads, dim)
 
 
@@ -250,13 +265,13 @@ def test_paged_attention_window_edge(kernels, dtype, window):
 
 
 def _rewrite_cell(batch, cell, per_request, page, dtype):
-    keys, values = key_rows(cell.keys.cpu().float()), cell.values.cpu().float()
+    keys, values = key_rows(cell.keys.cpu().float()), value_rows(cell.values.cpu().float())
     tables = batch.groups[0].block_tables.cpu()
     for index, (q, k, v) in enumerate(per_request):
         for position in range(k.shape[0]):
             keys[tables[index, position // page], :, position % page] = k[position]
             values[tables[index, position // page], :, :, position % page] = v[position]
-    cell.keys, cell.values = key_pieces(keys).to("cuda", dtype), values.to("cuda", dtype)
+    cell.keys, cell.values = key_pieces(keys).to("cuda", dtype), value_pieces(values).to("cuda", dtype)
     return batch, cell, per_request, None
 
 
@@ -390,14 +405,14 @@ def test_rotate_and_store(kernels, dtype, pairing, heads, kv_heads, dim, page):
     torch.testing.assert_close(qkv.cpu().double().view_as(expected), expected, **TOLERANCE[dtype])
     slots = batch.groups[0].slot_mapping.cpu().long()
     stored_k = key_rows(cell.keys.cpu().double())[slots // page, :, slots % page]
-    stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
+    stored_v = value_rows(cell.values.cpu().double())[slots // page, :, :, slots % page]
     torch.testing.assert_close(stored_k, expected[:, heads : heads + kv_heads], **TOLERANCE[dtype])
     torch.testing.assert_close(stored_v, expected[:, heads + kv_heads :], atol=0, rtol=0)
     untouched = torch.ones(cell.keys.shape[0], page, dtype=torch.bool)
     untouched[slots // page, slots % page] = False
     same = lambda a, b: torch.equal(torch.nan_to_num(a.float().cpu(), nan=7.0), torch.nan_to_num(b.float().cpu(), nan=7.0))
     assert same(key_rows(cell.keys).transpose(1, 2)[untouched], key_rows(before_keys).transpose(1, 2)[untouched])
-    assert same(cell.values.permute(0, 3, 1, 2)[untouched], before_values.permute(0, 3, 1, 2)[untouched])
+    assert same(value_rows(cell.values).permute(0, 3, 1, 2)[untouched], value_rows(before_values).permute(0, 3, 1, 2)[untouched])
     # a cell that is only read stores nothing
     readonly = types.SimpleNamespace(writable=False)
     again = on_gpu(rows, dtype)
@@ -555,7 +570,7 @@ def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
     _rewrite_cell(batch, cell, per_request, page, dtype)
     slots = batch.groups[0].slot_mapping.cpu().long()
     cell.keys[slots // page, :, :, slots % page] = float("nan")
-    cell.values[slots // page, :, :, slots % page] = float("nan")
+    cell.put_value_rows(slots // page, slots % page, torch.full((len(slots), cell.values.shape[1], cell.values.shape[3]), float("nan"), device=cell.values.device))
     rows = []  # the step's rows carry unrotated q and k
     for (q, k, v), original in zip(per_request, [p[1] for p in paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=dim + page)[2]]):
         rows.append(torch.cat([q[-1:].flatten(1), original[-1:].flatten(1), v[-1:].flatten(1)], dim=1))
@@ -563,7 +578,7 @@ def test_fused_decode_attention(kernels, pairing, heads, kv_heads, dim, page):
     out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None if pairing == "none" else on_gpu(inverse), pairing, 0.2, None)
     torch.testing.assert_close(out.cpu().double(), torch.cat(expected), **TOLERANCE[dtype])
     stored_k = key_rows(cell.keys.cpu().double())[slots // page, :, slots % page]
-    stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
+    stored_v = value_rows(cell.values.cpu().double())[slots // page, :, :, slots % page]
     want_k = torch.stack([p[1][-1].double() for p in per_request])
     want_v = torch.stack([rounded(p[2][-1], dtype) for p in per_request])
     torch.testing.assert_close(stored_k, want_k, **TOLERANCE[dtype])
@@ -586,7 +601,7 @@ def test_fused_decode_attention_over_long_contexts(kernels, requests):
     _rewrite_cell(batch, cell, per_request, page, dtype)
     slots = batch.groups[0].slot_mapping.cpu().long()
     cell.keys[slots // page, :, :, slots % page] = float("nan")  # the step itself stores the newest key and value
-    cell.values[slots // page, :, :, slots % page] = float("nan")
+    cell.put_value_rows(slots // page, slots % page, torch.full((len(slots), cell.values.shape[1], cell.values.shape[3]), float("nan"), device=cell.values.device))
     qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
     out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, None, "none", 1.0, None).cpu().double()
     for index, ((q, k, v), far) in enumerate(zip(per_request, places)):
@@ -808,12 +823,12 @@ def test_rotation_store_and_attention_of_prompt_portions(kernels, dtype, pairing
     _rewrite_cell(batch, cell, per_request, page, dtype)
     slots = batch.groups[0].slot_mapping.cpu().long()
     cell.keys[slots // page, :, :, slots % page] = float("nan")  # the step stores these itself
-    cell.values[slots // page, :, :, slots % page] = float("nan")
+    cell.put_value_rows(slots // page, slots % page, torch.full((len(slots), cell.values.shape[1], cell.values.shape[3]), float("nan"), device=cell.values.device))
     qkv = on_gpu(step_rows(originals, counts, heads, kv_heads, dim), dtype)
     out = kernels[dtype].rotate_store_attend(qkv, layout, batch, cell, on_gpu(inverse), pairing, 0.2, None)
     torch.testing.assert_close(out.cpu().double(), torch.cat(expected), **TOLERANCE[dtype])
     stored_k = key_rows(cell.keys.cpu().double())[slots // page, :, slots % page]
-    stored_v = cell.values.cpu().double()[slots // page, :, :, slots % page]
+    stored_v = value_rows(cell.values.cpu().double())[slots // page, :, :, slots % page]
     want_k = torch.cat([k_rot[-count:] for k_rot, count in zip(rotated_keys, counts)])
     want_v = torch.cat([rounded(v, dtype)[-count:] for (q, k, v), count in zip(originals, counts)])
     torch.testing.assert_close(stored_k, want_k, **TOLERANCE[dtype])

@@ -86,7 +86,7 @@ class TorchKernels:
             slots = group.slot_mapping.long()
             pages, offsets = slots // group.page_size, slots % group.page_size
             cell.put_key_rows(pages, offsets, view[:, heads : heads + kv_heads])  # pages are [kv, dim / w, offset, w]
-            cell.values[pages, :, :, offsets] = view[:, heads + kv_heads :]  # pages are [kv, dim, offset]
+            cell.put_value_rows(pages, offsets, view[:, heads + kv_heads :])  # pages are [kv, offset / v, dim, v]
 
     def paged_attention(self, qkv, layout, batch, cell, scale, window, *, score_slopes=None, soft_cap=None):
         tokens = qkv.shape[0]
@@ -103,7 +103,7 @@ class TorchKernels:
                 pages = table[where // group.page_size]
                 assert (pages >= 0).all(), "attention reads a page that was given back"
                 keys = cell.key_rows(pages, where % group.page_size).float()  # [n, kv, D]
-                values = cell.values[pages, :, :, where % group.page_size].float()
+                values = cell.value_rows(pages, where % group.page_size).float()
                 keys = keys.repeat_interleave(heads // kv_heads, dim=1)
                 values = values.repeat_interleave(heads // kv_heads, dim=1)
                 scores = torch.einsum("hd,nhd->hn", queries[row], keys) * scale
