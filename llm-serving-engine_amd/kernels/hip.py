@@ -140,6 +140,7 @@ class HipKernels:
         self.library_products = library_products
         self.shared_portions = shared_portions
         self.merge_in_product = True  # decode attention leaves its key splits to the product that reads them
+        self.merge_weight_bytes = 8 << 20  # ... where that product's weight is at most this large (measured at 4.7 and 25.7 MB)
         name = torch.cuda.get_device_properties(self.device).gcnArchName
         if not name.startswith("gfx950"):
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this GPU is {name}")
@@ -840,10 +841,13 @@ class HipKernels:
                 and rows <= 16
                 and project.weight.dtype == torch.bfloat16
                 and project.in_features == layout.num_heads * dim
-                # every workgroup of the product reads all splits of its K range: rows * splits / 16 times what it
-                # reads of the weights.  Small next to the fixed costs at the 1.5B sizes (4.7 MB of weights), but at
-                # the 7B sizes (25.7 MB) it made a step of 8 rows 3.82 ms against 3.67 with the merging kernel.
-                and project.weight.numel() <= (1 << 22)
+                # Every workgroup of the product reads all splits of its K range, rows * splits / 16 times the bytes
+                # of its weights more than a plain product, and the kernel that merges as it loads is built for a
+                # small weight (one tile a wave).  Ahead at the 1.5B sizes (4.7 MB of weights: attention and projection
+                # 14.5 us against 15.3), behind at the 7B sizes (25.7 MB) at every number of rows, also where the
+                # splits are few bytes (a step of 1 / 2 / 4 / 8 rows 3.27 / 3.31 / 3.36 / 3.82 ms against 3.21 / 3.24 /
+                # 3.29 / 3.67 with the merging kernel): what decides is the weight, so the gate is its size.
+                and project.weight.numel() * project.weight.element_size() <= self.merge_weight_bytes
             )
             left = self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), fuse=(table, pairing), unmerged=merging)
             if left is None:
