@@ -589,23 +589,30 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
 }
 
 // ---------------------------------------------------------------------------- prompt portions, D = 128
-// For portions of many tokens the kernel above reads every key once per few tokens; this one shares
-// each step's K and V among the four waves of a workgroup through LDS.  A workgroup takes up to
-// 4 * COLUMN_TILES column tiles of a request (128 (token, head) pairs with two tiles: 21 tokens at six
-// query heads a kv head); every wave owns its own column tiles and walks all of their keys
-// itself (no key split, nothing to merge).  A step's 32 K rows and 128 x 32 V^T block (16 KB) are
-// brought in by all 256 threads, four 16-byte pieces each: requested into registers two steps ahead,
-// written to one of two LDS stages one step ahead.  A 16-byte piece of a row lies in the slot
-// (piece ^ f(row)) of its row, f chosen so that the 16 lanes that read one piece of 16 different
-// rows for an MFMA operand hit different banks.
-// (Loads that go from global memory straight into LDS were tried for this: the compiler makes every
-// read of LDS wait for all of them, whichever array they fill, so they cannot run two steps ahead.)
+// For portions of many tokens the kernel above reads every key once per few tokens, and what bounds it
+// then is the path from the caches into the registers (every wave asks for its own 16 KB a step).  This
+// one shares each step's K and V among the four waves of a workgroup through LDS.  A workgroup takes up
+// to 4 * COLUMN_TILES column tiles of a request (128 (token, head) pairs with two tiles: 21 tokens at six
+// query heads a kv head); every wave owns its own column tiles and walks all of their keys itself (no
+// key split inside the workgroup, nothing to merge).  A step's 32 K rows and 128 x 32 V^T block (16 KB)
+// go from memory straight into LDS (global_load_lds_dwordx4: each lane names its own 16 bytes of memory,
+// and the 64 lanes of an instruction fill 1 KB of LDS in lane order), sixteen such instructions a step,
+// four from each wave, two steps ahead of their use, into one of three stages.  Who asks for what is
+// chosen so that LDS holds the operands as the products read them, a whole wave 1 KB in a row:
+//   K: chunks 2j and 2j+1 (1 KB each) = pieces 4j .. 4j+3 (eight elements each) of the 16 rows of the "lo"
+//      and of the "hi" tile of the first product (for lane (c, q) piece 4j + q of row c)
+//   V: chunk t (1 KB) = tile t of V^T: for lane (c, q) the keys 8q .. 8q+7 of row 16 t + c.
+// The loads are written in assembly: the compiler knows that such a load writes LDS but not where, and
+// makes every later read of LDS wait for all of them, so they could not run ahead.  Here the waits are
+// counted by hand (the loop holds no other vector memory instruction): before the barrier that ends a
+// step, every wave waits until only its four youngest loads (the step after next) are still under way.
 #if HEAD_DIM == 128
-constexpr int PORTION_STAGE = 2 * KEYS * D;  // bf16 elements of a stage: K rows, then V^T rows
+constexpr int PORTION_STAGE_BYTES = 2 * KEYS * D * 2;  // K rows, then V^T rows
+constexpr int PORTION_STAGES = 3;
 
-struct StagedPieces {  // a lane's share of a step on its way to LDS
-  bf16x8 k[2], v[2];
-};
+__device__ __forceinline__ void load_to_lds(const bf16_t* from, unsigned to) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(to), "v"(from) : "memory");
+}
 
 template <int COLUMN_TILES>
 __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
@@ -613,7 +620,7 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
     const bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
     int page_size, int page_shift, float scale, int window) {
-  __shared__ __attribute__((aligned(16))) bf16_t stage_0[PORTION_STAGE], stage_1[PORTION_STAGE];  // each [K: 32 x 128 | V^T: 128 x 32]
+  __shared__ __attribute__((aligned(1024))) char stages[PORTION_STAGES * PORTION_STAGE_BYTES];
   const int group = heads / kv_heads;
   const int kv_head = blockIdx.y % kv_heads, head_tile = blockIdx.y / kv_heads;
   const int heads_here = min(group - head_tile * 16, 16);
@@ -657,6 +664,13 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
 #pragma unroll
     for (int d = 0; d < D_TILES; ++d) columns.acc[t][d] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
+  // The queries were asked for with ordinary loads, which the compiler counts: made to wait for them here, it
+  // knows them arrived; left to wait at their first use, inside the walk, it would wait there for everything
+  // that is under way, the loads into LDS included.
+#pragma unroll
+  for (int t = 0; t < COLUMN_TILES; ++t)
+#pragma unroll
+    for (int s = 0; s < QK_STEPS; ++s) asm volatile("" ::"v"(columns.query[t][s].v));
 
   const int step_first_all = first_key_all / KEYS, step_last_all = last_key_all / KEYS;
   const int step_first = first_key / KEYS, step_last = tokens > 0 ? last_key / KEYS : -1;
@@ -665,66 +679,90 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   const int low_limit = first_key_all & ~7, high_limit = last_key_all & ~7;
   auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
 
-  // This lane's four pieces of a step: of K rows 8 wave .. 8 wave + 7 and of V^T rows 32 wave .. 32 wave + 31.
-  // The four groups of eight keys of a step each lie in one page, looked up through scalar loads.
-  auto fetch_step = [&](int step, StagedPieces& pieces) {
+  // The four groups of eight keys of a step each lie in one page; pages of 16 or 32 keys (or multiples)
+  // hold two or all four of them.  Looked up through scalar loads, a step before the step's rows are asked for.
+  struct StepPageNumbers {
+    int a, b, c, d;
+    __device__ __forceinline__ int of_group(int i) const { return i == 0 ? a : i == 1 ? b : i == 2 ? c : d; }
+  };
+  const int lookups = page_size % 32 == 0 ? 1 : page_size % 16 == 0 ? 2 : 4;
+  auto pages_of_step = [&](int step) {
+    StepPageNumbers pages;
+    if (page_shift >= 4 && step * KEYS >= first_key_all && step * KEYS + KEYS - 1 <= last_key_all) {  // (see quick_pages)
+      const int* entry = table + ((step * KEYS) >> page_shift);
+      pages.a = entry[0];
+      pages.c = page_shift == 4 ? entry[1] : pages.a;
+      pages.b = pages.a;
+      pages.d = pages.c;
+      return pages;
+    }
+    auto of = [&](int i) { return table[page_index(min(max(step * KEYS + 8 * i, first_key_all), last_key_all))]; };
+    pages.a = of(0);
+    pages.c = lookups >= 2 ? of(2) : pages.a;
+    pages.b = lookups == 4 ? of(1) : pages.a;
+    pages.d = lookups == 4 ? of(3) : pages.c;
+    return pages;
+  };
+  // What this lane asks for in every step: of K the piece 4 wave + lane / 16 of row lane % 16 of the "lo" tile
+  // (key 8 (row / 4) + row % 4 of the step) and of the same row of the "hi" tile (four keys on: 64 bytes on in
+  // the page); of V^T the keys 8 (lane / 16) .. + 7 of rows 32 wave + lane % 16 and sixteen further (256 bytes on).
+  const int row_key = 8 * (c >> 2) + (c & 3);
+  const unsigned k_piece = 4 * wave + q;
+  const unsigned v_row = 32 * wave + c;
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) void*)stages;
+  // Steps that lie wholly inside the item's keys, in pages of a power of two from 16 keys on, need no more than
+  // a page number times the bytes of a page on top of what is fixed for the lane (and, with pages of more than
+  // 32 keys, for the step); the others (the first steps under a window, the last one, odd page sizes) go the long way.
+  const bool quick_pages = page_shift >= 4;
+  const unsigned in_page = (unsigned)page_size - 1;
+  const char* k_lane = (const char*)(keys + (head_offset + (k_piece * page_size + ((unsigned)row_key & in_page)) * KEY_PIECE));
+  const char* v_lane = (const char*)(values + (head_offset + ((8u * q) & in_page) * D + v_row * VALUE_PIECE));
+  const unsigned page_bytes = page_stride * 2;
+  const bool k_upper = c >= 8, v_upper = q >= 2;  // which of a step's two pages of 16 keys
+  auto fill_step = [&](int step, const StepPageNumbers& pages, int stage) {
     const int key0 = step * KEYS;
-    int pages[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) pages[i] = table[page_index(min(max(key0 + 8 * i, first_key_all), last_key_all))];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      // K: lane l takes piece 8 j + l / 8 of row 8 wave + l % 8: eight lanes read 128 bytes in a row
-      const int row = 8 * wave + (lane & 7);
-      const int key = min(max(key0 + row, first_key_all), last_key_all);
-      const int offset = key - page_index(key) * page_size;
-      pieces.k[j] = *(const bf16x8*)(keys + (size_t)(unsigned)pages[wave] * page_stride +
-                                     (head_offset + ((unsigned)(8 * j + (lane >> 3)) * page_size + offset) * KEY_PIECE));
+    const unsigned to = __builtin_amdgcn_readfirstlane(lds_base + (unsigned)stage * PORTION_STAGE_BYTES + (unsigned)wave * 2048);
+    const char *k_from, *k_from_hi, *v_from;
+    if (quick_pages && key0 >= first_key_all && key0 + KEYS - 1 <= last_key_all) {
+      const unsigned of_step = (unsigned)key0 & in_page;  // (0 unless a page holds several steps)
+      k_from = k_lane + (size_t)(unsigned)(k_upper ? pages.c : pages.a) * page_bytes + of_step * (KEY_PIECE * 2);
+      k_from_hi = k_from + 4 * KEY_PIECE * 2;
+      v_from = v_lane + (size_t)(unsigned)(v_upper ? pages.c : pages.a) * page_bytes + of_step * (D * 2);
+    } else {
+      // keys outside the item's range are read from a key inside it (their weights are zero), so that no page is
+      // touched that the request does not hold
+      const bf16_t* page = keys + (size_t)(unsigned)pages.of_group(row_key >> 3) * page_stride + head_offset;
+      const int key = min(max(key0 + row_key, first_key_all), last_key_all);
+      const int key_hi = min(max(key0 + row_key + 4, first_key_all), last_key_all);
+      k_from = (const char*)(page + (k_piece * page_size + (key - page_index(key) * page_size)) * KEY_PIECE);
+      k_from_hi = (const char*)(page + (k_piece * page_size + (key_hi - page_index(key_hi) * page_size)) * KEY_PIECE);
+      const int v_key = min(max(key0 + 8 * q, low_limit), high_limit);
+      const int v_offset = v_key - page_index(v_key) * page_size;
+      v_from = (const char*)(values + (size_t)(unsigned)pages.of_group(q) * page_stride +
+                             (head_offset + ((unsigned)v_offset * D + v_row * VALUE_PIECE)));
     }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      // V^T: lane l takes piece l / 16 (the keys 8 piece .. 8 piece + 7 of the step) of row 16 (2 wave + j) + l % 16:
-      // sixteen lanes read 256 bytes in a row (a page keeps a piece of eight keys of all rows side by side)
-      const int d = 16 * (2 * wave + j) + (lane & 15);
-      const int piece = lane >> 4;
-      const int key = min(max(key0 + 8 * piece, low_limit), high_limit);
-      const int page = piece == 0 ? pages[0] : piece == 1 ? pages[1] : piece == 2 ? pages[2] : pages[3];
-      const int offset = key - page_index(key) * page_size;
-      pieces.v[j] = *(const bf16x8*)(values + (size_t)(unsigned)page * page_stride +
-                                     (head_offset + ((unsigned)offset * D + (unsigned)d * VALUE_PIECE)));
-    }
+    load_to_lds((const bf16_t*)k_from, to);
+    load_to_lds((const bf16_t*)k_from_hi, to + 1024);
+    load_to_lds((const bf16_t*)v_from, to + KEYS * D * 2);
+    load_to_lds((const bf16_t*)(v_from + 16 * VALUE_PIECE * 2), to + KEYS * D * 2 + 1024);
   };
-  auto write_step = [&](const StagedPieces& pieces, bf16_t* stage) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int row = 8 * wave + (lane & 7);
-      const int slot = (8 * j + (lane >> 3)) ^ ((row & 3) | ((row >> 3) << 2));
-      *(bf16x8*)(stage + (size_t)row * D + slot * 8) = pieces.k[j];
-      const int d = 16 * (2 * wave + j) + (lane & 15);
-      *(bf16x8*)(stage + KEYS * D + (size_t)d * KEYS + ((lane >> 4) ^ ((d >> 1) & 3)) * 8) = pieces.v[j];
-    }
-  };
+  // every wave has read the stage that the next loads fill, and what it asked for two steps ago has arrived
+  // (its four youngest loads may still be under way); after the barrier that holds for all waves
+  auto end_of_step = [&]() { asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
   const float scale_log2 = scale * 1.44269504088896f;
-  const int row_lo = 8 * (c >> 2) + (c & 3);  // this lane's K row in the "lo" tile ("hi": four further)
-  const int k_swizzle = (row_lo & 3) | ((row_lo >> 3) << 2), v_swizzle = (c >> 1) & 3;
-  // One step: its operands are in `stage`.  `ahead` holds the pieces of the next step, requested two
-  // steps ago: they go to `other`, which was read last a step ago, and `ahead` is requested anew
-  // for the step after the one after next.
-  auto walk_step = [&](int step, const bf16_t* stage, bf16_t* other, StagedPieces& ahead) {
-    write_step(ahead, other);
-    fetch_step(step + 3, ahead);
+  const unsigned read_k = lane * 16, read_v = KEYS * D * 2 + lane * 16;  // this lane's bytes within a stage
+  auto walk_step = [&](int step, int stage) {
     if (step >= step_first && step <= step_last) {
+      const char* from = stages + stage * PORTION_STAGE_BYTES;
       StepLoads loads;
 #pragma unroll
       for (int s = 0; s < QK_STEPS; ++s) {
-        const int slot = ((s * 4 + q) ^ k_swizzle) * 8;
-        loads.k_lo[s].v = *(const bf16x8*)(stage + (size_t)row_lo * D + slot);
-        loads.k_hi[s].v = *(const bf16x8*)(stage + (size_t)(row_lo + 4) * D + slot);
+        loads.k_lo[s].v = *(const bf16x8*)(from + read_k + s * 2048);
+        loads.k_hi[s].v = *(const bf16x8*)(from + read_k + s * 2048 + 1024);
       }
 #pragma unroll
-      for (int d = 0; d < D_TILES; ++d)
-        loads.v[d] = *(const bf16x8*)(stage + KEYS * D + (size_t)(d * 16 + c) * KEYS + (q ^ v_swizzle) * 8);
+      for (int d = 0; d < D_TILES; ++d) loads.v[d] = *(const bf16x8*)(from + read_v + d * 1024);
       f32x4 s_lo[COLUMN_TILES], s_hi[COLUMN_TILES];
       scores_of(columns, loads, s_lo, s_hi);
       const int key0 = step * KEYS;
@@ -732,25 +770,26 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
       weigh_and_add(columns, loads, s_lo, s_hi, key0, q, interior, last_key_all,
                     min(max(key0 + 8 * q, low_limit), high_limit), scale_log2);
     }
-    // what was written to `other` is there for everyone, and everyone has read `stage` (a bare barrier:
-    // the loads under way are not to be waited for)
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   };
-  StagedPieces even, odd;  // the pieces of the even and of the odd steps, counted from the first
-  fetch_step(step_first_all, even);
-  fetch_step(step_first_all + 1, odd);
-  write_step(even, stage_0);
-  fetch_step(step_first_all + 2, even);
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  for (int step = step_first_all; step <= step_last_all; step += 2) {  // (a step past the last one is walked empty)
-    walk_step(step, stage_0, stage_1, odd);
-    walk_step(step + 1, stage_1, stage_0, even);
+  fill_step(step_first_all, pages_of_step(step_first_all), 0);
+  fill_step(step_first_all + 1, pages_of_step(step_first_all + 1), 1);
+  StepPageNumbers next_pages = pages_of_step(step_first_all + 2);
+  end_of_step();
+  int stage = 0;
+  for (int step = step_first_all; step <= step_last_all; ++step) {
+    const int ahead = stage == 0 ? 2 : stage - 1;  // (stage + 2) % 3: read last in the step before this one
+    fill_step(step + 2, next_pages, ahead);  // (steps past the last ask for its keys again: the count of loads stays four)
+    next_pages = pages_of_step(step + 3);
+    walk_step(step, stage);
+    end_of_step();
+    stage = stage == 2 ? 0 : stage + 1;
   }
-  // (the last barrier of the walk has passed: LDS is free)
+  // LDS is used once more below: nothing may still be on its way into it
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 
-  // each wave's columns leave through its own half of a stage (16 columns x 128 floats) as whole rows of `out`
+  // each wave's columns leave through 8 KB of LDS of its own (16 columns x 128 floats) as whole rows of `out`
   constexpr int STRIDE = D;
-  float* mine = (float*)(wave < 2 ? stage_0 : stage_1) + (size_t)(wave & 1) * 16 * STRIDE;
+  float* mine = (float*)stages + (size_t)wave * 16 * STRIDE;
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
     float sum = columns.running_sum[t];
