@@ -676,73 +676,41 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   const int step_first = first_key / KEYS, step_last = tokens > 0 ? last_key / KEYS : -1;
   const unsigned page_stride = (unsigned)kv_heads * page_size * D;
   const unsigned head_offset = (unsigned)kv_head * page_size * D;
-  const int low_limit = first_key_all & ~7, high_limit = last_key_all & ~7;
-  auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
 
-  // The four groups of eight keys of a step each lie in one page; pages of 16 or 32 keys (or multiples)
-  // hold two or all four of them.  Looked up through scalar loads, a step before the step's rows are asked for.
-  struct StepPageNumbers {
-    int a, b, c, d;
-    __device__ __forceinline__ int of_group(int i) const { return i == 0 ? a : i == 1 ? b : i == 2 ? c : d; }
-  };
-  const int lookups = page_size % 32 == 0 ? 1 : page_size % 16 == 0 ? 2 : 4;
+  // Pages hold 16 keys, or a power of two beyond (the entry point refuses others): a step lies in two pages or in
+  // one.  Their numbers come through scalar loads, asked for a step before the step's rows are; the entries looked
+  // at are kept within the blocks that hold the item's keys, so that a step that reaches beyond them (the last
+  // one, the first under a window, the steps asked for past the end) reads rows of a page the request holds:
+  // rows of other keys than it wants, all of which the mask weighs with zero.
+  struct StepPages { int first, second; };
+  const int first_block = first_key_all >> page_shift, last_block = last_key_all >> page_shift;
+  const int second_page = page_shift == 4 ? 1 : 0;
   auto pages_of_step = [&](int step) {
-    StepPageNumbers pages;
-    if (page_shift >= 4 && step * KEYS >= first_key_all && step * KEYS + KEYS - 1 <= last_key_all) {  // (see quick_pages)
-      const int* entry = table + ((step * KEYS) >> page_shift);
-      pages.a = entry[0];
-      pages.c = page_shift == 4 ? entry[1] : pages.a;
-      pages.b = pages.a;
-      pages.d = pages.c;
-      return pages;
-    }
-    auto of = [&](int i) { return table[page_index(min(max(step * KEYS + 8 * i, first_key_all), last_key_all))]; };
-    pages.a = of(0);
-    pages.c = lookups >= 2 ? of(2) : pages.a;
-    pages.b = lookups == 4 ? of(1) : pages.a;
-    pages.d = lookups == 4 ? of(3) : pages.c;
-    return pages;
+    const int block = (step * KEYS) >> page_shift;
+    return StepPages{table[min(max(block, first_block), last_block)],
+                     table[min(max(block + second_page, first_block), last_block)]};
   };
   // What this lane asks for in every step: of K the piece 4 wave + lane / 16 of row lane % 16 of the "lo" tile
   // (key 8 (row / 4) + row % 4 of the step) and of the same row of the "hi" tile (four keys on: 64 bytes on in
   // the page); of V^T the keys 8 (lane / 16) .. + 7 of rows 32 wave + lane % 16 and sixteen further (256 bytes on).
+  // So an address is the page's number times the bytes of a page on top of what is fixed for the lane and, with
+  // pages of more than 32 keys, for the step.
   const int row_key = 8 * (c >> 2) + (c & 3);
   const unsigned k_piece = 4 * wave + q;
   const unsigned v_row = 32 * wave + c;
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) void*)stages;
-  // Steps that lie wholly inside the item's keys, in pages of a power of two from 16 keys on, need no more than
-  // a page number times the bytes of a page on top of what is fixed for the lane (and, with pages of more than
-  // 32 keys, for the step); the others (the first steps under a window, the last one, odd page sizes) go the long way.
-  const bool quick_pages = page_shift >= 4;
   const unsigned in_page = (unsigned)page_size - 1;
   const char* k_lane = (const char*)(keys + (head_offset + (k_piece * page_size + ((unsigned)row_key & in_page)) * KEY_PIECE));
   const char* v_lane = (const char*)(values + (head_offset + ((8u * q) & in_page) * D + v_row * VALUE_PIECE));
   const unsigned page_bytes = page_stride * 2;
   const bool k_upper = c >= 8, v_upper = q >= 2;  // which of a step's two pages of 16 keys
-  auto fill_step = [&](int step, const StepPageNumbers& pages, int stage) {
-    const int key0 = step * KEYS;
+  auto fill_step = [&](int step, const StepPages& pages, int stage) {
     const unsigned to = __builtin_amdgcn_readfirstlane(lds_base + (unsigned)stage * PORTION_STAGE_BYTES + (unsigned)wave * 2048);
-    const char *k_from, *k_from_hi, *v_from;
-    if (quick_pages && key0 >= first_key_all && key0 + KEYS - 1 <= last_key_all) {
-      const unsigned of_step = (unsigned)key0 & in_page;  // (0 unless a page holds several steps)
-      k_from = k_lane + (size_t)(unsigned)(k_upper ? pages.c : pages.a) * page_bytes + of_step * (KEY_PIECE * 2);
-      k_from_hi = k_from + 4 * KEY_PIECE * 2;
-      v_from = v_lane + (size_t)(unsigned)(v_upper ? pages.c : pages.a) * page_bytes + of_step * (D * 2);
-    } else {
-      // keys outside the item's range are read from a key inside it (their weights are zero), so that no page is
-      // touched that the request does not hold
-      const bf16_t* page = keys + (size_t)(unsigned)pages.of_group(row_key >> 3) * page_stride + head_offset;
-      const int key = min(max(key0 + row_key, first_key_all), last_key_all);
-      const int key_hi = min(max(key0 + row_key + 4, first_key_all), last_key_all);
-      k_from = (const char*)(page + (k_piece * page_size + (key - page_index(key) * page_size)) * KEY_PIECE);
-      k_from_hi = (const char*)(page + (k_piece * page_size + (key_hi - page_index(key_hi) * page_size)) * KEY_PIECE);
-      const int v_key = min(max(key0 + 8 * q, low_limit), high_limit);
-      const int v_offset = v_key - page_index(v_key) * page_size;
-      v_from = (const char*)(values + (size_t)(unsigned)pages.of_group(q) * page_stride +
-                             (head_offset + ((unsigned)v_offset * D + v_row * VALUE_PIECE)));
-    }
+    const unsigned of_step = (unsigned)(step * KEYS) & in_page;  // (0 unless a page holds several steps)
+    const char* k_from = k_lane + (size_t)(unsigned)(k_upper ? pages.second : pages.first) * page_bytes + of_step * (KEY_PIECE * 2);
+    const char* v_from = v_lane + (size_t)(unsigned)(v_upper ? pages.second : pages.first) * page_bytes + of_step * (D * 2);
     load_to_lds((const bf16_t*)k_from, to);
-    load_to_lds((const bf16_t*)k_from_hi, to + 1024);
+    load_to_lds((const bf16_t*)(k_from + 4 * KEY_PIECE * 2), to + 1024);
     load_to_lds((const bf16_t*)v_from, to + KEYS * D * 2);
     load_to_lds((const bf16_t*)(v_from + 16 * VALUE_PIECE * 2), to + KEYS * D * 2 + 1024);
   };
@@ -766,22 +734,25 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
       f32x4 s_lo[COLUMN_TILES], s_hi[COLUMN_TILES];
       scores_of(columns, loads, s_lo, s_hi);
       const int key0 = step * KEYS;
-      const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
-      weigh_and_add(columns, loads, s_lo, s_hi, key0, q, interior, last_key_all,
-                    min(max(key0 + 8 * q, low_limit), high_limit), scale_log2);
+      const bool interior = key0 >= first_key_all && key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
+      // (which keys' values the lane really read: those of a block that the item's keys lie in)
+      const int value_block = min(max((key0 + 8 * q) >> page_shift, first_block), last_block);
+      const int value_key = (value_block << page_shift) + ((key0 + 8 * q) & (int)in_page);
+      weigh_and_add(columns, loads, s_lo, s_hi, key0, q, interior, last_key_all, value_key, scale_log2);
     }
   };
   fill_step(step_first_all, pages_of_step(step_first_all), 0);
   fill_step(step_first_all + 1, pages_of_step(step_first_all + 1), 1);
-  StepPageNumbers next_pages = pages_of_step(step_first_all + 2);
+  StepPages next_pages = pages_of_step(step_first_all + 2);
   end_of_step();
   int stage = 0;
   for (int step = step_first_all; step <= step_last_all; ++step) {
+    const StepPages after_next = pages_of_step(step + 3);  // (used a step from now: nothing waits for them here)
     const int ahead = stage == 0 ? 2 : stage - 1;  // (stage + 2) % 3: read last in the step before this one
-    fill_step(step + 2, next_pages, ahead);  // (steps past the last ask for its keys again: the count of loads stays four)
-    next_pages = pages_of_step(step + 3);
+    fill_step(step + 2, next_pages, ahead);  // (steps past the last ask for rows of the last block: the count of loads stays four)
     walk_step(step, stage);
     end_of_step();
+    next_pages = after_next;
     stage = stage == 2 ? 0 : stage + 1;
   }
   // LDS is used once more below: nothing may still be on its way into it
@@ -821,18 +792,19 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
 
 // `work` holds `items` entries as for llmserve_attention_tiles; an item covers at most 4 * column_tiles
 // column tiles (column_tiles 1 or 2), tokens_per_tile = max(1, 16 / (heads /
-// kv_heads)).  page_size a multiple of 8.
+// kv_heads)).  page_size a power of two from 16 on.
 extern "C" int llmserve_attention_portions(const void* qkv, int row_width, void* out, const void* keys,
                                            const void* values, const int* block_tables, int table_width,
                                            const int* positions, const int* work, int items, int column_tiles,
                                            int heads, int kv_heads, int page_size, float scale, int window,
                                            hipStream_t stream) {
   if (items <= 0) return 0;
-  if (heads % kv_heads || page_size % 8 || (column_tiles != 1 && column_tiles != 2)) return ERR_BAD_ARGUMENT;
-  if ((long)kv_heads * page_size * D >= (1L << 31)) return ERR_BAD_ARGUMENT;
+  if (heads % kv_heads || page_size < 16 || (page_size & (page_size - 1)) != 0 || (column_tiles != 1 && column_tiles != 2))
+    return ERR_BAD_ARGUMENT;
+  if ((long)kv_heads * page_size * D >= (1L << 30)) return ERR_BAD_ARGUMENT;  // a page's bytes are counted in 32 bits
   const int group = heads / kv_heads;
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
-  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+  const int page_shift = __builtin_ctz(page_size);
   const dim3 grid(items, kv_heads * ((group + 15) / 16));
   if (column_tiles == 1)
     hipLaunchKernelGGL(attention_portions_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)qkv, row_width,

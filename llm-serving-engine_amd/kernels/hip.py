@@ -732,7 +732,8 @@ class HipKernels:
         launches = [(1, *self._attention_work(batch, group_size, 1, 0, per_tile)[:2])]
         shared = False
         padded = getattr(batch, "padded_to", None) is not None  # a captured step: the same launches whatever it holds
-        if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never" and not padded:
+        whole_pages = group.page_size >= 16 and group.page_size & (group.page_size - 1) == 0  # (what that kernel takes)
+        if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never" and not padded and whole_pages:
             # Prompt portions at this head size may go to the kernel whose waves share each step's K and V
             # through LDS (a quarter of the cache traffic).  Its workgroups walk all their keys step after
             # step, 1.2 us a step whatever the arithmetic, so it is ahead where the walks are many and short:
