@@ -588,6 +588,48 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   }
 }
 
+// Merges the key splits of one (token, head): out = sum_s acc_s * 2^(m_s - m) / sum_s l_s *
+// 2^(m_s - m), in split order (the maxima are kept in units of log2).  A second kernel rather than "the last workgroup merges": a
+// workgroup that reads what others wrote needs the other chiplets' L2 written back first, and
+// that costs more than this launch.
+// One wave a (token, head), at most 64 splits: lane s asks for split s's maximum and sum (one trip to
+// memory for all of them, where a loop over the splits made one after the other: nine splits took
+// 14.6 us, thirty-three 41), the wave agrees on the largest and on the total, and every lane then adds
+// up its dimensions over the splits, whose partial sums it asks for eight at a time.
+#define MERGE_SPLITS_MAX 64
+__global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ partial_acc,
+                                                               const float* __restrict__ partial_ml,
+                                                               bf16_t* __restrict__ out, int splits) {
+  const size_t pair = blockIdx.x;  // row * heads + head
+  const int lane = threadIdx.x;
+  const float2 mine = lane < splits ? *(const float2*)(partial_ml + (pair * splits + lane) * 2) : make_float2(-INFINITY, 0.f);
+  const float best = wave_max(mine.x);
+  const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
+  const float total = wave_sum(mine.y * weight);  // (lanes beyond the splits add 0)
+  const float inverse = total > 0.f ? 1.f / total : 0.f;
+  const float* acc = partial_acc + pair * splits * D;
+  for (int d = lane; d < D; d += WAVE) {
+    float sum = 0.f;
+    for (int first = 0; first < splits; first += 8) {
+      float part[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) part[i] = acc[(size_t)min(first + i, splits - 1) * D + d];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float w = __shfl(weight, min(first + i, MERGE_SPLITS_MAX - 1), WAVE);
+        if (first + i < splits && w != 0.f) sum += part[i] * w;
+      }
+    }
+    out[pair * D + d] = (bf16_t)(sum * inverse);
+  }
+}
+
+static int launch_merge(float* partial_acc, float* partial_ml, void* out, int splits, size_t pairs, hipStream_t stream) {
+  hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)pairs), dim3(WAVE), 0, stream, partial_acc, partial_ml,
+                     (bf16_t*)out, splits);
+  return LAUNCH_STATUS();
+}
+
 // ---------------------------------------------------------------------------- prompt portions, D = 128
 // For portions of many tokens the kernel above reads every key once per few tokens, and what bounds it
 // then is the path from the caches into the registers (every wave asks for its own 16 KB a step).  This
@@ -616,10 +658,11 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* from, unsigned to) {
 
 template <int COLUMN_TILES>
 __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
-    const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, const bf16_t* __restrict__ keys,
+    const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
+    float* __restrict__ partial_ml, const bf16_t* __restrict__ keys,
     const bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
-    int page_size, int page_shift, float scale, int window) {
+    int page_size, int page_shift, float scale, int window, int splits) {
   __shared__ __attribute__((aligned(1024))) char stages[PORTION_STAGES * PORTION_STAGE_BYTES];
   const int group = heads / kv_heads;
   const int kv_head = blockIdx.y % kv_heads, head_tile = blockIdx.y / kv_heads;
@@ -672,7 +715,11 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
 #pragma unroll
     for (int s = 0; s < QK_STEPS; ++s) asm volatile("" ::"v"(columns.query[t][s].v));
 
-  const int step_first_all = first_key_all / KEYS, step_last_all = last_key_all / KEYS;
+  // the item's steps, of which this workgroup walks one of `splits` runs (blockIdx.z; possibly none)
+  const int step_first_item = first_key_all / KEYS, step_last_item = last_key_all / KEYS;
+  const int per_split = (step_last_item - step_first_item + splits) / splits;
+  const int step_first_all = step_first_item + (int)blockIdx.z * per_split;
+  const int step_last_all = min(step_last_item, step_first_all + per_split - 1);
   const int step_first = first_key / KEYS, step_last = tokens > 0 ? last_key / KEYS : -1;
   const unsigned page_stride = (unsigned)kv_heads * page_size * D;
   const unsigned head_offset = (unsigned)kv_head * page_size * D;
@@ -758,18 +805,22 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   // LDS is used once more below: nothing may still be on its way into it
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 
-  // each wave's columns leave through 8 KB of LDS of its own (16 columns x 128 floats) as whole rows of `out`
+  // each wave's columns leave through 8 KB of LDS of its own (16 columns x 128 floats) as whole rows: of `out`,
+  // divided by the sum of weights, or (splits > 1) of the split's partial sums as they are, with the column's
+  // reference maximum and sum of weights beside them, for the kernel that merges
   constexpr int STRIDE = D;
   float* mine = (float*)stages + (size_t)wave * 16 * STRIDE;
+  float2* mine_ml = (float2*)((float*)stages + 4 * 16 * STRIDE) + wave * 16;
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
     float sum = columns.running_sum[t];
     sum += __shfl_xor(sum, 16, WAVE);
     sum += __shfl_xor(sum, 32, WAVE);
-    const float inverse = sum > 0.f ? 1.f / sum : 0.f;
+    const float inverse = splits > 1 ? 1.f : sum > 0.f ? 1.f / sum : 0.f;
 #pragma unroll
     for (int d = 0; d < D_TILES; ++d)
       *(f32x4*)(mine + (size_t)c * STRIDE + d * 16 + 4 * q) = columns.acc[t][d] * inverse;
+    if (splits > 1 && q == 0) mine_ml[c] = make_float2(columns.running_max[t], sum);
     // lane (column l / 4, quarter l % 4) writes 32 values of the column's row
     const int column = lane >> 2, quarter = lane & 3;
     int token, head_here;
@@ -777,14 +828,23 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
     map.of(t, column, token, head_here, live);
     if (live) {
       const int head = kv_head * group + head_tile * 16 + head_here;
-      bf16_t* dst = out + ((size_t)(row0 + token) * heads + head) * D + quarter * 32;
+      const float* from = mine + (size_t)column * STRIDE + quarter * 32;
+      if (splits > 1) {
+        const size_t slot = ((size_t)(row0 + token) * heads + head) * splits + blockIdx.z;
+        float* dst = partial_acc + slot * D + quarter * 32;
 #pragma unroll
-      for (int piece = 0; piece < 4; ++piece) {
-        const f32x4 lo = *(const f32x4*)(mine + (size_t)column * STRIDE + quarter * 32 + piece * 8);
-        const f32x4 hi = *(const f32x4*)(mine + (size_t)column * STRIDE + quarter * 32 + piece * 8 + 4);
-        bf16_t packed[8] = {(bf16_t)lo[0], (bf16_t)lo[1], (bf16_t)lo[2], (bf16_t)lo[3],
-                            (bf16_t)hi[0], (bf16_t)hi[1], (bf16_t)hi[2], (bf16_t)hi[3]};
-        *(uint4*)(dst + piece * 8) = *(const uint4*)packed;
+        for (int piece = 0; piece < 8; ++piece) *(f32x4*)(dst + piece * 4) = *(const f32x4*)(from + piece * 4);
+        if (quarter == 0) *(float2*)(partial_ml + slot * 2) = mine_ml[column];
+      } else {
+        bf16_t* dst = out + ((size_t)(row0 + token) * heads + head) * D + quarter * 32;
+#pragma unroll
+        for (int piece = 0; piece < 4; ++piece) {
+          const f32x4 lo = *(const f32x4*)(from + piece * 8);
+          const f32x4 hi = *(const f32x4*)(from + piece * 8 + 4);
+          bf16_t packed[8] = {(bf16_t)lo[0], (bf16_t)lo[1], (bf16_t)lo[2], (bf16_t)lo[3],
+                              (bf16_t)hi[0], (bf16_t)hi[1], (bf16_t)hi[2], (bf16_t)hi[3]};
+          *(uint4*)(dst + piece * 8) = *(const uint4*)packed;
+        }
       }
     }
   }
@@ -793,71 +853,42 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
 // `work` holds `items` entries as for llmserve_attention_tiles; an item covers at most 4 * column_tiles
 // column tiles (column_tiles 1 or 2), tokens_per_tile = max(1, 16 / (heads /
 // kv_heads)).  page_size a power of two from 16 on.
-extern "C" int llmserve_attention_portions(const void* qkv, int row_width, void* out, const void* keys,
+extern "C" int llmserve_attention_portions(const void* qkv, int row_width, void* out, float* partial_acc,
+                                           float* partial_ml, const void* keys,
                                            const void* values, const int* block_tables, int table_width,
                                            const int* positions, const int* work, int items, int column_tiles,
-                                           int heads, int kv_heads, int page_size, float scale, int window,
-                                           hipStream_t stream) {
+                                           int rows, int heads, int kv_heads, int page_size, float scale, int window,
+                                           int splits, hipStream_t stream) {
   if (items <= 0) return 0;
   if (heads % kv_heads || page_size < 16 || (page_size & (page_size - 1)) != 0 || (column_tiles != 1 && column_tiles != 2))
     return ERR_BAD_ARGUMENT;
+  if (splits < 1 || splits > MERGE_SPLITS_MAX || (splits > 1 && (!partial_acc || !partial_ml))) return ERR_BAD_ARGUMENT;
   if ((long)kv_heads * page_size * D >= (1L << 30)) return ERR_BAD_ARGUMENT;  // a page's bytes are counted in 32 bits
   const int group = heads / kv_heads;
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
   const int page_shift = __builtin_ctz(page_size);
-  const dim3 grid(items, kv_heads * ((group + 15) / 16));
+  const dim3 grid(items, kv_heads * ((group + 15) / 16), splits);
   if (column_tiles == 1)
     hipLaunchKernelGGL(attention_portions_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)qkv, row_width,
-                       (bf16_t*)out, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width, positions,
-                       work, heads, kv_heads, tokens_per_tile, page_size, page_shift, scale, window);
+                       (bf16_t*)out, partial_acc, partial_ml, (const bf16_t*)keys, (const bf16_t*)values, block_tables,
+                       table_width, positions, work, heads, kv_heads, tokens_per_tile, page_size, page_shift, scale,
+                       window, splits);
   else
     hipLaunchKernelGGL(attention_portions_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)qkv, row_width,
-                       (bf16_t*)out, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width, positions,
-                       work, heads, kv_heads, tokens_per_tile, page_size, page_shift, scale, window);
-  return LAUNCH_STATUS();
+                       (bf16_t*)out, partial_acc, partial_ml, (const bf16_t*)keys, (const bf16_t*)values, block_tables,
+                       table_width, positions, work, heads, kv_heads, tokens_per_tile, page_size, page_shift, scale,
+                       window, splits);
+  const int status = LAUNCH_STATUS();
+  if (status != 0 || splits == 1) return status;
+  return launch_merge(partial_acc, partial_ml, out, splits, (size_t)rows * heads, stream);
 }
 #else
-extern "C" int llmserve_attention_portions(const void*, int, void*, const void*, const void*, const int*, int,
-                                           const int*, const int*, int, int, int, int, int, float, int, hipStream_t) {
+extern "C" int llmserve_attention_portions(const void*, int, void*, float*, float*, const void*, const void*, const int*,
+                                           int, const int*, const int*, int, int, int, int, int, int, float, int, int,
+                                           hipStream_t) {
   return ERR_BAD_ARGUMENT;  // built for head size 128 only
 }
 #endif
-
-// Merges the key splits of one (token, head): out = sum_s acc_s * 2^(m_s - m) / sum_s l_s *
-// 2^(m_s - m), in split order (the maxima are kept in units of log2).  A second kernel rather than "the last workgroup merges": a
-// workgroup that reads what others wrote needs the other chiplets' L2 written back first, and
-// that costs more than this launch.
-// One wave a (token, head), at most 64 splits: lane s asks for split s's maximum and sum (one trip to
-// memory for all of them, where a loop over the splits made one after the other: nine splits took
-// 14.6 us, thirty-three 41), the wave agrees on the largest and on the total, and every lane then adds
-// up its dimensions over the splits, whose partial sums it asks for eight at a time.
-#define MERGE_SPLITS_MAX 64
-__global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ partial_acc,
-                                                               const float* __restrict__ partial_ml,
-                                                               bf16_t* __restrict__ out, int splits) {
-  const size_t pair = blockIdx.x;  // row * heads + head
-  const int lane = threadIdx.x;
-  const float2 mine = lane < splits ? *(const float2*)(partial_ml + (pair * splits + lane) * 2) : make_float2(-INFINITY, 0.f);
-  const float best = wave_max(mine.x);
-  const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
-  const float total = wave_sum(mine.y * weight);  // (lanes beyond the splits add 0)
-  const float inverse = total > 0.f ? 1.f / total : 0.f;
-  const float* acc = partial_acc + pair * splits * D;
-  for (int d = lane; d < D; d += WAVE) {
-    float sum = 0.f;
-    for (int first = 0; first < splits; first += 8) {
-      float part[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) part[i] = acc[(size_t)min(first + i, splits - 1) * D + d];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float w = __shfl(weight, min(first + i, MERGE_SPLITS_MAX - 1), WAVE);
-        if (first + i < splits && w != 0.f) sum += part[i] * w;
-      }
-    }
-    out[pair * D + d] = (bf16_t)(sum * inverse);
-  }
-}
 
 // waves of a workgroup of the fused decode form: eight walk a tile's keys where the registers allow it
 #ifndef FUSED_WAVES
@@ -947,7 +978,5 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
     return ERR_BAD_ARGUMENT;
   }
   if (status != 0 || splits == 1 || unmerged) return status;
-  hipLaunchKernelGGL(attention_merge_kernel, dim3(rows * heads), dim3(WAVE), 0, stream, partial_acc, partial_ml,
-                     (bf16_t*)out, splits);
-  return LAUNCH_STATUS();
+  return launch_merge(partial_acc, partial_ml, out, splits, (size_t)rows * heads, stream);
 }

@@ -65,7 +65,7 @@ _SIGNATURES = {
     "llmserve_attention_generic": "pipipppippiiiiifipfp",
     "llmserve_attention_f32": "pippppppippiiiiiifiipfp",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
-    "llmserve_attention_portions": "pippppippiiiiifip",
+    "llmserve_attention_portions": "pippppppippiiiiiifiip",
     "llmserve_attention_can_fuse": "i",
     "llmserve_argmax": "ppppiip",
     "llmserve_argmax_static": "ppiip",
@@ -139,6 +139,7 @@ class HipKernels:
         self.device = torch.device(device)
         self.library_products = library_products
         self.shared_portions = shared_portions
+        self.portion_splits: int | None = None  # runs of keys a workgroup of that kernel's items is cut into; None: by rule
         self.merge_in_product = True  # decode attention leaves its key splits to the product that reads them
         self.merge_weight_bytes = 8 << 20  # ... where that product's weight is at most this large (measured at 4.7 and 25.7 MB)
         name = torch.cuda.get_device_properties(self.device).gcnArchName
@@ -747,10 +748,15 @@ class HipKernels:
                 steps * kv_heads * head_tiles >= (8 * longest + 110) * longest
             )
         if shared:
+            splits = int(getattr(self, "portion_splits", None) or 1)
+            partial_acc = partial_ml = None
+            if splits > 1:
+                partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), torch.float32)
+                partial_ml = self._empty((tokens * heads * splits * 2,), torch.float32)
             status = library.llmserve_attention_portions(
-                _pointer(qkv), layout.width, _pointer(out), _pointer(cell.keys), _pointer(cell.values),
-                _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items,
-                2, heads, kv_heads, group.page_size, scale, window, self._stream,
+                _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml), _pointer(cell.keys),
+                _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work),
+                items, 2, tokens, heads, kv_heads, group.page_size, scale, window, splits, self._stream,
             )
             _check(status, "paged_attention")
         elif batch.max_query_length > per_tile:

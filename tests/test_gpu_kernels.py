@@ -291,16 +291,20 @@ def test_paged_attention_finds_a_far_key_among_hundreds(kernels, dtype):
         torch.testing.assert_close(out[0], rounded(v, dtype)[far, 0], atol=5e-2, rtol=0)
 
 
+@pytest.mark.parametrize("splits", [1, 3])
 @pytest.mark.parametrize("window", [None, 21, 64])
-@pytest.mark.parametrize("heads,kv_heads,page", [(12, 2, 16), (28, 4, 8), (40, 2, 16), (5, 5, 24), (3, 1, 32), (40, 8, 16), (10, 2, 16)])
-def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, window):
+@pytest.mark.parametrize("heads,kv_heads,page", [(12, 2, 16), (28, 4, 8), (40, 2, 16), (5, 5, 24), (3, 1, 32), (40, 8, 16), (10, 2, 16), (12, 2, 64), (7, 1, 128)])
+def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, window, splits):
     """At head size 128 prompt portions may go to the kernel whose four waves share each step's K and V
-    through LDS: portions that fill its workgroups, that leave waves empty, that end inside a step of 32
-    keys and that begin long after the sequence's start, with and without a window."""
+    through LDS (pages of a power of two from 16 keys on; the others stay with the kernel above): portions that
+    fill its workgroups, that leave waves empty, that end inside a step of 32 keys and that begin long after the
+    sequence's start, with and without a window, whole or in three runs of keys that a second kernel merges
+    (some of them empty: a request of five keys has one step)."""
     from llmserve_amd.kernels import HipKernels
 
     dim, dtype = 128, torch.bfloat16
     shared = HipKernels(dtype, shared_portions="always")
+    shared.portion_splits = splits
     apart = HipKernels(dtype, shared_portions="never")
     lengths = [130, 97, 33, 300, 64, 5]
     counts = [130, 40, 33, 70, 17, 3]
