@@ -736,19 +736,32 @@ class HipKernels:
         whole_pages = group.page_size >= 16 and group.page_size & (group.page_size - 1) == 0  # (what that kernel takes)
         if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never" and not padded and whole_pages:
             # Prompt portions at this head size may go to the kernel whose waves share each step's K and V
-            # through LDS (a quarter of the cache traffic).  Its workgroups walk all their keys step after
-            # step, 1.2 us a step whatever the arithmetic, so it is ahead where the walks are many and short:
-            # measured at 5 to 7 query heads a kv head over thirty shapes, it wins (by up to a third) where the
-            # steps of all walks together are more than 8 x longest + 110 times the longest walk (sixteen
-            # prompts of 512 tokens, 64 of 128, eight of 1,024 at the 7B sizes), and loses elsewhere (one
-            # prompt of any length, a portion behind a long context, four prompts of 4,096).
+            # through LDS (a quarter of the cache traffic; what bounds the kernel above over long walks is the
+            # path from the caches into the registers).  Its workgroups take 128 columns and walk all their keys,
+            # so there are few of them: 192 for a 2,048-token portion of the 1.5B sizes, where the chip holds 512
+            # and the kernel above would start 768.  So it is taken where it has 400 workgroups by itself (or
+            # half as many very short walks), and where walks of 256 steps or more can be cut into runs of at
+            # least 64 steps that a second kernel merges, 768 workgroups or so.  Measured (us, this kernel against
+            # the one above, the same box and process): at 12 / 2 heads one prompt of 8,192 tokens 289 / 333,
+            # eight of 2,048 202 / 236, sixteen of 512 47 / 71, a 2,048-token portion behind 8,192 keys 142 / 152
+            # (four runs), behind 16,384 245-254 / 305-315, behind 32,704 455-485 / 593-706, 512 tokens behind
+            # 32,704 168 / 272; at 28 / 4 heads (448 workgroups a 2,048-token portion) behind 4,096 to 8,192 keys
+            # 133-262 / 142-287, behind 32,704 1,035 / 1,223, one prompt of 8,192 582 / 729; left to the kernel
+            # above at 12 / 2 heads: one prompt of 2,048 to 6,144 tokens (43 / 66, 95 / 116, 188 / 209 the other
+            # way round) and a portion behind up to 6,144 keys (112 / 116).
             work, items, steps = self._attention_work(batch, group_size, 8, per_tile, None)
-            longest = batch.max_context_length / 32
-            shared = self.shared_portions == "always" or (
-                steps * kv_heads * head_tiles >= (8 * longest + 110) * longest
-            )
+            groups = items * kv_heads * head_tiles
+            longest = -(-batch.max_context_length // 32)
+            splits = 1
+            if groups >= 400 or (groups >= 192 and longest <= 32):
+                shared = True
+            elif longest >= 256:
+                splits = max(1, min(8, longest // 64, -(-768 // groups)))
+                shared = groups * splits >= 384
+            if self.portion_splits:
+                splits = int(self.portion_splits)
+            shared = shared or self.shared_portions == "always"
         if shared:
-            splits = int(getattr(self, "portion_splits", None) or 1)
             partial_acc = partial_ml = None
             if splits > 1:
                 partial_acc = self._empty((tokens * heads * splits * layout.head_dim,), torch.float32)
