@@ -166,11 +166,11 @@ __device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, St
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[i] = fmaf(i < 4 ? s_lo[t][i] : s_hi[t][i - 4], scale_log2, -reference);
     if (!interior) {
+      // key0 + 8q + i outside [first, position], counted from the lane's first key (nothing to add per key)
+      const int last_seen = columns.position[t] - (key0 + 8 * q), first_seen = columns.first[t] - (key0 + 8 * q);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int key = key0 + 8 * q + i;
-        if (key > columns.position[t] || key < columns.first[t]) x[i] = -INFINITY;
-      }
+      for (int i = 0; i < 8; ++i)
+        if (i > last_seen || i < first_seen) x[i] = -INFINITY;
     }
     // (the largest of three in one instruction, written out: through fmaxf the compiler first passes every
     // score through a v_max with itself, thirteen instructions for eight scores where four do)
@@ -639,7 +639,7 @@ static int launch_merge(float* partial_acc, float* partial_ml, void* out, int sp
 // key split inside the workgroup, nothing to merge).  A step's 32 K rows and 128 x 32 V^T block (16 KB)
 // go from memory straight into LDS (global_load_lds_dwordx4: each lane names its own 16 bytes of memory,
 // and the 64 lanes of an instruction fill 1 KB of LDS in lane order), sixteen such instructions a step,
-// four from each wave, two steps ahead of their use, into one of three stages.  Who asks for what is
+// four from each wave, a pair of steps ahead of their use, into one of four stages.  Who asks for what is
 // chosen so that LDS holds the operands as the products read them, a whole wave 1 KB in a row:
 //   K: chunks 2j and 2j+1 (1 KB each) = pieces 4j .. 4j+3 (eight elements each) of the 16 rows of the "lo"
 //      and of the "hi" tile of the first product (for lane (c, q) piece 4j + q of row c)
@@ -647,10 +647,10 @@ static int launch_merge(float* partial_acc, float* partial_ml, void* out, int sp
 // The loads are written in assembly: the compiler knows that such a load writes LDS but not where, and
 // makes every later read of LDS wait for all of them, so they could not run ahead.  Here the waits are
 // counted by hand (the loop holds no other vector memory instruction): before the barrier that ends a
-// step, every wave waits until only its four youngest loads (the step after next) are still under way.
+// pair of steps, every wave waits for the loads it asked for at the pair's beginning.
 #if HEAD_DIM == 128
 constexpr int PORTION_STAGE_BYTES = 2 * KEYS * D * 2;  // K rows, then V^T rows
-constexpr int PORTION_STAGES = 3;
+constexpr int PORTION_STAGES = 4;
 
 __device__ __forceinline__ void load_to_lds(const bf16_t* from, unsigned to) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(to), "v"(from) : "memory");
@@ -761,14 +761,15 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
     load_to_lds((const bf16_t*)v_from, to + KEYS * D * 2);
     load_to_lds((const bf16_t*)(v_from + 16 * VALUE_PIECE * 2), to + KEYS * D * 2 + 1024);
   };
-  // every wave has read the stage that the next loads fill, and what it asked for two steps ago has arrived
-  // (its four youngest loads may still be under way); after the barrier that holds for all waves
-  auto end_of_step = [&]() { asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  // Two steps a barrier: the four stages are two pairs, one being read while the other is filled.  At the end of
+  // a pair of steps every wave has read its stages and waits for what it asked for at the pair's beginning; after
+  // the barrier that holds for all waves.
+  auto end_of_pair = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
   const float scale_log2 = scale * 1.44269504088896f;
   const unsigned read_k = lane * 16, read_v = KEYS * D * 2 + lane * 16;  // this lane's bytes within a stage
   auto walk_step = [&](int step, int stage) {
-    if (step >= step_first && step <= step_last) {
+    if (step >= step_first && step <= min(step_last, step_last_all)) {
       const char* from = stages + stage * PORTION_STAGE_BYTES;
       StepLoads loads;
 #pragma unroll
@@ -790,17 +791,21 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   };
   fill_step(step_first_all, pages_of_step(step_first_all), 0);
   fill_step(step_first_all + 1, pages_of_step(step_first_all + 1), 1);
-  StepPages next_pages = pages_of_step(step_first_all + 2);
-  end_of_step();
-  int stage = 0;
-  for (int step = step_first_all; step <= step_last_all; ++step) {
-    const StepPages after_next = pages_of_step(step + 3);  // (used a step from now: nothing waits for them here)
-    const int ahead = stage == 0 ? 2 : stage - 1;  // (stage + 2) % 3: read last in the step before this one
-    fill_step(step + 2, next_pages, ahead);  // (steps past the last ask for rows of the last block: the count of loads stays four)
-    walk_step(step, stage);
-    end_of_step();
-    next_pages = after_next;
-    stage = stage == 2 ? 0 : stage + 1;
+  StepPages next_even = pages_of_step(step_first_all + 2), next_odd = pages_of_step(step_first_all + 3);
+  end_of_pair();
+  int pair = 0;
+  for (int step = step_first_all; step <= step_last_all; step += 2) {
+    // (page numbers for the pair after next: used an iteration from now, nothing waits for them here)
+    const StepPages after_even = pages_of_step(step + 4), after_odd = pages_of_step(step + 5);
+    // (steps past the last ask for rows of the last block)
+    fill_step(step + 2, next_even, 2 - 2 * pair);
+    fill_step(step + 3, next_odd, 3 - 2 * pair);
+    walk_step(step, 2 * pair);
+    walk_step(step + 1, 2 * pair + 1);
+    end_of_pair();
+    next_even = after_even;
+    next_odd = after_odd;
+    pair = 1 - pair;
   }
   // LDS is used once more below: nothing may still be on its way into it
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
