@@ -652,8 +652,13 @@ static int launch_merge(float* partial_acc, float* partial_ml, void* out, int sp
 constexpr int PORTION_STAGE_BYTES = 2 * KEYS * D * 2;  // K rows, then V^T rows
 constexpr int PORTION_STAGES = 4;
 
+// (the instruction takes its place in LDS from M0; the register is given back as it was, the compiler is not told of it)
 __device__ __forceinline__ void load_to_lds(const bf16_t* from, unsigned to) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(to), "v"(from) : "memory");
+  unsigned kept;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(kept)
+               : "s"(to), "v"(from)
+               : "memory");
 }
 
 template <int COLUMN_TILES>
