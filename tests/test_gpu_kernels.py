@@ -309,6 +309,14 @@ def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, wind
     lengths = [130, 97, 33, 300, 64, 5]
     counts = [130, 40, 33, 70, 17, 3]
     batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=heads)
+    if window:
+        # blocks that the window has passed are given back in the engine: here their table entries name a page
+        # nobody wrote (all NaN), which a kernel that looked there would carry into its sums
+        tables = batch.groups[0].block_tables.cpu()
+        unwritten = int(torch.isnan(cell.keys.float()).flatten(1).all(dim=1).nonzero()[0])
+        for index, (length, count) in enumerate(zip(lengths, counts)):
+            tables[index, : max(0, length - count - window + 1) // page] = unwritten
+        batch.groups[0].block_tables.copy_(tables)
     qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
     scale = 0.11
     out = shared.paged_attention(qkv, layout, batch, cell, scale, window).cpu().double()
