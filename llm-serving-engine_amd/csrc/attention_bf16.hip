@@ -88,6 +88,8 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
   const int* slots;           // [rows] page * page_size + offset of each token, negative: store nothing
   int unmerged;               // key splits are left for the reader to merge: each split's result is divided by its own
                               // sum of weights and stored as bfloat16 where partial_acc points, [rows][heads][splits][D]
+  int by_item;                // the splits' partial results are kept by work item (item * tokens_per_tile + token)
+                              // instead of by the step's row: for the few short requests of a step of long portions
 };
 
 // One step's operands as a lane holds them: its slices of the K rows of the two 16-row tiles and,
@@ -559,7 +561,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
 #pragma unroll
         for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
       } else {
-        const size_t slot = (row * heads + head) * splits + blockIdx.z;
+        const size_t kept_as = fused.by_item ? (size_t)(gridDim.x - 1 - blockIdx.x) * tokens_per_tile + token : row;
+        const size_t slot = (kept_as * heads + head) * splits + blockIdx.z;
         if (fused.unmerged) {
           // for the product that merges: [head][split][piece of 8][16 rows][8], the rows of a piece side by
           // side, so that the four lanes of its loads that hold four rows' share of a piece read 64 bytes
@@ -621,6 +624,35 @@ __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __re
       }
     }
     out[pair * D + d] = (bf16_t)(sum * inverse);
+  }
+}
+
+// The same for partial results that are kept by work item: workgroup (item, head) merges the item's tokens one
+// after the other (a few), and writes to the rows that the item names.
+__global__ __launch_bounds__(WAVE) void attention_merge_items_kernel(const float* __restrict__ partial_acc,
+                                                                     const float* __restrict__ partial_ml,
+                                                                     bf16_t* __restrict__ out, const int* __restrict__ work,
+                                                                     int splits, int heads, int group, int tokens_per_tile) {
+  const int* item = work + (size_t)blockIdx.x * 4;
+  const int tokens = group <= 16 ? (item[2] + item[3] + group - 1) / group : item[3];
+  const int head = blockIdx.y, lane = threadIdx.x;
+  for (int token = 0; token < tokens; ++token) {
+    const size_t kept_as = ((size_t)blockIdx.x * tokens_per_tile + token) * heads + head;
+    const size_t pair = ((size_t)item[1] + token) * heads + head;
+    const float2 mine = lane < splits ? *(const float2*)(partial_ml + (kept_as * splits + lane) * 2) : make_float2(-INFINITY, 0.f);
+    const float best = wave_max(mine.x);
+    const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);
+    const float total = wave_sum(mine.y * weight);
+    const float inverse = total > 0.f ? 1.f / total : 0.f;
+    const float* acc = partial_acc + kept_as * splits * D;
+    for (int d = lane; d < D; d += WAVE) {
+      float sum = 0.f;
+      for (int split = 0; split < splits; ++split) {
+        const float w = __shfl(weight, split, WAVE);
+        if (w != 0.f) sum += acc[(size_t)split * D + d] * w;
+      }
+      out[pair * D + d] = (bf16_t)(sum * inverse);
+    }
   }
 }
 
@@ -948,6 +980,9 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // of the step must lie in one of the tiles: a second kernel merges the splits of all rows.
 // With `fuse` tile i is row i, the one token of request i (`work` is not read), qkv is as the projection left it, and the kernel
 // rotates (table of cos and sin per row, pairing) and stores the token's key and value at slots[row] itself.
+// `fuse` = 4 (column_tiles 1, splits > 1): the items are the few short requests of a step that also holds long portions;
+// partial_acc [tiles * tokens_per_tile * heads * splits * D] and partial_ml are kept by item, and only the items' rows
+// are merged and written.
 // `fuse` + 2 leaves the key splits unmerged for a reader that merges them itself (gemm_merged; at most 16 rows):
 // partial_acc is then bfloat16 [heads][splits][D / 8][16 rows][8], each split's result divided by its own sum of
 // weights, and partial_ml [heads][splits][16 rows][2] holds each split's maximum (in units of log2) and sum of
@@ -967,8 +1002,10 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   const int tokens_per_tile = group >= 16 ? 1 : 16 / group;
   const bool unmerged = (fuse & 2) != 0 && splits > 1;  // the splits stay as they are: whoever reads them merges them
   if (unmerged && rows > 16) return ERR_BAD_ARGUMENT;
+  const bool by_item = (fuse & 4) != 0 && splits > 1;  // partial results by work item, merged for the items' rows only
+  if (by_item && ((fuse & 3) != 0 || column_tiles != 1)) return ERR_BAD_ARGUMENT;
   fuse &= 1;
-  FusedDecode fused = {(const float2*)table, pairing, slots, unmerged ? 1 : 0};
+  FusedDecode fused = {(const float2*)table, pairing, slots, unmerged ? 1 : 0, by_item ? 1 : 0};
   int status;
   if (fuse) {
     if (column_tiles != 1 || tiles != rows || !slots || !llmserve_attention_can_fuse(pairing) || (pairing != 0 && !table))
@@ -988,5 +1025,10 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
     return ERR_BAD_ARGUMENT;
   }
   if (status != 0 || splits == 1 || unmerged) return status;
+  if (by_item) {
+    hipLaunchKernelGGL(attention_merge_items_kernel, dim3(tiles, heads), dim3(WAVE), 0, stream, partial_acc, partial_ml,
+                       (bf16_t*)out, work, splits, heads, group, tokens_per_tile);
+    return LAUNCH_STATUS();
+  }
   return launch_merge(partial_acc, partial_ml, out, splits, (size_t)rows * heads, stream);
 }

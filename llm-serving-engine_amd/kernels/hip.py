@@ -784,7 +784,20 @@ class HipKernels:
             if items == 0:
                 continue
             splits, partial_acc, partial_ml = 1, None, None
-            if batch.max_query_length <= per_tile:  # few tiles, maybe long: split the keys
+            by_item = False
+            if shared:
+                # The few short requests (decoded tokens) of a step whose portions went to the other kernel: alone
+                # in this launch, so a long context is walked by one workgroup a kv head (30,000 keys: 237 us) unless
+                # it is cut; their partial results are kept by item, not by the step's rows, which are mostly the
+                # portions'.
+                longest_few = max((chunk.start + chunk.count for chunk in batch.chunks if chunk.count <= per_tile), default=0)
+                steps = -(-longest_few // 32)
+                splits = max(1, min(-(-steps // 32), max(1, 2048 // (items * kv_heads * head_tiles)), 64))
+                if splits > 1:
+                    by_item = True
+                    partial_acc = self._empty((items * per_tile * heads * splits * layout.head_dim,), torch.float32)
+                    partial_ml = self._empty((items * per_tile * heads * splits * 2,), torch.float32)
+            elif batch.max_query_length <= per_tile:  # few tiles, maybe long: split the keys
                 # a wave walks its share of the keys step after step (32 keys each), and a walk of
                 # a few steps costs less than the second kernel that merges splits: split only when
                 # a wave would walk more than 8 steps and the chip has room for more workgroups
@@ -816,7 +829,7 @@ class HipKernels:
             status = library.llmserve_attention_tiles(
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
                 _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
-                group.page_size, scale, window, splits, (1 if fuse is not None else 0) + (2 if unmerged else 0),
+                group.page_size, scale, window, splits, (1 if fuse is not None else 0) + (2 if unmerged else 0) + (4 if by_item else 0),
                 _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), self._stream,
             )
             _check(status, "paged_attention")

@@ -329,6 +329,30 @@ def test_prompt_portions_that_share_keys_through_lds(heads, kv_heads, page, wind
     torch.testing.assert_close(out, other, **TOLERANCE[dtype])
 
 
+@pytest.mark.parametrize("heads,kv_heads", [(12, 2), (40, 2), (7, 7)])
+def test_decoded_tokens_beside_portions_that_share_keys_through_lds(heads, kv_heads):
+    """A step of long portions beside single decoded tokens over long contexts: the portions go to the kernel
+    that shares K and V through LDS, the decoded tokens to a launch of their own whose keys are cut into runs
+    (partial results kept by work item, merged for those rows only); a far key dominates one decoded token."""
+    from llmserve_amd.kernels import HipKernels
+
+    dim, page, dtype = 128, 16, torch.bfloat16
+    shared = HipKernels(dtype, shared_portions="always")
+    lengths, counts = [3100, 4200, 600, 2500, 90], [1, 600, 300, 1, 1]
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=5)
+    q, k, v = per_request[0]
+    k[40] = 3.0 * q[-1, :: heads // kv_heads]  # for the first query head of every kv head this key dominates
+    _rewrite_cell(batch, cell, per_request, page, dtype)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    out = shared.paged_attention(qkv, layout, batch, cell, 1.0, None).cpu().double()
+    expected = []
+    for (q, k, v), count in zip(per_request, counts):
+        full = plain.causal_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), 1.0, None)
+        expected.append(full[-count:].flatten(1))
+    torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
+    torch.testing.assert_close(out[0].view(heads, dim)[0], rounded(per_request[0][2], dtype)[40, 0], atol=5e-2, rtol=0)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("window", [None, 1500])
 def test_paged_attention_portion_of_a_long_context(kernels, window, dtype):
