@@ -18,6 +18,12 @@ the same model in float32, and the 7B and 32B layer sizes.
 
 prints the reference's own kernel-level table instead (one attention layer, context 128, batch
 1/2/4/8, its protocol: scripts/benchmark_triton_paged_attention.py:60-107).
+
+    python bench.py --op prefill-attention
+
+times the paged attention of prompt portions alone (the configuration's heads; whole prompts of 2,048
+and 8,192 tokens, a 2,048-token portion behind 8,192 to 32,704 keys, sixteen prompts of 512) and prints
+microseconds and PFLOP/s, counting the causal half only.
 """
 
 from __future__ import annotations
@@ -59,7 +65,7 @@ def parse() -> argparse.Namespace:
                         help="leave out decoding at contexts of 8k and 30k (batch 8) and 4k (batch 64), and the long prompts")
     parser.add_argument("--skip-other-models", action="store_true",
                         help="leave out the float32 run and the 7B and 32B layer sizes")
-    parser.add_argument("--op", choices=("decode-attention",), default=None,
+    parser.add_argument("--op", choices=("decode-attention", "prefill-attention"), default=None,
                         help="measure one operation alone instead, as the reference's kernel benchmark does")
     return parser.parse_args()
 
@@ -315,6 +321,90 @@ def decode_attention_table(args) -> int:
     return 0
 
 
+def prefill_attention_table(args) -> int:
+    """The engine's paged attention for prompt portions alone, through the call the layers make
+    (`HipKernels.paged_attention`), over pages of random keys and values laid out as the cache manager lays them
+    out: per shape five untimed calls, then five repeats of ten calls between device events.  Flops count the
+    keys a query sees (the causal half of a whole prompt), 4 * head size a (query, key, head)."""
+    import torch
+
+    from llmserve_amd.cache import CacheCell
+    from llmserve_amd.engine.batch import GroupBatch, SequenceChunk, StepBatch
+    from llmserve_amd.kernels import HipKernels
+    from llmserve_amd.parts import HeadLayout, PagedKeyValue
+    from llmserve_amd.weights import read_config, run_dtype
+
+    _, config = read_config(args.config)
+    dtype = run_dtype(args.dtype)
+    device = torch.device("cuda:0")
+    kernels = HipKernels(dtype, device)
+    heads, kv_heads, dim = config.num_attention_heads, config.num_key_value_heads, config.head_dim
+    layout = HeadLayout(heads, kv_heads, dim)
+    need = PagedKeyValue(kv_heads, dim)
+    generator = torch.Generator(device=device).manual_seed(args.seed)
+    shapes = [([2048], [2048]), ([8192], [8192]), ([8192], [2048]), ([16384], [2048]), ([32704], [2048]), ([512] * 16, [512] * 16)]
+    repeats, iterations = 5, 10
+    rows = []
+    for contexts, portions in shapes:
+        blocks = [-(-context // PAGE) for context in contexts]
+        pages, width = sum(blocks) + 1, max(blocks)
+        tables = torch.zeros((len(contexts), width), dtype=torch.int32)
+        positions, sequence, slots, chunks, first_page = [], [], [], [], 0
+        for index, (context, count) in enumerate(zip(contexts, portions)):
+            tables[index, : blocks[index]] = torch.arange(first_page, first_page + blocks[index], dtype=torch.int32)
+            mine = torch.arange(context - count, context)
+            positions.append(mine)
+            sequence.append(torch.full((count,), index))
+            slots.append(first_page * PAGE + mine)
+            chunks.append(SequenceChunk(f"r{index}", index, context - count, count))
+            first_page += blocks[index]
+        ints = lambda values: torch.as_tensor(values, dtype=torch.int32, device=device)
+        starts = [0]
+        for count in portions:
+            starts.append(starts[-1] + count)
+        tokens = sum(portions)
+        group = GroupBatch(PAGE, tables.to(device), ints(torch.cat(slots)), width)
+        batch = StepBatch(
+            num_tokens=tokens, chunks=chunks, token_ids=ints([0] * tokens), positions=ints(torch.cat(positions)),
+            token_sequence=ints(torch.cat(sequence)), query_start=ints(starts), context_lengths=ints(contexts),
+            state_slots=ints(list(range(len(contexts)))), groups=[group], logit_rows=ints([]), num_logit_rows=0,
+            max_query_length=max(portions), max_context_length=max(contexts),
+        )
+        fields = {name: torch.randn((pages, *shape), generator=generator, device=device).to(dtype)
+                  for name, shape in need.page_fields(PAGE).items()}
+        cell = CacheCell(need, True, 0, fields=fields)
+        qkv = torch.randn((tokens, layout.width), generator=generator, device=device).to(dtype)
+        scale = dim ** -0.5
+
+        def run_once() -> None:
+            kernels.paged_attention(qkv, layout, batch, cell, scale, None)
+
+        with torch.inference_mode():
+            for _ in range(5):
+                run_once()
+            torch.cuda.synchronize()
+            times = []
+            for _ in range(repeats):
+                began, ended = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                began.record()
+                for _ in range(iterations):
+                    run_once()
+                ended.record()
+                ended.synchronize()
+                times.append(began.elapsed_time(ended) / iterations * 1e3)
+        flops = sum(4.0 * heads * dim * (count * (context - count) + count * (count + 1) / 2) for context, count in zip(contexts, portions))
+        median = statistics.median(times)
+        rows.append({"contexts": f"{len(contexts)} x {contexts[0]}", "portion": portions[0], "us": round(median, 1),
+                     "us_min": round(min(times), 1), "us_max": round(max(times), 1),
+                     "pflops": round(flops / median / 1e9, 3), "frac": round(flops / median / 1e9 / (PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"] / 1e15), 3)})
+        del fields, cell, qkv
+    print(json.dumps({
+        "op": "prefill-attention", "dtype": args.dtype, "repeats": repeats, "micro_iterations": iterations,
+        "sizes": f"Hq{heads} Hkv{kv_heads} D{dim}, page {PAGE}", "summaries": rows,
+    }))
+    return 0
+
+
 def main() -> int:
     args = parse()
     if args.gpus != 1:
@@ -322,6 +412,8 @@ def main() -> int:
         return 2
     if args.op == "decode-attention":
         return decode_attention_table(args)
+    if args.op == "prefill-attention":
+        return prefill_attention_table(args)
 
     import torch
 
