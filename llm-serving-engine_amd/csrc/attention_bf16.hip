@@ -225,7 +225,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
     bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
     int page_size, int page_shift, float scale, int window, int splits, FusedDecode fused) {
-  extern __shared__ float lds[];  // [WAVES][16 columns][D + 2]
+  extern __shared__ float lds[];  // [WAVES][16 columns][D + 4]
   if (FUSED)  // a short kernel: fetch all arguments in one go rather than each before its first use
     asm volatile("" ::"s"(row_width), "s"(table_width), "s"(heads), "s"(kv_heads), "s"(page_size), "s"(page_shift),
                  "s"(scale), "s"(window), "s"(splits), "s"(fused.pairing));
@@ -520,7 +520,9 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
 
   // merge the waves, one column tile at a time: each wave leaves, per column, D sums, its
   // maximum and its sum of weights
-  constexpr int STRIDE = D + 2;
+  // (a column's row is D sums, then its maximum and its sum of weights; rows 16 bytes apart in the banks, so that a
+  // lane's four sums of a tile go and come as one 16-byte piece)
+  constexpr int STRIDE = D + 4;
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
     float sum = running_sum[t];
@@ -528,13 +530,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
     sum += __shfl_xor(sum, 32, WAVE);
     float* mine = lds + ((size_t)wave * 16 + c) * STRIDE;
 #pragma unroll
-    for (int d = 0; d < D_TILES; ++d)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mine[d * 16 + 4 * q + i] = acc[t][d][i];
-    if (q == 0) {
-      mine[D] = running_max[t];
-      mine[D + 1] = sum;
-    }
+    for (int d = 0; d < D_TILES; ++d) *(f32x4*)(mine + d * 16 + 4 * q) = acc[t][d];
+    if (q == 0) *(float2*)(mine + D) = make_float2(running_max[t], sum);
     __syncthreads();
     for (int index = threadIdx.x; index < 16 * (D / 4); index += WAVES * 64) {
       const int column = index / (D / 4), d4 = (index % (D / 4)) * 4;
@@ -542,24 +539,32 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
       bool live;
       map.of(t, column, token, head_here, live);
       if (!live) continue;
-      float best = -INFINITY;
-      for (int w = 0; w < WAVES; ++w) best = fmaxf(best, lds[((size_t)w * 16 + column) * STRIDE + D]);
-      float total = 0.f;
-      f32x4 merged = {0.f, 0.f, 0.f, 0.f};
+      float2 theirs_ml[WAVES];
+      f32x4 theirs_acc[WAVES];
+#pragma unroll
       for (int w = 0; w < WAVES; ++w) {
         const float* theirs = lds + ((size_t)w * 16 + column) * STRIDE;
-        const float factor = theirs[D] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(theirs[D] - best);
-        total += theirs[D + 1] * factor;
+        theirs_ml[w] = *(const float2*)(theirs + D);
+        theirs_acc[w] = *(const f32x4*)(theirs + d4);
+      }
+      float best = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) merged[i] += theirs[d4 + i] * factor;
+      for (int w = 0; w < WAVES; ++w) best = fmaxf(best, theirs_ml[w].x);
+      float total = 0.f;
+      f32x4 merged = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        const float factor = theirs_ml[w].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(theirs_ml[w].x - best);
+        total += theirs_ml[w].y * factor;
+        merged += theirs_acc[w] * factor;
       }
       const int head = kv_head * group + head_tile * 16 + head_here;
       const size_t row = (size_t)row0 + token;
       if (splits == 1) {
-        bf16_t* dst = out + (row * heads + head) * D + d4;
         const float inverse = total > 0.f ? 1.f / total : 0.f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
+        const bf16x4 rounded = {(bf16_t)(merged[0] * inverse), (bf16_t)(merged[1] * inverse), (bf16_t)(merged[2] * inverse),
+                                (bf16_t)(merged[3] * inverse)};
+        *(bf16x4*)(out + (row * heads + head) * D + d4) = rounded;
       } else {
         const size_t kept_as = fused.by_item ? (size_t)(gridDim.x - 1 - blockIdx.x) * tokens_per_tile + token : row;
         const size_t slot = (kept_as * heads + head) * splits + blockIdx.z;
@@ -570,20 +575,13 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
           const size_t of_split = (size_t)head * splits + blockIdx.z;
           bf16_t* dst = (bf16_t*)partial_acc + ((of_split * (D / 8) + d4 / 8) * 16 + row) * 8 + d4 % 8;
           const float inverse = total > 0.f ? 1.f / total : 0.f;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)(merged[i] * inverse);
-          if (d4 == 0) {
-            partial_ml[(of_split * 16 + row) * 2] = best;
-            partial_ml[(of_split * 16 + row) * 2 + 1] = total;
-          }
+          const bf16x4 rounded = {(bf16_t)(merged[0] * inverse), (bf16_t)(merged[1] * inverse), (bf16_t)(merged[2] * inverse),
+                                  (bf16_t)(merged[3] * inverse)};
+          *(bf16x4*)dst = rounded;
+          if (d4 == 0) *(float2*)(partial_ml + (of_split * 16 + row) * 2) = make_float2(best, total);
         } else {
-          float* dst = partial_acc + slot * D + d4;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) dst[i] = merged[i];
-          if (d4 == 0) {
-            partial_ml[slot * 2] = best;
-            partial_ml[slot * 2 + 1] = total;
-          }
+          *(f32x4*)(partial_acc + slot * D + d4) = merged;
+          if (d4 == 0) *(float2*)(partial_ml + slot * 2) = make_float2(best, total);
         }
       }
     }
@@ -945,7 +943,7 @@ static int launch_tiles(const void* qkv, int row_width, void* out, float* partia
   const int group = heads / kv_heads;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
   const int head_tiles = (group + 15) / 16;
-  const size_t shared = (size_t)WAVES * 16 * (D + 2) * sizeof(float);
+  const size_t shared = (size_t)WAVES * 16 * (D + 4) * sizeof(float);
   if (shared > 64 * 1024) {  // more dynamic LDS than a kernel gets by default: ask for it once
     static bool asked = false;
     if (!asked) {
