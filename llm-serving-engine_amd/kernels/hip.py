@@ -800,10 +800,14 @@ class HipKernels:
             elif batch.max_query_length <= per_tile:  # few tiles, maybe long: split the keys
                 # a wave walks its share of the keys step after step (32 keys each), and a walk of
                 # a few steps costs less than the second kernel that merges splits: split only when
-                # a wave would walk more than 8 steps and the chip has room for more workgroups
+                # a wave would walk more than 8 steps and the chip has room for more workgroups.  Room: about
+                # 192 workgroups of eight waves in all, swept over 1 to 64 requests and 1,500 to 30,000 keys at
+                # 12 / 2 heads (us a layer, the splits this gives against the 2,048 workgroups allowed before: 64
+                # requests over 4,096 keys 40.6 / 47.4, over 2,500 27.2 / 33.4, over 1,500 18.8 / 21.8; 32 over
+                # 8,192 44.0 / 47.0; 16 over 16,384 43.9 / 48.1; up to 8 requests as before).
                 blocks = items * kv_heads * head_tiles
                 steps = -(-batch.max_context_length // 32)
-                splits = max(1, min(-(-steps // 32), max(1, 2048 // blocks), 64))
+                splits = max(1, min(-(-steps // 32), max(1, 192 // blocks), 64))
                 if unmerged:
                     # Nothing merges in a kernel of its own here, so a split costs only what its reader pays to
                     # read it (about 0.8 us a split in the product): a workgroup's eight waves get one step each.
@@ -821,6 +825,10 @@ class HipKernels:
                         splits = next(allowed for allowed in (1, 2, 3, 4, 6, 8) if allowed >= wanted)
                     else:
                         unmerged = False
+                if not unmerged and blocks <= 8 and steps >= 128:
+                    # very few requests over a long context: runs of 16 steps, two a wave (one request over 8,192
+                    # keys 12.6 -> 11.5 us a layer, four 15.1 -> 13.4)
+                    splits = max(splits, min(-(-steps // 16), 192 // blocks, 64))
                 if splits > 1:
                     held = 16 if unmerged else tokens  # the product that merges wants 16 rows side by side
                     partial_acc = self._empty((held * heads * splits * layout.head_dim,), qkv.dtype if unmerged else torch.float32)
