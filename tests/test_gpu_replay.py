@@ -353,3 +353,62 @@ def test_nine_thousand_keys_through_the_whole_engine(tmp_path_factory, dtype):
         checked += 2
     assert checked == 26 and runner.step_counts["replayed"] >= 6
     runner.close()
+
+
+def test_long_portions_at_many_heads_beside_a_decoded_token(tmp_path_factory):
+    """Portions of 2,048 tokens at 28 / 4 heads of 128 go to the attention kernel that shares K and V through LDS
+    unsplit (448 workgroups), the second one behind 2,048 cached keys and beside another request's decoded token
+    whose 2,100 keys are cut into runs in a launch of its own; then both requests decode.  Against the plain
+    forward of a narrow model."""
+    from llmserve_amd import CacheConfig, ModelRunner, StepEntry
+    from llmserve_amd.kernels import HipKernels
+    from llmserve_amd.weights import load_model_folder, write_model_folder
+    from tests.tiny import LOUD, MANY_HEADS
+
+    folder = write_model_folder(tmp_path_factory.mktemp("heads") / "heads", MANY_HEADS, seed=78, norm_std=0.1, **LOUD)
+    plain_config, weights = plain.PlainConfig.from_folder(folder), plain.read_weights(folder)
+    sequences = [random_tokens(4206, MANY_HEADS.vocab_size, seed=823), random_tokens(2106, MANY_HEADS.vocab_size, seed=824)]
+    expected = [plain.forward(weights, plain_config, tokens) for tokens in sequences]
+    spread = float(expected[0].std())
+    bound = dict(atol=BF16_LARGEST * spread, rtol=3e-2)
+    loaded = load_model_folder(folder, "bfloat16")
+    kernels = HipKernels(loaded.dtype)
+    library = kernels._attention_library(MANY_HEADS.head_dim)  # count which launches the steps below make
+    calls = {"shared": 0, "by item": 0}
+    shared_entry, tiles_entry = library.llmserve_attention_portions, library.llmserve_attention_tiles
+
+    def counted_shared(*arguments):
+        calls["shared"] += 1
+        return shared_entry(*arguments)
+
+    def counted_tiles(*arguments):
+        calls["by item"] += 1 if arguments[20] & 4 and arguments[19] > 1 else 0  # (fuse, splits)
+        return tiles_entry(*arguments)
+
+    library.llmserve_attention_portions, library.llmserve_attention_tiles = counted_shared, counted_tiles
+    runner = ModelRunner(loaded, kernels, CacheConfig(PAGE_WIDE, 420, 4))
+
+    def check(logits, row, sequence, position):
+        torch.testing.assert_close(logits[row].cpu().double(), expected[sequence][position], **bound,
+                                   msg=lambda m: f"sequence {sequence} position {position}: {m}")
+
+    logits = runner.step([StepEntry("other", sequences[1][:2100], [2099])], create_missing=True)
+    check(logits, 0, 1, 2099)
+    logits = runner.step([StepEntry("long", sequences[0][:2048], [0, 1000, 2047])], create_missing=True)
+    for row, position in enumerate((0, 1000, 2047)):
+        check(logits, row, 0, position)
+    logits = runner.step([StepEntry("long", sequences[0][2048:4096], [0, 700, 2047]), StepEntry("other", [sequences[1][2100]], [0])])
+    for row, position in enumerate((2048, 2748, 4095)):
+        check(logits, row, 0, position)
+    check(logits, 3, 1, 2100)
+    logits = runner.step([StepEntry("long", sequences[0][4096:4200], [103]), StepEntry("other", [sequences[1][2101]], [0])])
+    check(logits, 0, 0, 4199)
+    check(logits, 1, 1, 2101)
+    for step in range(4):
+        entries = [StepEntry("long", [sequences[0][4200 + step]], [0]), StepEntry("other", [sequences[1][2102 + step]], [0])]
+        logits = runner.step(entries)
+        check(logits, 0, 0, 4200 + step)
+        check(logits, 1, 1, 2102 + step)
+    library.llmserve_attention_portions, library.llmserve_attention_tiles = shared_entry, tiles_entry
+    assert calls == {"shared": 3, "by item": 1}, calls  # the prompts' three long portions; the token beside the second
+    runner.close()

@@ -147,6 +147,22 @@ LONG = Qwen2Config(
     rope_pairing="half",
 )
 
+MANY_HEADS = Qwen2Config(  # narrow, with the 7B sizes' heads: a 2,048-token portion is 448 workgroups of 128 columns
+    vocab_size=517,
+    hidden_size=256,
+    intermediate_size=384,
+    num_layers=1,
+    num_attention_heads=28,
+    num_key_value_heads=4,
+    head_dim=128,
+    max_position_embeddings=8192,
+    rope_theta=1e6,
+    rms_norm_eps=1e-6,
+    attention_bias=True,
+    tie_word_embeddings=True,
+    rope_pairing="half",
+)
+
 WIDE_CONFIGS = {"1.5B": (WIDE, 31), "7B": (WIDE_7B, 37), "32B": (WIDE_32B, 41)}
 
 
