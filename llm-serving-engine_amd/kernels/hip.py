@@ -594,6 +594,11 @@ class HipKernels:
         work = np.stack([request, starts[request] + first // per_token, first % per_token, columns], axis=1).astype(np.int32)
         begins = np.array([chunk.start for chunk in chunks], dtype=np.int64)[which]
         steps = int((items * ((begins + counts[which] / 2) / 32 + 1)).sum())
+        # The kernels start the list's last item first, and an item walks the keys up to its last token: in the
+        # order of those positions the longest walks start first, whichever request they belong to (portions of
+        # several requests at different depths of their prompts).
+        last_position = np.repeat(begins, items) + (first + columns - 1) // per_token
+        work = work[np.argsort(last_position, kind="stable")]
         return work, steps
 
     @staticmethod
@@ -755,6 +760,12 @@ class HipKernels:
             splits = 1
             if groups >= 400 or (groups >= 192 and longest <= 32):
                 shared = True
+                # Enough workgroups, but one request's portion may lie far deeper in its prompt than the others':
+                # where the longest walk is well beyond a slot's share of all walks the kernel would wait for those
+                # few workgroups, and all walks are cut (the short ones into runs of a few steps).
+                share = max(1, steps * kv_heads * head_tiles // 512)
+                if longest >= 256 and 2 * longest > 3 * share:
+                    splits = max(1, min(8, longest // 64, -(-longest // share)))
             elif longest >= 256:
                 splits = max(1, min(8, longest // 64, -(-768 // groups)))
                 shared = groups * splits >= 384
