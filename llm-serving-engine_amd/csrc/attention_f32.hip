@@ -50,7 +50,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
   __shared__ float wave_max[WAVES][COLUMN_TILES][16];
   __shared__ float wave_sum[WAVES][COLUMN_TILES][16];
   __shared__ __attribute__((aligned(16))) float merged[COLUMN_TILES][D_STEPS][64][4];
-  const int* item = work + 4 * blockIdx.x;
+  const int* item = work + 4 * (gridDim.x - 1 - blockIdx.x);  // the list's last items walk the most keys: they start first
   const int request = item[0], first_row = item[1], first_head = item[2], columns = item[3];
   if (columns <= 0) return;  // an item that only pads a captured step's list
   const int kv_head = blockIdx.y, split = blockIdx.z;
