@@ -845,10 +845,10 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   // LDS is used once more below: nothing may still be on its way into it
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 
-  // each wave's columns leave through 8 KB of LDS of its own (16 columns x 128 floats) as whole rows: of `out`,
+  // each wave's columns leave through LDS of its own (16 columns x 128 floats) as whole rows: of `out`,
   // divided by the sum of weights, or (splits > 1) of the split's partial sums as they are, with the column's
   // reference maximum and sum of weights beside them, for the kernel that merges
-  constexpr int STRIDE = D;
+  constexpr int STRIDE = D + 4;  // (a row of 128 floats would put all sixteen columns into the same banks)
   float* mine = (float*)stages + (size_t)wave * 16 * STRIDE;
   float2* mine_ml = (float2*)((float*)stages + 4 * 16 * STRIDE) + wave * 16;
 #pragma unroll
