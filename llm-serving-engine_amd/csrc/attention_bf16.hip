@@ -106,10 +106,14 @@ struct StepLoads {
 struct ColumnMap {
   int heads_here, first_head, columns;
   bool packed;
+  // (a column's number is below 256 and there are at most 16 heads here: the quotient by a multiplication, exact for
+  // numbers below 65,536 / heads_here; a division proper costs forty instructions, several times a workgroup)
+  unsigned reciprocal = 65536u / (unsigned)heads_here + 1u;
+  __device__ __forceinline__ int over_heads(int flat) const { return (int)(((unsigned)flat * reciprocal) >> 16); }
   __device__ __forceinline__ void of(int tile, int c, int& token, int& head, bool& live) const {
     if (packed) {
       const int flat = first_head + tile * 16 + c;
-      token = flat / heads_here;
+      token = over_heads(flat);
       head = flat - token * heads_here;
       live = tile * 16 + c < columns;
     } else {
@@ -118,7 +122,7 @@ struct ColumnMap {
       live = tile < columns && c < heads_here;
     }
   }
-  __device__ __forceinline__ int tokens() const { return packed ? (first_head + columns - 1) / heads_here + 1 : columns; }
+  __device__ __forceinline__ int tokens() const { return packed ? over_heads(first_head + columns - 1) + 1 : columns; }
 };
 
 // What a lane keeps for its column in each of its column tiles.
@@ -715,8 +719,8 @@ __global__ __launch_bounds__(256, 2) void attention_portions_kernel(
   const int last_key_all = position_first + tokens_all - 1;
   const int first_key_all = window > 0 ? max(0, position_first - window + 1) : 0;
   const int skipped = wave * COLUMN_TILES * (all.packed ? 16 : 1);  // columns (packed) or tokens before this wave's
-  const int mine_first = all.packed ? (all.first_head + skipped) / heads_here : skipped;  // its first token, within the item
-  const ColumnMap map = {heads_here, all.packed ? (all.first_head + skipped) % heads_here : 0,
+  const int mine_first = all.packed ? all.over_heads(all.first_head + skipped) : skipped;  // its first token, within the item
+  const ColumnMap map = {heads_here, all.packed ? all.first_head + skipped - mine_first * heads_here : 0,
                          max(0, min(all.columns - skipped, COLUMN_TILES * (all.packed ? 16 : 1))), all.packed};
   const int tokens = map.columns > 0 ? map.tokens() : 0;  // 0: nothing of its own
   const int row0 = row_first + mine_first, position0 = position_first + mine_first;
