@@ -803,7 +803,9 @@ class HipKernels:
                 # portions'.
                 longest_few = max((chunk.start + chunk.count for chunk in batch.chunks if chunk.count <= per_tile), default=0)
                 steps = -(-longest_few // 32)
-                splits = max(1, min(-(-steps // 32), max(1, 2048 // (items * kv_heads * head_tiles)), 64))
+                # (about 384 workgroups of four waves in all, as many waves as the 192 of a step of single tokens:
+                # 63 decoded tokens over 2,048 keys beside a 2,048-token portion at 40 / 8 heads 510 -> 478 us)
+                splits = max(1, min(-(-steps // 32), max(1, 384 // (items * kv_heads * head_tiles)), 64))
                 if splits > 1:
                     by_item = True
                     partial_acc = self._empty((items * per_tile * heads * splits * layout.head_dim,), torch.float32)
