@@ -24,6 +24,9 @@
 // When every request of the step brings one token (FUSED), the kernel also does what comes
 // before and after it in a decode step: it rotates the queries in registers, the workgroup
 // that owns the newest key rotates that key and stores key and value in their page first.
+// CHANGED: a score is changed before the softmax, for encodings and models that want it (the
+// reference has neither): `soft_cap` > 0 squashes it to cap * tanh(score / cap), and `slopes` (one
+// per query head) then takes slope * (query position - key position) off it.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -92,6 +95,11 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
                               // instead of by the step's row: for the few short requests of a step of long portions
 };
 
+struct ScoreChange {          // unused unless CHANGED
+  const float* slopes;        // [heads], or null
+  float soft_cap;             // 0: none
+};
+
 // One step's operands as a lane holds them: its slices of the K rows of the two 16-row tiles and,
 // for every 16-row tile of V^T, eight consecutive keys of its row.
 struct StepLoads {
@@ -130,6 +138,7 @@ template <int COLUMN_TILES>
 struct Columns {
   int position[COLUMN_TILES], first[COLUMN_TILES];  // the keys the column sees: [first, position]
   QkOperand query[COLUMN_TILES][QK_STEPS];
+  float slope[COLUMN_TILES];  // of the column's head, in units of log2 a key; set and read only where scores are changed
   float running_max[COLUMN_TILES], running_sum[COLUMN_TILES];
   f32x4 acc[COLUMN_TILES][D_TILES];
 };
@@ -158,10 +167,12 @@ __device__ __forceinline__ void scores_of(const Columns<COLUMN_TILES>& columns, 
 // own eight scores.  `interior`: every column of the wave sees all 32 keys of the step (no masks).
 // `v_start`: the first of the eight keys this lane's V values were really read from; values of keys
 // after `last_key` (slots never written) are kept out of 0 * x.
-template <int COLUMN_TILES>
+// CHANGED: `soft_cap` > 0 squashes a score to cap * tanh(score * scale / cap), as 1 - 2 / (1 + e^(2 score * scale / cap))
+// (right at both ends: e^x = inf gives 1, 0 gives -1), and the column's slope times the key's distance comes off it.
+template <int COLUMN_TILES, bool CHANGED = false>
 __device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, StepLoads& L, const f32x4* s_lo,
                                               const f32x4* s_hi, int key0, int q, bool interior, int last_key,
-                                              int v_start, float scale_log2) {
+                                              int v_start, float scale_log2, float soft_cap = 0.f) {
   bf16x8 weights[COLUMN_TILES];
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
@@ -171,6 +182,19 @@ __device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, St
     float x[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[i] = fmaf(i < 4 ? s_lo[t][i] : s_hi[t][i - 4], scale_log2, -reference);
+    if constexpr (CHANGED) {
+      if (soft_cap > 0.f) {
+        const float cap_log2 = soft_cap * 1.44269504088896f, doubled = 2.f * scale_log2 / soft_cap;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float e = __builtin_amdgcn_exp2f((i < 4 ? s_lo[t][i] : s_hi[t][i - 4]) * doubled);
+          x[i] = fmaf(cap_log2, 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e), -reference);
+        }
+      }
+      const float distance = (float)(columns.position[t] - (key0 + 8 * q));  // of the lane's first key
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] -= columns.slope[t] * (distance - (float)i);
+    }
     if (!interior) {
       // key0 + 8q + i outside [first, position], counted from the lane's first key (nothing to add per key)
       const int last_seen = columns.position[t] - (key0 + 8 * q), first_seen = columns.first[t] - (key0 + 8 * q);
@@ -222,13 +246,14 @@ __device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, St
       columns.acc[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(L.v[d], weights[t], columns.acc[t][d], 0, 0, 0);
 }
 
-template <int COLUMN_TILES, bool FUSED, int WAVES>
+template <int COLUMN_TILES, bool FUSED, int WAVES, bool CHANGED = false>
 __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || WAVES > 4) ? 1 : 2) void attention_tiles_kernel(
     const bf16_t* __restrict__ qkv, int row_width, bf16_t* __restrict__ out, float* __restrict__ partial_acc,
     float* __restrict__ partial_ml, bf16_t* __restrict__ keys,
     bf16_t* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ positions, const int* __restrict__ work, int heads, int kv_heads, int tokens_per_tile,
-    int page_size, int page_shift, float scale, int window, int splits, FusedDecode fused) {
+    int page_size, int page_shift, float scale, int window, int splits, FusedDecode fused, ScoreChange change) {
+  static_assert(!(FUSED && CHANGED), "the fused decode form takes plain scores only");
   extern __shared__ float lds[];  // [WAVES][16 columns][D + 4]
   if (FUSED)  // a short kernel: fetch all arguments in one go rather than each before its first use
     asm volatile("" ::"s"(row_width), "s"(table_width), "s"(heads), "s"(kv_heads), "s"(page_size), "s"(page_shift),
@@ -314,6 +339,7 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
     const int head = kv_head * group + head_tile * 16 + head_here;
     column_position[t] = column_live[t] ? position0 + safe : -1;
     column_first[t] = window > 0 ? column_position[t] - window + 1 : 0;
+    if constexpr (CHANGED) columns.slope[t] = change.slopes ? change.slopes[head] * 1.44269504088896f : 0.f;
     const bf16_t* q_row = qkv + (size_t)(row0 + safe) * row_width + (size_t)head * D;
 #pragma unroll
     for (int s = 0; s < QK_STEPS; ++s) query[t][s] = load_qk(q_row, KEY_PIECE, s, q);  // a query's row is in one piece
@@ -514,8 +540,8 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
       if (more) fetch_keys(step + WAVES, pages, loads);
       const int key0 = step * KEYS;
       const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
-      weigh_and_add(columns, loads, s_lo, s_hi, key0, q, interior, last_key,
-                    min(max(key0 + 8 * q, low_limit), high_limit), scale_log2);
+      weigh_and_add<COLUMN_TILES, CHANGED>(columns, loads, s_lo, s_hi, key0, q, interior, last_key,
+                                           min(max(key0 + 8 * q, low_limit), high_limit), scale_log2, change.soft_cap);
       if (more) fetch_values(step + WAVES, pages, loads);
       if (step + 2 * WAVES < step_end) pages = pages_of(step + 2 * WAVES);
     }
@@ -938,12 +964,12 @@ extern "C" int llmserve_attention_portions(const void*, int, void*, float*, floa
 #ifndef FUSED_WAVES
 #define FUSED_WAVES (HEAD_DIM > 128 ? 4 : 8)
 #endif
-template <int COLUMN_TILES, bool FUSED, int WAVES>
+template <int COLUMN_TILES, bool FUSED, int WAVES, bool CHANGED = false>
 static int launch_tiles(const void* qkv, int row_width, void* out, float* partial_acc, float* partial_ml,
                         void* keys, void* values, const int* block_tables, int table_width,
                         const int* positions, const int* work, int tiles, int heads, int kv_heads,
                         int tokens_per_tile, int page_size, float scale, int window, int splits, FusedDecode fused,
-                        hipStream_t stream) {
+                        hipStream_t stream, ScoreChange change = {nullptr, 0.f}) {
   const int group = heads / kv_heads;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
   const int head_tiles = (group + 15) / 16;
@@ -951,16 +977,16 @@ static int launch_tiles(const void* qkv, int row_width, void* out, float* partia
   if (shared > 64 * 1024) {  // more dynamic LDS than a kernel gets by default: ask for it once
     static bool asked = false;
     if (!asked) {
-      if (hipFuncSetAttribute((const void*)attention_tiles_kernel<COLUMN_TILES, FUSED, WAVES>,
+      if (hipFuncSetAttribute((const void*)attention_tiles_kernel<COLUMN_TILES, FUSED, WAVES, CHANGED>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shared) != hipSuccess)
         return ERR_BAD_ARGUMENT;
       asked = true;
     }
   }
-  hipLaunchKernelGGL((attention_tiles_kernel<COLUMN_TILES, FUSED, WAVES>), dim3(tiles, kv_heads * head_tiles, splits),
+  hipLaunchKernelGGL((attention_tiles_kernel<COLUMN_TILES, FUSED, WAVES, CHANGED>), dim3(tiles, kv_heads * head_tiles, splits),
                      dim3(WAVES * 64), shared, stream, (const bf16_t*)qkv, row_width, (bf16_t*)out, partial_acc,
                      partial_ml, (bf16_t*)keys, (bf16_t*)values, block_tables, table_width, positions, work,
-                     heads, kv_heads, tokens_per_tile, page_size, page_shift, scale, window, splits, fused);
+                     heads, kv_heads, tokens_per_tile, page_size, page_shift, scale, window, splits, fused, change);
   return LAUNCH_STATUS();
 }
 
@@ -989,14 +1015,19 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // partial_acc is then bfloat16 [heads][splits][D / 8][16 rows][8], each split's result divided by its own sum of
 // weights, and partial_ml [heads][splits][16 rows][2] holds each split's maximum (in units of log2) and sum of
 // weights.
+// `slopes` (float32 [heads], or null) and `soft_cap` (0 for none) change the scores before the softmax (see the head of
+// this file); not together with `fuse` & 1.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
                                         float* partial_ml, void* keys, void* values,
                                         const int* block_tables, int table_width, const int* positions,
                                         const int* work, int tiles, int column_tiles, int rows, int heads,
                                         int kv_heads, int page_size, float scale, int window, int splits, int fuse,
-                                        const float* table, int pairing, const int* slots,
-                                        hipStream_t stream) {
+                                        const float* table, int pairing, const int* slots, const float* slopes,
+                                        float soft_cap, hipStream_t stream) {
   if (tiles <= 0) return 0;
+  const bool changed = slopes != nullptr || soft_cap > 0.f;
+  if (soft_cap < 0.f || (changed && (fuse & 1))) return ERR_BAD_ARGUMENT;
+  const ScoreChange change = {slopes, soft_cap};
   if (heads % kv_heads || page_size % 8 || splits < 1 || splits > MERGE_SPLITS_MAX || (splits > 1 && (!partial_acc || !partial_ml)))
     return ERR_BAD_ARGUMENT;
   if ((long)kv_heads * page_size * D >= (1L << 31)) return ERR_BAD_ARGUMENT;  // a page's elements are counted in 32 bits
@@ -1015,6 +1046,14 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
     status = launch_tiles<1, true, FUSED_WAVES>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
                                         table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile,
                                         page_size, scale, window, splits, fused, stream);
+  } else if (changed && column_tiles == 1) {
+    status = launch_tiles<1, false, 4, true>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
+                                          table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile,
+                                          page_size, scale, window, splits, fused, stream, change);
+  } else if (changed && column_tiles == 2) {
+    status = launch_tiles<2, false, 4, true>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
+                                          table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile,
+                                          page_size, scale, window, splits, fused, stream, change);
   } else if (column_tiles == 1) {
     status = launch_tiles<1, false, 4>(qkv, row_width, out, partial_acc, partial_ml, keys, values, block_tables,
                                     table_width, positions, work, tiles, heads, kv_heads, tokens_per_tile, page_size,

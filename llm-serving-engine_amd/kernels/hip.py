@@ -64,7 +64,7 @@ _SIGNATURES = {
     "llmserve_gemm_wide": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifipfp",
     "llmserve_attention_f32": "pippppppippiiiiiifiipfp",
-    "llmserve_attention_tiles": "pippppppippiiiiiifiiipipp",
+    "llmserve_attention_tiles": "pippppppippiiiiiifiiipippfp",
     "llmserve_attention_portions": "pippppppippiiiiiifiip",
     "llmserve_attention_can_fuse": "i",
     "llmserve_argmax": "ppppiip",
@@ -658,8 +658,8 @@ class HipKernels:
         score_slopes: torch.Tensor | None = None, soft_cap: float | None = None,
     ) -> torch.Tensor:
         """`score_slopes` (float32 [heads]) and `soft_cap` change the scores before the softmax: cap * tanh(score /
-        cap), then minus slope * distance.  The float32 kernels take them; in bfloat16 the matrix-core kernels
-        are passed by when either is given, for the generic kernel."""
+        cap), then minus slope * distance.  The matrix-core kernels of both precisions take them (in bfloat16
+        not the forms that fuse the rotation or share keys through LDS)."""
         tokens = qkv.shape[0]
         group = batch.groups[cell.group]
         if cell.keys.dtype != qkv.dtype:
@@ -671,14 +671,15 @@ class HipKernels:
         out = self._empty((tokens, layout.num_heads * layout.head_dim), qkv.dtype)
         dim = layout.head_dim
         plain_scores = score_slopes is None and soft_cap is None
-        if plain_scores and qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
-            self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0))
+        if qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
+            changed = None if plain_scores else (score_slopes, float(soft_cap or 0.0))
+            self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), changed=changed)
             return out
         if qkv.dtype == torch.float32 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
             self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0), score_slopes, soft_cap)
             return out
         if qkv.dtype == torch.bfloat16:
-            why = "its scores carry a bias or a soft cap" if not plain_scores else f"head size {dim} and pages of {group.page_size}"
+            why = f"head size {dim} and pages of {group.page_size}"
             self._tell_once(f"generic attention: {why}", f"bfloat16 attention runs on the generic kernel, not on the matrix cores: {why}")
         status = self._attention_generic.llmserve_attention_generic(
             _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
@@ -721,14 +722,18 @@ class HipKernels:
         )
         _check(status, "paged_attention")
 
-    def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None, unmerged=False):
+    def _attention_tiles(self, qkv, out, layout, batch, cell, group, scale: float, window: int, fuse=None, unmerged=False, changed=None):
         """The MFMA kernel: requests that bring a few tokens (decoding) one column tile per
         wave, split over the keys when there are few of them; longer portions two tiles
         per wave.  `fuse` = (rotary table, pairing) lets a step of single tokens rotate and
         store inside the same kernel.  With `unmerged` (a step of single tokens whose reader merges
         key splits itself) the keys are split more finely and the splits are returned as they are
         (their results in bfloat16, laid out for `gemm_merged`; their maxima and sums in float32; how
-        many), instead of `out`."""
+        many), instead of `out`.  `changed` = (slopes or None, soft cap or 0.0): scores changed before the softmax,
+        which neither `fuse` nor the kernel that shares keys through LDS takes."""
+        if changed is not None and fuse is not None:
+            raise KernelError("paged_attention: the fused decode form takes plain scores only")
+        slopes, soft_cap = changed if changed is not None else (None, 0.0)
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
         per_tile = max(1, 16 // (heads // kv_heads))
@@ -739,7 +744,7 @@ class HipKernels:
         shared = False
         padded = getattr(batch, "padded_to", None) is not None  # a captured step: the same launches whatever it holds
         whole_pages = group.page_size >= 16 and group.page_size & (group.page_size - 1) == 0  # (what that kernel takes)
-        if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and self.shared_portions != "never" and not padded and whole_pages:
+        if batch.max_query_length > per_tile and layout.head_dim == 128 and fuse is None and changed is None and self.shared_portions != "never" and not padded and whole_pages:
             # Prompt portions at this head size may go to the kernel whose waves share each step's K and V
             # through LDS (a quarter of the cache traffic; what bounds the kernel above over long walks is the
             # path from the caches into the registers).  Its workgroups take 128 columns and walk all their keys,
@@ -851,7 +856,7 @@ class HipKernels:
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
                 _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
                 group.page_size, scale, window, splits, (1 if fuse is not None else 0) + (2 if unmerged else 0) + (4 if by_item else 0),
-                _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), self._stream,
+                _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), _pointer(slopes), soft_cap, self._stream,
             )
             _check(status, "paged_attention")
             if unmerged and splits > 1:

@@ -894,7 +894,8 @@ def test_gated_products_with_every_gate_activation(kernels, dtype, activation, r
 @pytest.mark.parametrize("heads,kv_heads,dim,page,cap", [(6, 2, 32, 8, 1.5), (4, 1, 128, 16, None), (5, 5, 48, 4, 0.7)])
 def test_paged_attention_with_a_distance_bias_and_a_soft_cap(kernels, dtype, heads, kv_heads, dim, page, cap):
     """Scores squashed to cap * tanh(score / cap), then lowered by slope[head] * distance: portions beside decoded
-    tokens, in float32 on the matrix-core kernel and in bfloat16 on the generic one, against the formula."""
+    tokens, on the matrix-core kernels of both precisions (pages of 4 in bfloat16: the generic one), against the
+    formula."""
     lengths, counts = [45, 17, 70], [20, 1, 70]
     batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, page, dtype, shuffle_seed=heads)
     qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
@@ -913,4 +914,30 @@ def test_paged_attention_with_a_distance_bias_and_a_soft_cap(kernels, dtype, hea
         scores = (scores - slopes.double().view(-1, 1, 1) * distance).masked_fill(distance < 0, float("-inf"))
         full = torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), v)
         expected.append(full[-count:].flatten(1))
+    torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("lengths,counts,window", [([2100, 700, 5], [1, 1, 1], None), ([300, 2100, 900], [300, 64, 1], 512)])
+@pytest.mark.parametrize("heads,kv_heads,dim,cap", [(12, 2, 128, 4.0), (7, 7, 64, None)])
+def test_changed_scores_over_long_contexts(kernels, dtype, lengths, counts, window, heads, kv_heads, dim, cap):
+    """The same change of the scores where the keys are split over workgroups and merged (single tokens over long
+    contexts), in long portions, and under a window; slopes small enough that far keys still count, one head's zero."""
+    batch, cell, per_request, layout = paged_case(lengths, counts, heads, kv_heads, dim, 16, dtype, shuffle_seed=3)
+    qkv = on_gpu(step_rows(per_request, counts, heads, kv_heads, dim), dtype)
+    slopes = torch.tensor([0.0 if head == 1 else 0.004 * (1 + head % 3) for head in range(heads)], dtype=torch.float32)
+    scale = 1.0 / math.sqrt(dim)
+    out = kernels[dtype].paged_attention(qkv, layout, batch, cell, scale, window, score_slopes=on_gpu(slopes), soft_cap=cap).cpu().double()
+    expected = []
+    for (q, k, v), count in zip(per_request, counts):
+        q, k, v = rounded(q, dtype)[-count:], rounded(k, dtype), rounded(v, dtype)
+        length = k.shape[0]
+        k, v = k.repeat_interleave(heads // kv_heads, dim=1), v.repeat_interleave(heads // kv_heads, dim=1)
+        scores = torch.einsum("ihd,jhd->hij", q, k) * scale
+        if cap:
+            scores = cap * torch.tanh(scores / cap)
+        distance = (torch.arange(length - count, length).unsqueeze(1) - torch.arange(length).unsqueeze(0)).double()
+        unseen = (distance < 0) | (distance >= window if window else torch.zeros_like(distance, dtype=torch.bool))
+        scores = (scores - slopes.double().view(-1, 1, 1) * distance).masked_fill(unseen, float("-inf"))
+        expected.append(torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), v).flatten(1))
     torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
