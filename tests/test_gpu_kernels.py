@@ -4,6 +4,7 @@ in steps of 16, odd numbers of heads and groups, pages of several sizes, shuffle
 
 from __future__ import annotations
 
+import contextlib
 import math
 import types
 
@@ -941,3 +942,162 @@ def test_changed_scores_over_long_contexts(kernels, dtype, lengths, counts, wind
         scores = (scores - slopes.double().view(-1, 1, 1) * distance).masked_fill(unseen, float("-inf"))
         expected.append(torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), v).flatten(1))
     torch.testing.assert_close(out, torch.cat(expected), **TOLERANCE[dtype])
+
+
+def device_paged_case(requests, heads, kv_heads, dim, page, dtype, seed):
+    """As `paged_case`, made on the device without a loop over positions, for contexts of thousands of keys:
+    `requests` = [(cached tokens, of which this step's)].  Returns the batch, the cell (NaN in every slot that no
+    token owns) and per request its step's queries and all its keys and values, as the kernel sees them."""
+    from llmserve_amd.cache import CacheCell
+    from llmserve_amd.engine.batch import GroupBatch, SequenceChunk, StepBatch
+    from llmserve_amd.parts import HeadLayout, PagedKeyValue
+
+    generator = torch.Generator(device="cuda").manual_seed(seed)
+    blocks = [math.ceil(length / page) for length, _ in requests]
+    pages = sum(blocks) + 3
+    order = torch.randperm(pages, generator=torch.Generator().manual_seed(seed)).cuda()
+    width = max(blocks)
+    tables = torch.full((len(requests), width), -1, dtype=torch.int32, device="cuda")
+    keys = torch.full((pages, kv_heads, page, dim), float("nan"), dtype=dtype, device="cuda")
+    values = torch.full((pages, kv_heads, dim, page), float("nan"), dtype=dtype, device="cuda")
+    per_request, rows, slot_mapping, positions, token_sequence, chunks, taken = [], [], [], [], [], [], 0
+    for index, (length, count) in enumerate(requests):
+        mine = order[taken : taken + blocks[index]]
+        taken += blocks[index]
+        tables[index, : blocks[index]] = mine.int()
+        q = torch.randn(count, heads, dim, generator=generator, device="cuda").to(dtype)
+        k = torch.randn(length, kv_heads, dim, generator=generator, device="cuda").to(dtype)
+        v = torch.randn(length, kv_heads, dim, generator=generator, device="cuda").to(dtype)
+        where = torch.arange(length, device="cuda")
+        keys[mine[where // page], :, where % page] = k
+        values[mine[where // page], :, :, where % page] = v
+        per_request.append((q, k, v))
+        rows.append(torch.cat([q.flatten(1), k[-count:].flatten(1), v[-count:].flatten(1)], dim=1))
+        mine_cpu = mine.cpu().tolist()
+        for position in range(length - count, length):
+            slot_mapping.append(mine_cpu[position // page] * page + position % page)
+            positions.append(position)
+            token_sequence.append(index)
+        chunks.append(SequenceChunk(f"r{index}", index, length - count, count))
+    counts = [count for _, count in requests]
+    starts = [0]
+    for count in counts:
+        starts.append(starts[-1] + count)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+    batch = StepBatch(
+        num_tokens=sum(counts), chunks=chunks, token_ids=ints([0] * sum(counts)), positions=ints(positions),
+        token_sequence=ints(token_sequence), query_start=ints(starts), context_lengths=ints([length for length, _ in requests]),
+        state_slots=ints(list(range(len(requests)))), groups=[GroupBatch(page, tables, ints(slot_mapping), width)],
+        logit_rows=ints([]), num_logit_rows=0, max_query_length=max(counts), max_context_length=max(length for length, _ in requests),
+    )
+    cell = CacheCell(PagedKeyValue(kv_heads, dim), True, 0, key_pieces(keys), value_pieces(values))
+    return batch, cell, per_request, torch.cat(rows), HeadLayout(heads, kv_heads, dim)
+
+
+def device_attention(q, k, v, scale, window):
+    """softmax(q k^T * scale) v of a request's last rows over all its keys, causal (and windowed), float32 on the
+    device with torch's own operations, one kv head at a time."""
+    count, heads, dim = q.shape
+    length, kv_heads = k.shape[0], k.shape[1]
+    group = heads // kv_heads
+    position = torch.arange(length - count, length, device=q.device).view(1, -1, 1)
+    key = torch.arange(length, device=q.device).view(1, 1, -1)
+    unseen = key > position
+    if window:
+        unseen = unseen | (key <= position - window)
+    out = torch.empty(count, heads, dim, dtype=torch.float32, device=q.device)
+    for kv_head in range(kv_heads):
+        mine = q[:, kv_head * group : (kv_head + 1) * group].float()
+        scores = torch.einsum("igd,jd->gij", mine, k[:, kv_head].float()) * scale
+        weights = torch.softmax(scores.masked_fill(unseen, float("-inf")), dim=-1)
+        out[:, kv_head * group : (kv_head + 1) * group] = torch.einsum("gij,jd->igd", weights, v[:, kv_head].float())
+    return out.flatten(1)
+
+
+@pytest.mark.parametrize("dtype,draws", [(torch.bfloat16, 100), (torch.float32, 30)])
+def test_attention_at_random_step_shapes(dtype, draws):
+    """What a step holds decides which attention kernel it goes to and how its keys are cut (the kernel that shares
+    keys through LDS whole or in runs, the tiles kernel with one or two column tiles, key splits merged by row or
+    by work item): steps drawn at random around those rules (long portions far into their prompts, few or many
+    decoded tokens over short and long contexts, several head counts and pages, windows), each against torch's own
+    operations, and the bfloat16 draws together must have taken every way; the float32 kernel under the same draws."""
+    import random
+
+    from llmserve_amd.kernels import HipKernels
+
+    kernels = HipKernels(dtype)
+    library = kernels._attention_library(128)
+    ways = {"shared whole": 0, "shared in runs": 0, "tiles": 0, "tiles split": 0, "by item": 0}
+    shared_entry, tiles_entry = library.llmserve_attention_portions, library.llmserve_attention_tiles
+
+    def counted_shared(*arguments):
+        ways["shared in runs" if arguments[18] > 1 else "shared whole"] += 1  # (splits)
+        return shared_entry(*arguments)
+
+    def counted_tiles(*arguments):
+        splits, fuse = arguments[19], arguments[20]
+        ways["by item" if fuse & 4 and splits > 1 else "tiles split" if splits > 1 else "tiles"] += 1
+        return tiles_entry(*arguments)
+
+    library.llmserve_attention_portions, library.llmserve_attention_tiles = counted_shared, counted_tiles
+    try:
+        for seed in range(draws):
+            draw = random.Random(seed)
+            heads, kv_heads = draw.choice([(12, 2), (28, 4), (40, 8), (16, 2), (64, 8), (7, 7)])
+            page = draw.choice([16, 16, 32, 8, 64])
+            window = draw.choice([None, None, 700, 4096])
+            requests = []
+            for _ in range(draw.choice([0, 1, 1, 2, 3])):
+                count = draw.choice([64, 300, 512, 1024, 2048])
+                requests.append((count + draw.choice([0, 0, 700, 3000, 9000, 17000]), count))
+            for _ in range(draw.choice([0, 1, 5, 20, 40]) if requests else draw.choice([1, 5, 20, 40])):
+                requests.append((draw.randint(1, draw.choice([300, 3000, 12000])), 1))
+            draw.shuffle(requests)
+            batch, cell, per_request, qkv, layout = device_paged_case(requests, heads, kv_heads, 128, page, dtype, seed)
+            scale = 1.0 / math.sqrt(128)
+            out = kernels.paged_attention(qkv, layout, batch, cell, scale, window).float()
+            expected = torch.cat([device_attention(q, k, v, scale, window) for q, k, v in per_request])
+            torch.testing.assert_close(out, expected, **TOLERANCE[dtype], msg=lambda m: f"seed {seed}, {heads}/{kv_heads} heads, pages of {page}, window {window}, {requests}: {m}")
+            del batch, cell, per_request, qkv, out, expected
+    finally:
+        library.llmserve_attention_portions, library.llmserve_attention_tiles = shared_entry, tiles_entry
+    assert dtype == torch.float32 or all(ways.values()), ways
+
+
+@pytest.mark.parametrize("own", [False, True])
+def test_products_at_random_shapes(own):
+    """Rows, K and N decide which product kernel runs (weight-streaming with one, two or four tiles a wave, through
+    registers or LDS, K cut into partial sums, the kernels for 17 to 64 rows, the library or the tiled kernels beyond,
+    inside and outside a step that a graph will replay): shapes drawn at random around those rules, plain, with a
+    bias, as float32 partial sums and gated, against torch's float32 product of the same rounded operands."""
+    import random
+
+    from llmserve_amd.kernels import HipKernels
+
+    dtype = torch.bfloat16
+    k = HipKernels(dtype, library_products=not own)
+    generator = torch.Generator(device="cuda").manual_seed(5)
+    for seed in range(150):
+        draw = random.Random(1000 + seed)
+        rows = draw.choice([1, 2, 3, 5, 8, 13, 16, 17, 24, 32, 33, 48, 64, 65, 130, 300])
+        inner = 32 * draw.choice([1, 3, 4, 8, 12, 16, 28, 40, 48, 64, 70, 112, 148, 160, 216, 280])
+        outer = draw.choice([16, 48, 100, 256, 272, 1000, 1536, 2048, 4099, 5120, 17920])
+        if rows > 64 and inner * outer > 1 << 24:
+            outer = 1000
+        x = torch.randn(rows, inner, generator=generator, device="cuda").to(dtype)
+        w = (torch.randn(outer, inner, generator=generator, device="cuda") / math.sqrt(inner)).to(dtype)
+        up = (torch.randn(outer, inner, generator=generator, device="cuda") / math.sqrt(inner)).to(dtype)
+        b = torch.randn(outer, generator=generator, device="cuda").to(dtype)
+        said = f"draw {seed}: {rows} rows, K {inner}, N {outer}"
+        want = x.float() @ w.float().T
+        plain_weights, biased = k.prepare_linear([w], None), k.prepare_linear([w], [b])
+        gated_weights = k.prepare_gated_linear(w, up)
+        want_gated = F.silu(want) * (x.float() @ up.float().T)
+        for replayed in (False, True):
+            with k.replay_scope() if replayed else contextlib.nullcontext():
+                torch.testing.assert_close(k.linear(x, plain_weights).float(), want, **TOLERANCE[dtype], msg=lambda m: f"{said}, plain, replay {replayed}: {m}")
+                torch.testing.assert_close(k.linear(x, biased).float(), want + b.float(), **TOLERANCE[dtype], msg=lambda m: f"{said}, bias, replay {replayed}: {m}")
+                parts = k.linear(x, plain_weights, out_dtype=torch.float32, partial=True)
+                summed = parts if parts.ndim == 2 else parts.sum(0)
+                torch.testing.assert_close(summed, want, atol=2e-4, rtol=2e-4, msg=lambda m: f"{said}, partial sums, replay {replayed}: {m}")
+                torch.testing.assert_close(k.gated_linear(x, gated_weights).float(), want_gated, **TOLERANCE[dtype], msg=lambda m: f"{said}, gated, replay {replayed}: {m}")
