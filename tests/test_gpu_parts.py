@@ -412,6 +412,25 @@ def test_everything_at_once_matches_the_plain_decoder(model_folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_random_workloads_on_the_gpu(model_folders, dtype):
+    """The whole runs drawn at random that the CPU tests put through the torch stand-in (tests/random_runs.py:
+    pool, batch, budget, portion size, policy, who gives way, greedy and sampled requests with stop tokens, late
+    arrivals), here through the kernels, captured steps and steps queued ahead: in float32 the plain decoder's
+    tokens exactly, in bfloat16 (the loud folders) tokens that its rule can give for the run's own prefix."""
+    from llmserve_amd.kernels import HipKernels
+    from tests.random_runs import run_random_workload
+
+    def make(name, blocks, batch):
+        loaded = load_model_folder(model_folders[name], dtype)
+        return ModelRunner(loaded, HipKernels(loaded.dtype), CacheConfig(CONFIGS[name][1], blocks, batch))
+
+    names = ("A", "B") if dtype == "float32" else ("A-loud", "B-loud")
+    gave_way = [run_random_workload(3000 + case, model_folders, make, names, exact=dtype == "float32") for case in range(16)]
+    torch.cuda.synchronize()
+    assert sum(1 for count in gave_way if count > 0) >= 2, gave_way
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_second_tiny_workload_as_stated(model_folders, dtype):
     """Six requests with prompts of 2, 9, 23, 40, 64 and 100 tokens, fed in portions of 16 beside the
     decoded tokens of those that are ahead, twelve tokens each at temperature 0.8 from one seed: in
