@@ -817,6 +817,208 @@ extern "C" int llmserve_gemm_medium(const void* x, const void* w, const void* bi
                       : pick_medium<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
 }
 
+// ---------------------------------------------------------------------------- 17 to 64 rows through a ring
+// gemm_ring: the product for 17 to 64 rows of x, bound by how fast the weights come from memory.  A
+// workgroup of four waves owns NT tiles of 16 weight rows over its whole K range and MT tiles of x; both
+// go through a ring of DEPTH stages of KSTEPS * 32 k in LDS that the waves share, filled straight from
+// memory (global_load_lds_dwordx4, a chunk of 16 rows x 32 k in lane order, laid out and swizzled as in
+// gemm_stream) DEPTH - 1 stages ahead of the one being multiplied: what a CU has under way is then that
+// many stages of weights whatever the compiler does with the registers, and a weight row is read from memory
+// once for all rows of x.  The waves divide a stage's chunks between them; one barrier a stage says that
+// everyone's loads have landed and that the stage before may be filled again.  Wave w multiplies the tile
+// w % MT of x with its share of the weight tiles, so no sums meet at the end.
+__device__ __forceinline__ void ring_load(const bf16_t* from, unsigned to) {
+  // (M0 names the place in LDS; it is put back, the compiler keeps other things there)
+  unsigned kept;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(kept)
+               : "s"(to), "v"(from)
+               : "memory");
+}
+
+// waits until at most `younger` stages' loads of this wave (PER_WAVE each) are under way; younger <= MOST
+template <int PER_WAVE, int MOST>
+__device__ __forceinline__ void ring_wait(int younger) {
+  if constexpr (MOST == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  } else {
+    if (younger >= MOST) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(MOST * PER_WAVE) : "memory");
+    else ring_wait<PER_WAVE, MOST - 1>(younger);
+  }
+}
+
+template <int NT, int MT, int KSTEPS, int DEPTH, typename TO, bool GATED>
+__global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                        const void* __restrict__ bias, int bias_is_float,
+                                                        TO* __restrict__ out, int M, int N, int K, int k_split) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
+  constexpr int WAYS = 4 / MT;          // groups of waves that divide the weight tiles between them
+  constexpr int MINE = NT / WAYS;       // weight tiles a wave multiplies
+  constexpr int TILES = NT + MT;        // of a stage, each KSTEPS chunks of 1 KB
+  constexpr int STAGE_BYTES = TILES * KSTEPS * STREAM_CHUNK;
+  constexpr int PER_WAVE = TILES * KSTEPS / 4;  // chunks a wave brings per stage
+  constexpr int APART = 4 / KSTEPS;             // tiles between two chunks of a wave
+  static_assert(MT == 2 || MT == 4, "two or four tiles of x");
+  static_assert(KSTEPS == 2 || KSTEPS == 4, "stages of 64 or 128 k");
+  static_assert(NT % WAYS == 0, "the waves divide the weight tiles evenly");
+  static_assert(TILES * KSTEPS % 4 == 0, "the waves divide a stage's chunks evenly");
+  static_assert((DEPTH - 2) * PER_WAVE <= 63, "the loads under way are counted in vmcnt");
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int k_first = blockIdx.y * k_split;
+  const int load_row = lane >> 2, load_piece = (lane & 3) ^ ((load_row >> 1) & 3);
+  // chunk j of this wave: k-step wave % KSTEPS of tile j * APART + wave / KSTEPS (the weight tiles, then x's)
+  const int my_step = wave % KSTEPS, my_first = wave / KSTEPS;
+  const bf16_t* src[PER_WAVE];  // this lane's piece of each, in the first stage
+#pragma unroll
+  for (int j = 0; j < PER_WAVE; ++j) {
+    const int tile = j * APART + my_first;
+    // rows of x beyond M are read as row M - 1: their columns of the result are dropped at the end
+    const bf16_t* row = tile < NT ? w + (size_t)min(((int)blockIdx.x * NT + tile) * 16 + load_row, N - 1) * K
+                                  : x + (size_t)min((tile - NT) * 16 + load_row, M - 1) * K;
+    src[j] = row + k_first + my_step * STEP + load_piece * 8;
+  }
+  const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ring;
+  const int x_tile = wave % MT, first_tile = wave / MT;
+  const unsigned read_at = base + (unsigned)(4 * r + (g ^ ((r >> 1) & 3))) * 16;
+  const unsigned read_w = read_at + (unsigned)first_tile * KSTEPS * STREAM_CHUNK;
+  const unsigned read_x = read_at + (unsigned)(NT + x_tile) * KSTEPS * STREAM_CHUNK;
+
+  // the bias of the outputs this lane will finish: all asked for at once, of either type
+  float bias_here[MINE][4];
+  bf16_t bias_short[MINE][4];
+  const bool biased = bias && blockIdx.y == 0;
+#pragma unroll
+  for (int i = 0; i < MINE; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = min(((int)blockIdx.x * NT + first_tile + WAYS * i) * 16 + g * 4 + j, N - 1);
+      bias_here[i][j] = 0.f;
+      if (biased && bias_is_float) bias_here[i][j] = ((const float*)bias)[n];
+      if (biased && !bias_is_float) bias_short[i][j] = ((const bf16_t*)bias)[n];
+    }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // so that the counts below count the ring's loads alone
+  if (biased && !bias_is_float) {
+#pragma unroll
+    for (int i = 0; i < MINE; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bias_here[i][j] = (float)bias_short[i][j];
+  }
+
+  const int stages = k_split / (KSTEPS * STEP);
+  auto request = [&](int stage) {
+    const unsigned to = base + (unsigned)(stage % DEPTH) * STAGE_BYTES + (unsigned)(my_first * KSTEPS + my_step) * STREAM_CHUNK;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j)
+      ring_load(src[j] + (size_t)stage * (KSTEPS * STEP), to + (unsigned)(j * APART * KSTEPS) * STREAM_CHUNK);
+  };
+  f32x4 acc[MINE];
+#pragma unroll
+  for (int i = 0; i < MINE; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < DEPTH - 1; ++s)
+    if (s < stages) request(s);
+  for (int stage = 0; stage < stages; ++stage) {
+    // this wave's loads of the stage have landed once only the younger stages' are under way
+    ring_wait<PER_WAVE, DEPTH - 2>(stages - 1 - stage);
+    // everyone's have, and everyone has read the stage before this one: it may be filled again
+    asm volatile("s_barrier" ::: "memory");
+    if (stage + DEPTH - 1 < stages) request(stage + DEPTH - 1);
+    const unsigned slot = (unsigned)(stage % DEPTH) * STAGE_BYTES;
+    bf16x8 from_x[KSTEPS], from_w[MINE][KSTEPS];
+    StreamReads<0, KSTEPS>::run(from_x, read_x + slot);
+#pragma unroll
+    for (int i = 0; i < MINE; ++i) StreamReads<0, KSTEPS>::run(from_w[i], read_w + slot + (unsigned)(WAYS * i * KSTEPS) * STREAM_CHUNK);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int u = 0; u < KSTEPS; ++u) asm volatile("" : "+v"(from_x[u]));  // used only after the wait
+#pragma unroll
+    for (int i = 0; i < MINE; ++i)
+#pragma unroll
+      for (int u = 0; u < KSTEPS; ++u) asm volatile("" : "+v"(from_w[i][u]));
+#pragma unroll
+    for (int u = 0; u < KSTEPS; ++u)
+#pragma unroll
+      for (int i = 0; i < MINE; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(from_w[i][u], from_x[u], acc[i], 0, 0, 0);
+  }
+
+  const int m = x_tile * 16 + r;
+  if (m >= M) return;
+#pragma unroll
+  for (int i = 0; i < MINE; ++i) {
+    const int n_first = ((int)blockIdx.x * NT + first_tile + WAYS * i) * 16 + g * 4;
+    f32x4 total = acc[i];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) total[j] += bias_here[i][j];
+    if (GATED) {
+      TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (n_first + 2 * j + 1 < N) {
+          const float gate = total[2 * j], up = total[2 * j + 1];
+          dst[j] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+        }
+      }
+    } else {
+      TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n_first + j < N) dst[j] = from_float<TO>(total[j]);
+    }
+  }
+}
+
+template <int NT, int MT, int KSTEPS, int DEPTH, typename TO, bool GATED>
+static int launch_ring(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
+                       int splits, hipStream_t stream) {
+  const size_t lds = (size_t)DEPTH * (NT + MT) * KSTEPS * STREAM_CHUNK;
+  if ((K / splits) % (KSTEPS * STEP)) return ERR_BAD_ARGUMENT;
+  if (lds > 64 * 1024) {
+    static bool asked = false;
+    if (!asked) {
+      if (hipFuncSetAttribute((const void*)gemm_ring_kernel<NT, MT, KSTEPS, DEPTH, TO, GATED>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return ERR_BAD_ARGUMENT;
+      asked = true;
+    }
+  }
+  hipLaunchKernelGGL((gemm_ring_kernel<NT, MT, KSTEPS, DEPTH, TO, GATED>), dim3((N + 16 * NT - 1) / (16 * NT), splits),
+                     dim3(256), lds, stream, (const bf16_t*)x, (const bf16_t*)w, bias, bias_is_float, (TO*)out, M, N, K,
+                     K / splits);
+  return LAUNCH_STATUS();
+}
+
+// nt tiles of 16 weight rows a workgroup, stages of 128 k, four stages
+template <typename TO, bool GATED>
+static int pick_ring(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
+                     int splits, hipStream_t stream, int nt) {
+#define RING_CASE(NT_)                                                                                                  \
+  if (nt == NT_)                                                                                                        \
+    return M <= 32 ? launch_ring<NT_, 2, 4, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)      \
+                   : launch_ring<NT_, 4, 4, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  RING_CASE(2)
+  RING_CASE(4)
+  RING_CASE(6)
+#undef RING_CASE
+  if (nt == 5 && M > 32) return launch_ring<5, 4, 4, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  return ERR_BAD_ARGUMENT;
+}
+
+// As llmserve_gemm_skinny, for 16 < M <= 64 and K / splits a multiple of 128, through gemm_ring with `nt` tiles of
+// 16 weight rows a workgroup: 2, 4 or 6, or 5 for more than 32 rows.
+extern "C" int llmserve_gemm_ring(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
+                                  int out_is_float, int gated, int M, int N, int K, int splits, int nt,
+                                  hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || splits < 1 || K % splits || (gated && N % 2)) return ERR_BAD_ARGUMENT;
+  if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
+  if (gated)
+    return out_is_float ? pick_ring<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt)
+                        : pick_ring<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt);
+  return out_is_float ? pick_ring<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream, nt)
+                      : pick_ring<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt);
+}
+
 // ---------------------------------------------------------------------------- many rows
 // gemm_tiled: the same product for any number of rows of x (prompt portions), a tiled product:
 // a workgroup of four waves (2 x 2) computes a square tile of 64 * WT weight rows by 64 * WT rows

@@ -59,6 +59,7 @@ _SIGNATURES = {
     "llmserve_gemm_stream": "pppipiiiiiip",
     "llmserve_gemm_stream_shaped": "pppipiiiiiiiip",
     "llmserve_gemm_medium": "pppipiiiiiip",
+    "llmserve_gemm_ring": "pppipiiiiiiip",
     "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
     "llmserve_gemm_wide": "pppipiiiiiip",
@@ -151,6 +152,7 @@ class HipKernels:
         self._attention_generic = _declared(load_module("attention_generic"))
         self._gemm_bf16 = _declared(load_module("gemm_bf16")) if dtype == torch.bfloat16 else None
         self._pinned_stream: int | None = None
+        self.ring_products = True  # 17 to 64 rows of a large weight go to the kernel that streams it through a ring in LDS
         self._for_replay = False  # inside `replay_scope`: the step being launched is one that a graph will replay
         self._told: set[str] = set()
         if self._gemm_bf16 is not None and library_products:
@@ -310,6 +312,7 @@ class HipKernels:
 
     def _streaming(self, x: torch.Tensor, weights: LinearWeights, gated: bool = False) -> str | None:
         """Which MFMA kernel takes this product: "skinny" (up to 16 rows of x, weights streamed),
+        "ring" (17 to 64 rows of a middling weight, both operands through a ring of stages in LDS),
         "medium" (up to 64, x shared through LDS), "tiled" (any number, both operands through LDS),
         or None (the BLAS library, or the generic kernel)."""
         if x.dtype != torch.bfloat16 or weights.weight.dtype != torch.bfloat16:
@@ -317,6 +320,10 @@ class HipKernels:
         rows, inner = x.shape[0], weights.in_features
         if 0 < rows <= 16 and inner % 32 == 0:
             return "skinny"
+        if self.ring_products and 16 < rows <= 64 and inner % 128 == 0 and (1 << 22) < weights.out_features * inner <= 150_000_000:
+            # (a smaller weight: the kernels below; a larger one, which the library streams at what the memory gives: the
+            # 32B sizes' gate/up 103-115 us against 113-177, the 1.5B sizes' head 108-120 against 101-165)
+            return "ring"
         if self.library_products and (rows > 64 or self._for_replay):
             # On the device the library is ahead of "medium" as it stands, so a captured step (which
             # costs the host nothing per launch) takes the library; a step launched kernel by kernel
@@ -365,6 +372,34 @@ class HipKernels:
             if groups % splits == 0 and groups // splits >= shortest and tiles * splits <= 1024:
                 best = splits
         return best
+
+    @staticmethod
+    def _ring_shape(rows: int, out_features: int, in_features: int, may_split: bool) -> tuple[int, int]:
+        """How the product for 17 to 64 rows that streams its weights through a ring in LDS is shaped: (weight
+        tiles a workgroup, parts of K).  A workgroup fills most of a CU's LDS,
+        so the workgroups run in rounds of 256; a stage costs a workgroup what bringing its tiles of x costs plus
+        so much a weight tile, and a part of K what its partial sums cost to write and to add up.  The weights
+        of that estimate are fitted to measurements in a captured chain over different weights (us at 17 / 64
+        rows, the library or the older kernels against this one: 1.5B sizes gate/up 18.3 / 20.7 -> 14.9 / 17.6,
+        down 9.4 / 13.0 -> 9.1 / 12.2; 7B sizes gate/up 56.0 / 64.4 -> 50.8 / 58.9, down 34.1 / 44.1 -> 27.2 /
+        36.6, qkv 14.9 / 19.1 -> 13.2 / 17.0, o 12.9 / 14.1 -> 8.8 / 12.7; 32B sizes down 91.0 / 59.4 -> 57.3 /
+        60.9, o 20.4 / 22.3 -> 16.1 / 18.6)."""
+        tiles = -(-out_features // 16)
+        x_tiles = 2 if rows <= 32 else 4
+        stages = in_features // 128
+        best = None
+        for nt in (6, 5, 4, 2):
+            if nt == 5 and x_tiles != 4:
+                continue
+            groups = -(-tiles // nt)
+            for splits in range(1, 17 if may_split else 2):
+                if stages % splits or (stages // splits < 4 and splits > 1):
+                    continue
+                rounds = -(-groups * splits // 256)
+                cost = rounds * (stages // splits) * (0.25 * x_tiles + 0.45 * nt) + 0.5 * splits
+                if best is None or cost < best[0]:
+                    best = (cost, nt, splits)
+        return best[1], best[2]
 
     @staticmethod
     def _medium_splits(out_features: int, in_features: int) -> int:
@@ -423,6 +458,7 @@ class HipKernels:
         streaming = self._streaming(x, weights)
         if (
             streaming is None
+            and not self.ring_products
             and partial
             and out_dtype == torch.float32
             and x.dtype == torch.bfloat16
@@ -452,6 +488,15 @@ class HipKernels:
         bias_is_float = _is_float(bias) if bias is not None else 0
         if streaming is not None:
             splits = 1
+            if streaming == "ring":
+                tiles, splits = self._ring_shape(rows, weights.out_features, inner, partial and out_dtype == torch.float32)
+                out = self._empty((rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features), out_dtype or self.dtype)
+                status = self._gemm_bf16.llmserve_gemm_ring(
+                    _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out), _is_float(out), 0,
+                    rows, weights.out_features, inner, splits, tiles, self._stream,
+                )
+                _check(status, "linear")
+                return out
             if partial and out_dtype == torch.float32:
                 if streaming == "tiled":
                     splits = self._tiled_splits(rows, weights.out_features, inner)
@@ -538,6 +583,14 @@ class HipKernels:
             _check(status, "gated_linear")
             return out
         streaming = self._streaming(x, weights.both, gated=True)
+        if streaming == "ring":
+            tiles, _ = self._ring_shape(x.shape[0], 2 * weights.width, x.shape[1], False)
+            status = self._gemm_bf16.llmserve_gemm_ring(
+                _pointer(x), _pointer(weights.both.weight), None, 0, _pointer(out), _is_float(out), 1, x.shape[0],
+                2 * weights.width, x.shape[1], 1, tiles, self._stream,
+            )
+            _check(status, "gated_linear")
+            return out
         if streaming is not None:
             if streaming == "tiled":
                 status = self._gemm_bf16.llmserve_gemm_tiled(

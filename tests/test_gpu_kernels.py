@@ -1101,3 +1101,41 @@ def test_products_at_random_shapes(own):
                 summed = parts if parts.ndim == 2 else parts.sum(0)
                 torch.testing.assert_close(summed, want, atol=2e-4, rtol=2e-4, msg=lambda m: f"{said}, partial sums, replay {replayed}: {m}")
                 torch.testing.assert_close(k.gated_linear(x, gated_weights).float(), want_gated, **TOLERANCE[dtype], msg=lambda m: f"{said}, gated, replay {replayed}: {m}")
+
+
+@pytest.mark.parametrize("tiles", [2, 4, 5, 6])
+@pytest.mark.parametrize("rows,inner,outer,parts", [(17, 128, 48, 1), (33, 1536, 1000, 3), (64, 8960, 272, 10), (50, 384, 4099, 1), (32, 512, 130, 2)])
+def test_product_through_the_ring(kernels, tiles, rows, inner, outer, parts):
+    """The product for 17 to 64 rows whose weights and x go through a ring of stages in LDS, in every shape of
+    workgroup it has (2 to 6 tiles of 16 weight rows; 5 for more than 32 rows only): rows and weight rows that end
+    inside a tile, a K of one stage and of fewer stages than the ring has, with a bias, as float32 partial sums
+    and gated."""
+    from llmserve_amd.kernels.hip import KernelError, _check, _is_float, _pointer
+
+    k, dtype = kernels[torch.bfloat16], torch.bfloat16
+    library = k._gemm_bf16
+    x, w, b = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer)
+    up = torch.randn(outer, inner) / math.sqrt(inner)
+    want = rounded(x, dtype) @ rounded(w, dtype).T
+
+    def run(weight, bias, out, gated, splits):
+        return library.llmserve_gemm_ring(
+            _pointer(on_gpu(x, dtype)), _pointer(weight), _pointer(bias), _is_float(bias) if bias is not None else 0, _pointer(out),
+            _is_float(out), 1 if gated else 0, rows, weight.shape[0], inner, splits, tiles, k._stream)
+
+    weight, bias = on_gpu(w, dtype), on_gpu(b, dtype)
+    out = torch.empty(rows, outer, dtype=dtype, device="cuda")
+    if tiles == 5 and rows <= 32:
+        with pytest.raises(KernelError):
+            _check(run(weight, bias, out, False, 1), "ring")
+        return
+    _check(run(weight, bias, out, False, 1), "ring")
+    torch.testing.assert_close(out.cpu().double(), want + rounded(b, dtype), **TOLERANCE[dtype])
+    float_bias = on_gpu(b, torch.float32)
+    partial = torch.empty(parts, rows, outer, dtype=torch.float32, device="cuda")
+    _check(run(weight, float_bias, partial, False, parts), "ring")
+    torch.testing.assert_close(partial.sum(0).cpu().double(), want + b.double(), atol=1e-4, rtol=1e-4)
+    both = torch.stack([on_gpu(w, dtype), on_gpu(up, dtype)], dim=1).reshape(2 * outer, inner).contiguous()
+    gated = torch.empty(rows, outer, dtype=dtype, device="cuda")
+    _check(run(both, None, gated, True, 1), "ring")
+    torch.testing.assert_close(gated.cpu().double(), F.silu(want) * (rounded(x, dtype) @ rounded(up, dtype).T), **TOLERANCE[dtype])
