@@ -942,7 +942,49 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
       for (int i = 0; i < MINE; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(from_w[i][u], from_x[u], acc[i], 0, 0, 0);
   }
 
+  // The results leave through LDS as whole rows of the workgroup's tile, 16 bytes a lane, where the sizes allow it
+  // (each lane holds four neighbouring columns of one row: stored from the registers, an instruction writes 8 or 16
+  // bytes to each of sixteen rows).
+  constexpr int COLUMNS = GATED ? NT * 8 : NT * 16;        // of the workgroup's tile of the result
+  constexpr int PER_PIECE = 16 / (int)sizeof(TO);           // columns in 16 bytes
+  const int pitch = GATED ? N / 2 : N;                      // of a row of out
+  const int column0 = (int)blockIdx.x * COLUMNS;
+  const int valid = min(COLUMNS, pitch - column0);
+  TO* plane = out + (size_t)blockIdx.y * M * pitch;
+  const bool whole_pieces = pitch % PER_PIECE == 0 && valid % PER_PIECE == 0 && COLUMNS % PER_PIECE == 0 &&
+                            ((size_t)out & 15) == 0;
   const int m = x_tile * 16 + r;
+  if (whole_pieces) {
+    asm volatile("s_barrier" ::: "memory");  // everyone has read the last stage: the ring is free
+    TO* tile = (TO*)ring;                    // [16 MT rows][COLUMNS]
+#pragma unroll
+    for (int i = 0; i < MINE; ++i) {
+      f32x4 total = acc[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) total[j] += bias_here[i][j];
+      const int c_first = (first_tile + WAYS * i) * 16 + g * 4;  // column of the tile before gating
+      if (GATED) {
+        TO* dst = tile + m * COLUMNS + c_first / 2;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const float gate = total[2 * j], up = total[2 * j + 1];
+          dst[j] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+        }
+      } else {
+        TO* dst = tile + m * COLUMNS + c_first;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[j] = from_float<TO>(total[j]);
+      }
+    }
+    __syncthreads();
+    const int pieces_a_row = valid / PER_PIECE;
+    const int rows_here = min(M, 16 * MT);
+    for (int piece = threadIdx.x; piece < rows_here * pieces_a_row; piece += 256) {
+      const int row = piece / pieces_a_row, at = (piece - row * pieces_a_row) * PER_PIECE;
+      *(f32x4*)(plane + (size_t)row * pitch + column0 + at) = *(const f32x4*)(tile + row * COLUMNS + at);
+    }
+    return;
+  }
   if (m >= M) return;
 #pragma unroll
   for (int i = 0; i < MINE; ++i) {

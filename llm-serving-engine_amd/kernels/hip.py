@@ -380,10 +380,10 @@ class HipKernels:
         so the workgroups run in rounds of 256; a stage costs a workgroup what bringing its tiles of x costs plus
         so much a weight tile, and a part of K what its partial sums cost to write and to add up.  The weights
         of that estimate are fitted to measurements in a captured chain over different weights (us at 17 / 64
-        rows, the library or the older kernels against this one: 1.5B sizes gate/up 18.3 / 20.7 -> 14.9 / 17.6,
-        down 9.4 / 13.0 -> 9.1 / 12.2; 7B sizes gate/up 56.0 / 64.4 -> 50.8 / 58.9, down 34.1 / 44.1 -> 27.2 /
-        36.6, qkv 14.9 / 19.1 -> 13.2 / 17.0, o 12.9 / 14.1 -> 8.8 / 12.7; 32B sizes down 91.0 / 59.4 -> 57.3 /
-        60.9, o 20.4 / 22.3 -> 16.1 / 18.6)."""
+        rows, the library or the older kernels against this one: 1.5B sizes gate/up 18.2 / 20.7 -> 14.2 / 16.5,
+        down 9.4 / 12.9 -> 8.5 / 11.2; 7B sizes gate/up 56.1 / 64.9 -> 54.4 / 56.9, down 34.1 / 44.1 -> 26.8 /
+        35.6, qkv 15.0 / 19.2 -> 13.4 / 16.4, o 13.0 / 14.3 -> 8.3 / 11.5; 32B sizes down 91.1 / 59.6 -> 57.4 /
+        61.0, o 20.2 / 22.4 -> 15.6 / 18.6)."""
         tiles = -(-out_features // 16)
         x_tiles = 2 if rows <= 32 else 4
         stages = in_features // 128
