@@ -324,10 +324,11 @@ class HipKernels:
             # (a smaller weight: the kernels below; a larger one, which the library streams at what the memory gives: the
             # 32B sizes' gate/up 103-115 us against 113-177, the 1.5B sizes' head 108-120 against 101-165)
             return "ring"
-        if self.library_products and (rows > 64 or self._for_replay):
+        if self.library_products and (rows > 64 or self._for_replay or weights.out_features * inner > 150_000_000):
             # On the device the library is ahead of "medium" as it stands, so a captured step (which
             # costs the host nothing per launch) takes the library; a step launched kernel by kernel
-            # is bound by the host, where a torch call costs four times one of ours.
+            # is bound by the host, where a torch call costs four times one of ours (but a weight beyond what the
+            # ring takes goes to the library either way: the 1.5B sizes' head at 64 rows 112 us against 174).
             # Except a small weight: there the library's fixed cost shows (qkv and o of the 1.5B sizes in a
             # captured chain: 7.1-7.7 us each, against 4.8 and 4.0 at 17 rows, 5.0 and 4.5 at 32, 6.7 and 6.2 at
             # 64 for the kernel that brings two or four tiles of x through LDS beside a weight tile; where K is
