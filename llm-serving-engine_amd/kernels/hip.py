@@ -153,6 +153,7 @@ class HipKernels:
         self._gemm_bf16 = _declared(load_module("gemm_bf16")) if dtype == torch.bfloat16 else None
         self._pinned_stream: int | None = None
         self.ring_products = True  # 17 to 64 rows of a large weight go to the kernel that streams it through a ring in LDS
+        self.ring_rows_from = 4     # (and from this many rows on where K may be cut or the weight is very large)
         self._for_replay = False  # inside `replay_scope`: the step being launched is one that a graph will replay
         self._told: set[str] = set()
         if self._gemm_bf16 is not None and library_products:
@@ -310,7 +311,7 @@ class HipKernels:
         both = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
         return GatedLinearWeights(LinearWeights(both, None), gate.shape[0], activation)
 
-    def _streaming(self, x: torch.Tensor, weights: LinearWeights, gated: bool = False) -> str | None:
+    def _streaming(self, x: torch.Tensor, weights: LinearWeights, gated: bool = False, may_split: bool = False) -> str | None:
         """Which MFMA kernel takes this product: "skinny" (up to 16 rows of x, weights streamed),
         "ring" (17 to 64 rows of a middling weight, both operands through a ring of stages in LDS),
         "medium" (up to 64, x shared through LDS), "tiled" (any number, both operands through LDS),
@@ -318,9 +319,21 @@ class HipKernels:
         if x.dtype != torch.bfloat16 or weights.weight.dtype != torch.bfloat16:
             return None
         rows, inner = x.shape[0], weights.in_features
+        size = weights.out_features * inner
+        if self.ring_products and rows <= 16 and inner % 128 == 0 and size > (1 << 22):
+            # A few rows of a large weight do as well or better on the kernel written for 17 to 64 rows: from 4 rows on
+            # where the weight is very large or is large and its K may be cut over workgroups, from 12 rows on the
+            # middling ones.  Us at 4 / 8 / 16 rows in a captured chain over different weights: 7B sizes down 27.6 /
+            # 27.9 / 29.6 -> 26.1 / 26.4 / 26.6, gate/up 46.7 / 50.0 / 59.1 -> 47.7 / 48.1 / 50.4; 32B sizes gate/up 108.3
+            # / 111.2 / 120.6 -> 98.6 / 101.6 / 110.4; the 1.5B sizes' head 89.9 / 94.3 / 104.5 -> 82.7 / 88.0 / 97.1, their
+            # down projection and gate/up at 16 rows 9.5 and 15.9 -> 8.2 and 14.1 (at 8 rows 8.8 -> 8.1 alone, but
+            # the step it is in 1.434 -> 1.441 ms); a single row, and 7B qkv at 8 rows (11.8 -> 12.8), stay.
+            heavy = size > (1 << 26) or (may_split and size > (1 << 24))
+            if rows >= (self.ring_rows_from if heavy else max(12, self.ring_rows_from)) and (heavy or may_split or size > (1 << 24)):
+                return "ring"
         if 0 < rows <= 16 and inner % 32 == 0:
             return "skinny"
-        if self.ring_products and 16 < rows <= 64 and inner % 128 == 0 and (1 << 22) < weights.out_features * inner <= 150_000_000:
+        if self.ring_products and 16 < rows <= 64 and inner % 128 == 0 and (1 << 22) < size <= 150_000_000:
             # (a smaller weight: the kernels below; a larger one, which the library streams at what the memory gives: the
             # 32B sizes' gate/up 103-115 us against 113-177, the 1.5B sizes' head 108-120 against 101-165)
             return "ring"
@@ -396,7 +409,12 @@ class HipKernels:
             for splits in range(1, 17 if may_split else 2):
                 if stages % splits or (stages // splits < 4 and splits > 1):
                     continue
-                rounds = -(-groups * splits // 256)
+                # (a CU's LDS holds one such workgroup or two; two share what one would have alone, which costs a single
+                # round of them more than it costs many rounds, where the second hides the first's waits)
+                held, workgroups = min(2, 160 // ((nt + x_tiles) * 16)), groups * splits
+                rounds = -(-workgroups // (256 * held))
+                if held == 2 and workgroups > 256:
+                    rounds *= 1.8 if workgroups <= 512 else 1.5
                 cost = rounds * (stages // splits) * (0.25 * x_tiles + 0.45 * nt) + 0.5 * splits
                 if best is None or cost < best[0]:
                     best = (cost, nt, splits)
@@ -456,7 +474,7 @@ class HipKernels:
         if inner != weights.in_features:
             raise KernelError(f"linear: x has {inner} columns, the weight {weights.in_features}")
         bias = weights.bias
-        streaming = self._streaming(x, weights)
+        streaming = self._streaming(x, weights, may_split=partial and out_dtype == torch.float32)
         if (
             streaming is None
             and not self.ring_products
