@@ -257,26 +257,35 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
 }
 
 // out[column][:] = sum_s acc_s 2^(m_s - m) / sum_s l_s 2^(m_s - m) over the splits of a column, m the largest m_s.
+// One wave a column, at most 64 splits: lane s asks for split s's maximum and sum (one trip to memory for all of them;
+// a loop over the splits made one after the other), the wave agrees on the largest and on the total, and every lane
+// then adds up its dimensions over the splits, in split order, asking for eight of their partial sums at a time.
+#define MERGE_SPLITS_MAX 64
 __global__ __launch_bounds__(64) void attention_f32_merge_kernel(float* __restrict__ out,
                                                                 const float* __restrict__ partial_acc,
                                                                 const float* __restrict__ partial_ml, int splits,
                                                                 int columns_total) {
   const size_t column = blockIdx.x;
-  float best = -INFINITY;
-  for (int s = 0; s < splits; ++s) best = fmaxf(best, partial_ml[((size_t)s * columns_total + column) * 2]);
-  float sum = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float* ml = partial_ml + ((size_t)s * columns_total + column) * 2;
-    sum += ml[0] == -INFINITY ? 0.f : ml[1] * exp2f(ml[0] - best);
-  }
-  const float scale = sum > 0.f ? 1.f / sum : 0.f;
-  for (int d = threadIdx.x; d < D; d += 64) {
-    float total = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float m = partial_ml[((size_t)s * columns_total + column) * 2];
-      if (m != -INFINITY) total += partial_acc[((size_t)s * columns_total + column) * D + d] * exp2f(m - best);
+  const int lane = threadIdx.x;
+  const float2 mine = lane < splits ? *(const float2*)(partial_ml + ((size_t)lane * columns_total + column) * 2)
+                                    : make_float2(-INFINITY, 0.f);
+  const float best = wave_max(mine.x);
+  const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
+  const float total = wave_sum(mine.y * weight);                          // (lanes beyond the splits add 0)
+  const float inverse = total > 0.f ? 1.f / total : 0.f;
+  for (int d = lane; d < D; d += 64) {
+    float sum = 0.f;
+    for (int first = 0; first < splits; first += 8) {
+      float part[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) part[i] = partial_acc[((size_t)min(first + i, splits - 1) * columns_total + column) * D + d];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float w = __shfl(weight, min(first + i, MERGE_SPLITS_MAX - 1), 64);
+        if (first + i < splits && w != 0.f) sum += part[i] * w;
+      }
     }
-    out[column * D + d] = total * scale;
+    out[column * D + d] = sum * inverse;
   }
 }
 
@@ -292,7 +301,7 @@ extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* ou
                                       const float* slopes, float soft_cap, hipStream_t stream) {
   if (items <= 0 || tokens <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 4 || splits < 1 ||
-      (column_tiles != 1 && column_tiles != 2) || (splits > 1 && (!partial_acc || !partial_ml)))
+      splits > MERGE_SPLITS_MAX || (column_tiles != 1 && column_tiles != 2) || (splits > 1 && (!partial_acc || !partial_ml)))
     return ERR_BAD_ARGUMENT;
   const float scale_log2 = scale * 1.4426950408889634f;
   const int columns_total = tokens * heads;
