@@ -825,8 +825,8 @@ extern "C" int llmserve_gemm_medium(const void* x, const void* w, const void* bi
 // gemm_stream) DEPTH - 1 stages ahead of the one being multiplied: what a CU has under way is then that
 // many stages of weights whatever the compiler does with the registers, and a weight row is read from memory
 // once for all rows of x.  The waves divide a stage's chunks between them; one barrier a stage says that
-// everyone's loads have landed and that the stage before may be filled again.  Wave w multiplies the tile
-// w % MT of x with its share of the weight tiles, so no sums meet at the end.
+// everyone's loads have landed and that the stage before may be filled again.  A wave multiplies one tile of x
+// (two, with eight tiles of x: up to 128 rows) with its share of the weight tiles, so no sums meet at the end.
 __device__ __forceinline__ void ring_load(const bf16_t* from, unsigned to) {
   // (M0 names the place in LDS; it is put back, the compiler keeps other things there)
   unsigned kept;
@@ -852,13 +852,15 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
                                                         const void* __restrict__ bias, int bias_is_float,
                                                         TO* __restrict__ out, int M, int N, int K, int k_split) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
-  constexpr int WAYS = 4 / MT;          // groups of waves that divide the weight tiles between them
-  constexpr int MINE = NT / WAYS;       // weight tiles a wave multiplies
+  constexpr int XPW = MT > 4 ? MT / 4 : 1;   // tiles of x a wave multiplies
+  constexpr int XGROUPS = MT / XPW;          // groups of waves by their tiles of x
+  constexpr int WAYS = 4 / XGROUPS;          // groups of waves that divide the weight tiles between them
+  constexpr int MINE = NT / WAYS;            // weight tiles a wave multiplies
   constexpr int TILES = NT + MT;        // of a stage, each KSTEPS chunks of 1 KB
   constexpr int STAGE_BYTES = TILES * KSTEPS * STREAM_CHUNK;
   constexpr int PER_WAVE = TILES * KSTEPS / 4;  // chunks a wave brings per stage
   constexpr int APART = 4 / KSTEPS;             // tiles between two chunks of a wave
-  static_assert(MT == 2 || MT == 4, "two or four tiles of x");
+  static_assert(MT == 2 || MT == 4 || MT == 8, "two, four or eight tiles of x");
   static_assert(KSTEPS == 2 || KSTEPS == 4, "stages of 64 or 128 k");
   static_assert(NT % WAYS == 0, "the waves divide the weight tiles evenly");
   static_assert(TILES * KSTEPS % 4 == 0, "the waves divide a stage's chunks evenly");
@@ -879,7 +881,7 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
     src[j] = row + k_first + my_step * STEP + load_piece * 8;
   }
   const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ring;
-  const int x_tile = wave % MT, first_tile = wave / MT;
+  const int x_tile = (wave % XGROUPS) * XPW, first_tile = wave / XGROUPS;  // the wave's first tile of x, of weights
   const unsigned read_at = base + (unsigned)(4 * r + (g ^ ((r >> 1) & 3))) * 16;
   const unsigned read_w = read_at + (unsigned)first_tile * KSTEPS * STREAM_CHUNK;
   const unsigned read_x = read_at + (unsigned)(NT + x_tile) * KSTEPS * STREAM_CHUNK;
@@ -912,9 +914,11 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
     for (int j = 0; j < PER_WAVE; ++j)
       ring_load(src[j] + (size_t)stage * (KSTEPS * STEP), to + (unsigned)(j * APART * KSTEPS) * STREAM_CHUNK);
   };
-  f32x4 acc[MINE];
+  f32x4 acc[MINE][XPW];
 #pragma unroll
-  for (int i = 0; i < MINE; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < MINE; ++i)
+#pragma unroll
+    for (int j = 0; j < XPW; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < DEPTH - 1; ++s)
     if (s < stages) request(s);
@@ -925,13 +929,16 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
     asm volatile("s_barrier" ::: "memory");
     if (stage + DEPTH - 1 < stages) request(stage + DEPTH - 1);
     const unsigned slot = (unsigned)(stage % DEPTH) * STAGE_BYTES;
-    bf16x8 from_x[KSTEPS], from_w[MINE][KSTEPS];
-    StreamReads<0, KSTEPS>::run(from_x, read_x + slot);
+    bf16x8 from_x[XPW][KSTEPS], from_w[MINE][KSTEPS];
+#pragma unroll
+    for (int j = 0; j < XPW; ++j) StreamReads<0, KSTEPS>::run(from_x[j], read_x + slot + (unsigned)(j * KSTEPS) * STREAM_CHUNK);
 #pragma unroll
     for (int i = 0; i < MINE; ++i) StreamReads<0, KSTEPS>::run(from_w[i], read_w + slot + (unsigned)(WAYS * i * KSTEPS) * STREAM_CHUNK);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int u = 0; u < KSTEPS; ++u) asm volatile("" : "+v"(from_x[u]));  // used only after the wait
+    for (int j = 0; j < XPW; ++j)
+#pragma unroll
+      for (int u = 0; u < KSTEPS; ++u) asm volatile("" : "+v"(from_x[j][u]));  // used only after the wait
 #pragma unroll
     for (int i = 0; i < MINE; ++i)
 #pragma unroll
@@ -939,7 +946,10 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
 #pragma unroll
     for (int u = 0; u < KSTEPS; ++u)
 #pragma unroll
-      for (int i = 0; i < MINE; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(from_w[i][u], from_x[u], acc[i], 0, 0, 0);
+      for (int i = 0; i < MINE; ++i)
+#pragma unroll
+        for (int j = 0; j < XPW; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(from_w[i][u], from_x[j][u], acc[i][j], 0, 0, 0);
   }
 
   // The results leave through LDS as whole rows of the workgroup's tile, 16 bytes a lane, where the sizes allow it
@@ -953,27 +963,30 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
   TO* plane = out + (size_t)blockIdx.y * M * pitch;
   const bool whole_pieces = pitch % PER_PIECE == 0 && valid % PER_PIECE == 0 && COLUMNS % PER_PIECE == 0 &&
                             ((size_t)out & 15) == 0;
-  const int m = x_tile * 16 + r;
   if (whole_pieces) {
     asm volatile("s_barrier" ::: "memory");  // everyone has read the last stage: the ring is free
     TO* tile = (TO*)ring;                    // [16 MT rows][COLUMNS]
 #pragma unroll
-    for (int i = 0; i < MINE; ++i) {
-      f32x4 total = acc[i];
+    for (int t = 0; t < XPW; ++t) {
+      const int m = (x_tile + t) * 16 + r;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) total[j] += bias_here[i][j];
-      const int c_first = (first_tile + WAYS * i) * 16 + g * 4;  // column of the tile before gating
-      if (GATED) {
-        TO* dst = tile + m * COLUMNS + c_first / 2;
+      for (int i = 0; i < MINE; ++i) {
+        f32x4 total = acc[i][t];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const float gate = total[2 * j], up = total[2 * j + 1];
-          dst[j] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+        for (int j = 0; j < 4; ++j) total[j] += bias_here[i][j];
+        const int c_first = (first_tile + WAYS * i) * 16 + g * 4;  // column of the tile before gating
+        if (GATED) {
+          TO* dst = tile + m * COLUMNS + c_first / 2;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const float gate = total[2 * j], up = total[2 * j + 1];
+            dst[j] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+          }
+        } else {
+          TO* dst = tile + m * COLUMNS + c_first;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) dst[j] = from_float<TO>(total[j]);
         }
-      } else {
-        TO* dst = tile + m * COLUMNS + c_first;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) dst[j] = from_float<TO>(total[j]);
       }
     }
     __syncthreads();
@@ -985,27 +998,31 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(const bf16_t* __restrict
     }
     return;
   }
-  if (m >= M) return;
 #pragma unroll
-  for (int i = 0; i < MINE; ++i) {
-    const int n_first = ((int)blockIdx.x * NT + first_tile + WAYS * i) * 16 + g * 4;
-    f32x4 total = acc[i];
+  for (int t = 0; t < XPW; ++t) {
+    const int m = (x_tile + t) * 16 + r;
+    if (m >= M) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) total[j] += bias_here[i][j];
-    if (GATED) {
-      TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+    for (int i = 0; i < MINE; ++i) {
+      const int n_first = ((int)blockIdx.x * NT + first_tile + WAYS * i) * 16 + g * 4;
+      f32x4 total = acc[i][t];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if (n_first + 2 * j + 1 < N) {
-          const float gate = total[2 * j], up = total[2 * j + 1];
-          dst[j] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+      for (int j = 0; j < 4; ++j) total[j] += bias_here[i][j];
+      if (GATED) {
+        TO* dst = out + (size_t)m * (N / 2) + n_first / 2;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if (n_first + 2 * j + 1 < N) {
+            const float gate = total[2 * j], up = total[2 * j + 1];
+            dst[j] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+          }
         }
-      }
-    } else {
-      TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
+      } else {
+        TO* dst = out + ((size_t)blockIdx.y * M + m) * N + n_first;
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n_first + j < N) dst[j] = from_float<TO>(total[j]);
+        for (int j = 0; j < 4; ++j)
+          if (n_first + j < N) dst[j] = from_float<TO>(total[j]);
+      }
     }
   }
 }
@@ -1030,29 +1047,44 @@ static int launch_ring(const void* x, const void* w, const void* bias, int bias_
   return LAUNCH_STATUS();
 }
 
-// nt tiles of 16 weight rows a workgroup, stages of 128 k, four stages
+// nt tiles of 16 weight rows a workgroup, stages of 128 k; four stages, or three with eight tiles of x (65 to 128
+// rows), which fill the LDS with five weight tiles beside them
 template <typename TO, bool GATED>
 static int pick_ring(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
                      int splits, hipStream_t stream, int nt) {
 #define RING_CASE(NT_)                                                                                                  \
-  if (nt == NT_)                                                                                                        \
+  if (nt == NT_ && M <= 64)                                                                                             \
     return M <= 32 ? launch_ring<NT_, 2, 4, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)      \
                    : launch_ring<NT_, 4, 4, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
   RING_CASE(2)
   RING_CASE(4)
   RING_CASE(6)
 #undef RING_CASE
-  if (nt == 5 && M > 32) return launch_ring<5, 4, 4, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  if (nt == 5 && M > 32 && M <= 64) return launch_ring<5, 4, 4, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+#define ROWS_CASE(NT_)                                                                                                  \
+  if (nt == NT_ && M > 64) return launch_ring<NT_, 8, 4, 3, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  ROWS_CASE(2)
+  ROWS_CASE(4)
+  ROWS_CASE(5)
+#undef ROWS_CASE
+  // many weight tiles a workgroup, in stages of 64 k: for a weight of so many rows that fewer tiles make several rounds
+#define MANY_CASE(NT_)                                                                                                  \
+  if (nt == NT_ && M > 32)                                                                                              \
+    return M <= 64 ? launch_ring<NT_, 4, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)      \
+                   : launch_ring<NT_, 8, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  MANY_CASE(8)
+  MANY_CASE(10)
+#undef MANY_CASE
   return ERR_BAD_ARGUMENT;
 }
 
-// As llmserve_gemm_skinny, for 16 < M <= 64 and K / splits a multiple of 128, through gemm_ring with `nt` tiles of
-// 16 weight rows a workgroup: 2, 4 or 6, or 5 for more than 32 rows.
+// As llmserve_gemm_skinny, for M <= 128 and K / splits a multiple of 128, through gemm_ring with `nt` tiles of
+// 16 weight rows a workgroup: 2, 4 or 6 (up to 64 rows), or 5 (more than 32 rows).
 extern "C" int llmserve_gemm_ring(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
                                   int out_is_float, int gated, int M, int N, int K, int splits, int nt,
                                   hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || splits < 1 || K % splits || (gated && N % 2)) return ERR_BAD_ARGUMENT;
+  if (M > 128 || K <= 0 || splits < 1 || K % splits || (gated && N % 2)) return ERR_BAD_ARGUMENT;
   if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
   if (gated)
     return out_is_float ? pick_ring<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt)

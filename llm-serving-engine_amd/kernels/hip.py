@@ -337,6 +337,17 @@ class HipKernels:
             # (a smaller weight: the kernels below; a larger one, which the library streams at what the memory gives: the
             # 32B sizes' gate/up 103-115 us against 113-177, the 1.5B sizes' head 108-120 against 101-165)
             return "ring"
+        if self.ring_products and 64 < rows <= 128 and inner % 128 == 0 and (
+            (may_split and (1 << 20) < size <= 150_000_000) or (gated and (1 << 22) < size <= 150_000_000)
+        ):
+            # 65 to 128 rows, where the step from the kernel above to the library was a cliff (a decode step of the 1.5B
+            # sizes 2.01 ms at 64 rows and 2.76 at 65): the same kernel with eight tiles of x for the products whose K
+            # may be cut and the smaller gated ones.  Us at 65 / 128 rows in a captured chain over different weights,
+            # the library against it: 1.5B sizes gate/up with its activation 25.8 / 26.5 -> 21.9 / 22.3, down 21.8 / 23.2 ->
+            # 13.4 / 14.7, o 7.5 -> 5.8 / 6.3; 7B sizes down 40.1 / 52.4 -> 44.3 / 45.1, o 18.6 / 22.6 -> 13.2 / 14.3; the
+            # gate/up with ten weight tiles a workgroup, 237 workgroups, 67.1 / 72.1 -> 59.1 / 61.3 (80-82 with five, which
+            # make 474); the library keeps qkv (7.5 against 10.2; 19-23 against 21-23).
+            return "ring"
         if self.library_products and (rows > 64 or self._for_replay or weights.out_features * inner > 150_000_000):
             # On the device the library is ahead of "medium" as it stands, so a captured step (which
             # costs the host nothing per launch) takes the library; a step launched kernel by kernel
@@ -399,19 +410,21 @@ class HipKernels:
         35.6, qkv 15.0 / 19.2 -> 13.4 / 16.4, o 13.0 / 14.3 -> 8.3 / 11.5; 32B sizes down 91.1 / 59.6 -> 57.4 /
         61.0, o 20.2 / 22.4 -> 15.6 / 18.6)."""
         tiles = -(-out_features // 16)
-        x_tiles = 2 if rows <= 32 else 4
+        x_tiles = 2 if rows <= 32 else 4 if rows <= 64 else 8
         stages = in_features // 128
         best = None
-        for nt in (6, 5, 4, 2):
-            if nt == 5 and x_tiles != 4:
-                continue
+        for nt in (10, 8, 6, 5, 4, 2):
+            if (nt == 5 and x_tiles < 4) or (nt == 6 and x_tiles > 4) or (nt >= 8 and (x_tiles < 4 or may_split)):
+                continue  # (many tiles a workgroup are for the products whose K stays whole: cutting K makes workgroups enough)
+            # of LDS a tile: four stages of 4 KB, three beside eight tiles of x; eight and ten weight tiles in stages of 2 KB
+            stage_kb = 8 if nt >= 8 else 16 if x_tiles < 8 else 12
             groups = -(-tiles // nt)
             for splits in range(1, 17 if may_split else 2):
                 if stages % splits or (stages // splits < 4 and splits > 1):
                     continue
                 # (a CU's LDS holds one such workgroup or two; two share what one would have alone, which costs a single
                 # round of them more than it costs many rounds, where the second hides the first's waits)
-                held, workgroups = min(2, 160 // ((nt + x_tiles) * 16)), groups * splits
+                held, workgroups = min(2, 160 // ((nt + x_tiles) * stage_kb)), groups * splits
                 rounds = -(-workgroups // (256 * held))
                 if held == 2 and workgroups > 256:
                     rounds *= 1.8 if workgroups <= 512 else 1.5
@@ -585,6 +598,7 @@ class HipKernels:
         return best
 
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
+        """silu (or another activation) of the even rows' products times the odd rows'."""
         out = self._empty((x.shape[0], weights.width), self.dtype)
         if weights.activation != "silu":  # no fused epilogue: the product plain, the activation behind it
             both = self.linear(x, weights.both, out_dtype=torch.bfloat16 if self._library(x, weights.both) else torch.float32)
