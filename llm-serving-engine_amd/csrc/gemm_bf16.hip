@@ -1069,17 +1069,21 @@ static int pick_ring(const void* x, const void* w, const void* bias, int bias_is
 #undef ROWS_CASE
   // many weight tiles a workgroup, in stages of 64 k: for a weight of so many rows that fewer tiles make several rounds
 #define MANY_CASE(NT_)                                                                                                  \
-  if (nt == NT_ && M > 32)                                                                                              \
-    return M <= 64 ? launch_ring<NT_, 4, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)      \
-                   : launch_ring<NT_, 8, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  if (nt == NT_ && M <= 64)                                                                                             \
+    return M <= 32 ? launch_ring<NT_, 2, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)      \
+                   : launch_ring<NT_, 4, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
   MANY_CASE(8)
   MANY_CASE(10)
+  MANY_CASE(12)
+  MANY_CASE(14)
 #undef MANY_CASE
+  if (nt == 8 && M > 64) return launch_ring<8, 8, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
+  if (nt == 10 && M > 64) return launch_ring<10, 8, 2, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
   return ERR_BAD_ARGUMENT;
 }
 
 // As llmserve_gemm_skinny, for M <= 128 and K / splits a multiple of 128, through gemm_ring with `nt` tiles of
-// 16 weight rows a workgroup: 2, 4 or 6 (up to 64 rows), or 5 (more than 32 rows).
+// 16 weight rows a workgroup: 2, 4 or 6 (up to 64 rows), 5 (more than 32 rows), 8 or 10, or 12 or 14 (up to 64 rows).
 extern "C" int llmserve_gemm_ring(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
                                   int out_is_float, int gated, int M, int N, int K, int splits, int nt,
                                   hipStream_t stream) {

@@ -321,21 +321,26 @@ class HipKernels:
         rows, inner = x.shape[0], weights.in_features
         size = weights.out_features * inner
         if self.ring_products and rows <= 16 and inner % 128 == 0 and size > (1 << 22):
-            # A few rows of a large weight do as well or better on the kernel written for 17 to 64 rows: from 4 rows on
-            # where the weight is very large or is large and its K may be cut over workgroups, from 12 rows on the
-            # middling ones.  Us at 4 / 8 / 16 rows in a captured chain over different weights: 7B sizes down 27.6 /
-            # 27.9 / 29.6 -> 26.1 / 26.4 / 26.6, gate/up 46.7 / 50.0 / 59.1 -> 47.7 / 48.1 / 50.4; 32B sizes gate/up 108.3
-            # / 111.2 / 120.6 -> 98.6 / 101.6 / 110.4; the 1.5B sizes' head 89.9 / 94.3 / 104.5 -> 82.7 / 88.0 / 97.1, their
-            # down projection and gate/up at 16 rows 9.5 and 15.9 -> 8.2 and 14.1 (at 8 rows 8.8 -> 8.1 alone, but
-            # the step it is in 1.434 -> 1.441 ms); a single row, and 7B qkv at 8 rows (11.8 -> 12.8), stay.
+            # A few rows of a large weight do as well or better on the kernel written for 17 to 64 rows where its
+            # workgroups make one round: from 4 rows on where the weight is very large or is large and its K may be
+            # cut over workgroups, from 12 rows on the middling ones.  Us at 4 / 8 / 16 rows in a captured chain over
+            # different weights: 7B sizes down 27.5 / 28.0 / 29.6 -> 26.2 / 26.3 / 26.5, gate/up 46.9 / 49.9 / 58.9 -> 47.6 /
+            # 47.7 / 47.9; 32B sizes gate/up 108.3 / 110.9 / 120.2 -> 100.8 / 101.1 / 101.3; the 1.5B sizes' down projection
+            # and gate/up at 16 rows 10.3 and 15.8 -> 8.2 and 14.0 (at 8 rows 8.8 -> 8.1 alone, but the step it is in 1.434 ->
+            # 1.441 ms); a single row, 7B qkv at 8 rows (11.8 -> 12.8) and what would take several rounds (the 1.5B sizes'
+            # head 89.6 / 94.2 -> 93.3 / 94.9, the 32B sizes' down projection 52.5 -> 54.2) stay.
             heavy = size > (1 << 26) or (may_split and size > (1 << 24))
             if rows >= (self.ring_rows_from if heavy else max(12, self.ring_rows_from)) and (heavy or may_split or size > (1 << 24)):
-                return "ring"
+                if self._ring_shape(rows, weights.out_features, inner, may_split)[2] == 1:
+                    return "ring"
         if 0 < rows <= 16 and inner % 32 == 0:
             return "skinny"
-        if self.ring_products and 16 < rows <= 64 and inner % 128 == 0 and (1 << 22) < size <= 150_000_000:
-            # (a smaller weight: the kernels below; a larger one, which the library streams at what the memory gives: the
-            # 32B sizes' gate/up 103-115 us against 113-177, the 1.5B sizes' head 108-120 against 101-165)
+        if self.ring_products and 16 < rows <= 64 and inner % 128 == 0 and size > (1 << 22) and (
+            size <= 150_000_000 or weights.out_features <= 256 * 14 * 16
+        ):
+            # (a smaller weight: the kernels below; a larger one only while fourteen tiles a workgroup make one round of
+            # workgroups: the 32B sizes' gate/up 100-110 us at the library, 98-106 here, 113-177 in several rounds; the 1.5B
+            # sizes' head, 9,496 tiles, 108-120 against 101-165)
             return "ring"
         if self.ring_products and 64 < rows <= 128 and inner % 128 == 0 and (
             (may_split and (1 << 20) < size <= 150_000_000) or (gated and (1 << 22) < size <= 150_000_000)
@@ -399,9 +404,9 @@ class HipKernels:
         return best
 
     @staticmethod
-    def _ring_shape(rows: int, out_features: int, in_features: int, may_split: bool) -> tuple[int, int]:
+    def _ring_shape(rows: int, out_features: int, in_features: int, may_split: bool) -> tuple[int, int, int]:
         """How the product for 17 to 64 rows that streams its weights through a ring in LDS is shaped: (weight
-        tiles a workgroup, parts of K).  A workgroup fills most of a CU's LDS,
+        tiles a workgroup, parts of K, rounds of workgroups).  A workgroup fills most of a CU's LDS,
         so the workgroups run in rounds of 256; a stage costs a workgroup what bringing its tiles of x costs plus
         so much a weight tile, and a part of K what its partial sums cost to write and to add up.  The weights
         of that estimate are fitted to measurements in a captured chain over different weights (us at 17 / 64
@@ -413,8 +418,8 @@ class HipKernels:
         x_tiles = 2 if rows <= 32 else 4 if rows <= 64 else 8
         stages = in_features // 128
         best = None
-        for nt in (10, 8, 6, 5, 4, 2):
-            if (nt == 5 and x_tiles < 4) or (nt == 6 and x_tiles > 4) or (nt >= 8 and (x_tiles < 4 or may_split)):
+        for nt in (14, 12, 10, 8, 6, 5, 4, 2):
+            if (nt == 5 and x_tiles < 4) or (nt == 6 and x_tiles > 4) or (nt >= 8 and may_split) or (nt >= 12 and x_tiles > 4):
                 continue  # (many tiles a workgroup are for the products whose K stays whole: cutting K makes workgroups enough)
             # of LDS a tile: four stages of 4 KB, three beside eight tiles of x; eight and ten weight tiles in stages of 2 KB
             stage_kb = 8 if nt >= 8 else 16 if x_tiles < 8 else 12
@@ -422,16 +427,17 @@ class HipKernels:
             for splits in range(1, 17 if may_split else 2):
                 if stages % splits or (stages // splits < 4 and splits > 1):
                     continue
-                # (a CU's LDS holds one such workgroup or two; two share what one would have alone, which costs a single
-                # round of them more than it costs many rounds, where the second hides the first's waits)
+                # (a CU's LDS holds one such workgroup or two; two share what one would have alone)
                 held, workgroups = min(2, 160 // ((nt + x_tiles) * stage_kb)), groups * splits
                 rounds = -(-workgroups // (256 * held))
-                if held == 2 and workgroups > 256:
-                    rounds *= 1.8 if workgroups <= 512 else 1.5
                 cost = rounds * (stages // splits) * (0.25 * x_tiles + 0.45 * nt) + 0.5 * splits
+                if held == 2 and workgroups > 256:
+                    cost *= 1.8
+                if rounds > 1:
+                    cost *= 1.25  # (the last round is seldom full, and every round starts and ends)
                 if best is None or cost < best[0]:
-                    best = (cost, nt, splits)
-        return best[1], best[2]
+                    best = (cost, nt, splits, rounds)
+        return best[1], best[2], best[3]
 
     @staticmethod
     def _medium_splits(out_features: int, in_features: int) -> int:
@@ -521,7 +527,7 @@ class HipKernels:
         if streaming is not None:
             splits = 1
             if streaming == "ring":
-                tiles, splits = self._ring_shape(rows, weights.out_features, inner, partial and out_dtype == torch.float32)
+                tiles, splits, _ = self._ring_shape(rows, weights.out_features, inner, partial and out_dtype == torch.float32)
                 out = self._empty((rows, weights.out_features) if splits == 1 else (splits, rows, weights.out_features), out_dtype or self.dtype)
                 status = self._gemm_bf16.llmserve_gemm_ring(
                     _pointer(x), _pointer(weights.weight), _pointer(bias), bias_is_float, _pointer(out), _is_float(out), 0,
@@ -617,7 +623,7 @@ class HipKernels:
             return out
         streaming = self._streaming(x, weights.both, gated=True)
         if streaming == "ring":
-            tiles, _ = self._ring_shape(x.shape[0], 2 * weights.width, x.shape[1], False)
+            tiles, _, _ = self._ring_shape(x.shape[0], 2 * weights.width, x.shape[1], False)
             status = self._gemm_bf16.llmserve_gemm_ring(
                 _pointer(x), _pointer(weights.both.weight), None, 0, _pointer(out), _is_float(out), 1, x.shape[0],
                 2 * weights.width, x.shape[1], 1, tiles, self._stream,

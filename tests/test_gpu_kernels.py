@@ -1103,13 +1103,13 @@ def test_products_at_random_shapes(own):
                 torch.testing.assert_close(k.gated_linear(x, gated_weights).float(), want_gated, **TOLERANCE[dtype], msg=lambda m: f"{said}, gated, replay {replayed}: {m}")
 
 
-@pytest.mark.parametrize("tiles", [2, 4, 5, 6, 8, 10])
+@pytest.mark.parametrize("tiles", [2, 4, 5, 6, 8, 10, 12, 14])
 @pytest.mark.parametrize("rows,inner,outer,parts", [(17, 128, 48, 1), (33, 1536, 1000, 3), (64, 8960, 272, 10), (50, 384, 4099, 1), (32, 512, 130, 2),
                                                     (8, 1024, 300, 2), (65, 256, 100, 1), (100, 1536, 1000, 4), (128, 3584, 272, 7)])
 def test_product_through_the_ring(kernels, tiles, rows, inner, outer, parts):
     """The product for up to 128 rows whose weights and x go through a ring of stages in LDS, in every shape of
-    workgroup it has (2 to 10 tiles of 16 weight rows; 5, 8 and 10 for more than 32 rows only, 6 for up to 64): rows and
-    weight rows that end inside a tile, a K of one stage and of fewer stages than the ring has, with a bias, as float32
+    workgroup it has (2 to 14 tiles of 16 weight rows; 5 for more than 32 rows only, 6, 12 and 14 for up to 64): rows
+    and weight rows that end inside a tile, a K of one stage and of fewer stages than the ring has, with a bias, as float32
     partial sums and gated."""
     from llmserve_amd.kernels.hip import KernelError, _check, _is_float, _pointer
 
@@ -1126,7 +1126,7 @@ def test_product_through_the_ring(kernels, tiles, rows, inner, outer, parts):
 
     weight, bias = on_gpu(w, dtype), on_gpu(b, dtype)
     out = torch.empty(rows, outer, dtype=dtype, device="cuda")
-    if (tiles in (5, 8, 10) and rows <= 32) or (tiles == 6 and rows > 64):
+    if (tiles == 5 and rows <= 32) or (tiles in (6, 12, 14) and rows > 64):
         with pytest.raises(KernelError):
             _check(run(weight, bias, out, False, 1), "ring")
         return
