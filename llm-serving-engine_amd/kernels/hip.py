@@ -405,15 +405,18 @@ class HipKernels:
 
     @staticmethod
     def _ring_shape(rows: int, out_features: int, in_features: int, may_split: bool) -> tuple[int, int, int]:
-        """How the product for 17 to 64 rows that streams its weights through a ring in LDS is shaped: (weight
-        tiles a workgroup, parts of K, rounds of workgroups).  A workgroup fills most of a CU's LDS,
-        so the workgroups run in rounds of 256; a stage costs a workgroup what bringing its tiles of x costs plus
-        so much a weight tile, and a part of K what its partial sums cost to write and to add up.  The weights
-        of that estimate are fitted to measurements in a captured chain over different weights (us at 17 / 64
-        rows, the library or the older kernels against this one: 1.5B sizes gate/up 18.2 / 20.7 -> 14.2 / 16.5,
-        down 9.4 / 12.9 -> 8.5 / 11.2; 7B sizes gate/up 56.1 / 64.9 -> 54.4 / 56.9, down 34.1 / 44.1 -> 26.8 /
-        35.6, qkv 15.0 / 19.2 -> 13.4 / 16.4, o 13.0 / 14.3 -> 8.3 / 11.5; 32B sizes down 91.1 / 59.6 -> 57.4 /
-        61.0, o 20.2 / 22.4 -> 15.6 / 18.6)."""
+        """How the product that streams its weights through a ring in LDS is shaped: (weight tiles a workgroup,
+        parts of K, rounds of workgroups).  A workgroup fills most of a CU's LDS, so the workgroups run in
+        rounds of 256 (512 where two fit), and what decides is whether one round takes them all: five tiles a
+        workgroup of the 1.5B sizes' gate/up (224 workgroups) take 16.4 us at 64 rows, four (280) 25.2; ten tiles of
+        the 7B sizes' (237) 52.8, five (474) 56.3.  A stage costs a workgroup what bringing its tiles of x costs
+        plus so much a weight tile, a part of K what its partial sums cost to write and to add up, further rounds
+        a quarter more.  The weights of that estimate are fitted to measurements in a captured chain over
+        different weights (us at 17 / 64 rows, the library or the older kernels against this one: 1.5B sizes
+        gate/up 18.1 / 20.7 -> 14.4 / 16.4, down 9.5 / 13.0 -> 8.5 / 11.2; 7B sizes gate/up 55.9 / 64.5 -> 48.1 / 53.3,
+        down 34.4 / 44.0 -> 26.7 / 35.9, qkv 14.9 / 19.1 -> 13.6 / 16.5, o 13.0 / 14.2 -> 8.4 / 11.7; 32B sizes gate/up
+        103.4 / 114.8 -> 101.5 / 108.8, down 91.1 / 58.8 -> 52.1 / 59.1, o 20.2 / 22.3 -> 14.6 / 16.8, qkv 19.8 / 25.6 ->
+        18.8 / 27.7)."""
         tiles = -(-out_features // 16)
         x_tiles = 2 if rows <= 32 else 4 if rows <= 64 else 8
         stages = in_features // 128
