@@ -1077,9 +1077,9 @@ def test_products_at_random_shapes(own):
     dtype = torch.bfloat16
     k = HipKernels(dtype, library_products=not own)
     generator = torch.Generator(device="cuda").manual_seed(5)
-    for seed in range(150):
+    for seed in range(200):
         draw = random.Random(1000 + seed)
-        rows = draw.choice([1, 2, 3, 5, 8, 13, 16, 17, 24, 32, 33, 48, 64, 65, 130, 300])
+        rows = draw.choice([1, 2, 3, 5, 8, 13, 16, 17, 24, 32, 33, 48, 64, 65, 100, 128, 130, 300])
         inner = 32 * draw.choice([1, 3, 4, 8, 12, 16, 28, 40, 48, 64, 70, 112, 148, 160, 216, 280])
         outer = draw.choice([16, 48, 100, 256, 272, 1000, 1536, 2048, 4099, 5120, 17920])
         if rows > 64 and inner * outer > 1 << 24:
