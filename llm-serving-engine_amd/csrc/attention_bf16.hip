@@ -623,70 +623,77 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
 // 2^(m_s - m), in split order (the maxima are kept in units of log2).  A second kernel rather than "the last workgroup merges": a
 // workgroup that reads what others wrote needs the other chiplets' L2 written back first, and
 // that costs more than this launch.
-// One wave a (token, head), at most 64 splits: lane s asks for split s's maximum and sum (one trip to
+// A thread a dimension, at most 64 splits: in every wave lane s asks for split s's maximum and sum (one trip to
 // memory for all of them, where a loop over the splits made one after the other: nine splits took
-// 14.6 us, thirty-three 41), the wave agrees on the largest and on the total, and every lane then adds
-// up its dimensions over the splits, whose partial sums it asks for eight at a time.
+// 14.6 us, thirty-three 41), the wave agrees on the largest and on the total, and every thread then adds up
+// its dimension over the splits, whose partial sums it asks for up to thirty-two at a time (one wave that took two
+// dimensions a lane and eight splits at a time made six trips in a row for twenty-four splits; attention and merge
+// together, us a layer: one request over 8,192 keys in 64 splits 16.5 -> 11.4, four over 16,384 in 48 30.0 -> 26.9,
+// eight over 30,000 in 12 52.7 -> 50.5).
 #define MERGE_SPLITS_MAX 64
-__global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ partial_acc,
-                                                               const float* __restrict__ partial_ml,
-                                                               bf16_t* __restrict__ out, int splits) {
-  const size_t pair = blockIdx.x;  // row * heads + head
-  const int lane = threadIdx.x;
-  const float2 mine = lane < splits ? *(const float2*)(partial_ml + (pair * splits + lane) * 2) : make_float2(-INFINITY, 0.f);
+constexpr int MERGE_THREADS = (D + WAVE - 1) / WAVE * WAVE;
+
+template <int AT_ONCE>
+__device__ __forceinline__ float merge_some(const float* acc, int first, int splits, float weight) {
+  float part[AT_ONCE];
+#pragma unroll
+  for (int i = 0; i < AT_ONCE; ++i) part[i] = acc[(size_t)min(first + i, splits - 1) * D];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < AT_ONCE; ++i) {
+    const float w = __shfl(weight, min(first + i, MERGE_SPLITS_MAX - 1), WAVE);
+    if (first + i < splits && w != 0.f) sum += part[i] * w;
+  }
+  return sum;
+}
+
+// sum_s acc_s[d] w_s / sum_s l_s w_s of the splits whose maxima and sums lie at `ml` and partial sums at `acc`;
+// every lane of every wave must call it (the weights pass between lanes)
+__device__ __forceinline__ float merged_dimension(const float* ml, const float* acc, int splits, int d) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const float2 mine = lane < splits ? *(const float2*)(ml + (size_t)lane * 2) : make_float2(-INFINITY, 0.f);
   const float best = wave_max(mine.x);
   const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
-  const float total = wave_sum(mine.y * weight);  // (lanes beyond the splits add 0)
+  const float total = wave_sum(mine.y * weight);                          // (lanes beyond the splits add 0)
   const float inverse = total > 0.f ? 1.f / total : 0.f;
-  const float* acc = partial_acc + pair * splits * D;
-  for (int d = lane; d < D; d += WAVE) {
-    float sum = 0.f;
-    for (int first = 0; first < splits; first += 8) {
-      float part[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) part[i] = acc[(size_t)min(first + i, splits - 1) * D + d];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float w = __shfl(weight, min(first + i, MERGE_SPLITS_MAX - 1), WAVE);
-        if (first + i < splits && w != 0.f) sum += part[i] * w;
-      }
-    }
-    out[pair * D + d] = (bf16_t)(sum * inverse);
-  }
+  const float* mine_acc = acc + min(d, D - 1);
+  float sum = 0.f;
+  int first = 0;
+  for (; splits - first > 8; first += 32) sum += merge_some<32>(mine_acc, first, splits, weight);
+  if (first < splits) sum += merge_some<8>(mine_acc, first, splits, weight);
+  return sum * inverse;
+}
+
+__global__ __launch_bounds__(MERGE_THREADS) void attention_merge_kernel(const float* __restrict__ partial_acc,
+                                                                        const float* __restrict__ partial_ml,
+                                                                        bf16_t* __restrict__ out, int splits) {
+  const size_t pair = blockIdx.x;  // row * heads + head
+  const int d = threadIdx.x;
+  const float merged = merged_dimension(partial_ml + pair * splits * 2, partial_acc + pair * splits * D, splits, d);
+  if (d < D) out[pair * D + d] = (bf16_t)merged;
 }
 
 // The same for partial results that are kept by work item: workgroup (item, head) merges the item's tokens one
 // after the other (a few), and writes to the rows that the item names.
-__global__ __launch_bounds__(WAVE) void attention_merge_items_kernel(const float* __restrict__ partial_acc,
-                                                                     const float* __restrict__ partial_ml,
-                                                                     bf16_t* __restrict__ out, const int* __restrict__ work,
-                                                                     int splits, int heads, int group, int tokens_per_tile) {
+__global__ __launch_bounds__(MERGE_THREADS) void attention_merge_items_kernel(const float* __restrict__ partial_acc,
+                                                                              const float* __restrict__ partial_ml,
+                                                                              bf16_t* __restrict__ out,
+                                                                              const int* __restrict__ work, int splits,
+                                                                              int heads, int group, int tokens_per_tile) {
   const int* item = work + (size_t)blockIdx.x * 4;
   const int tokens = group <= 16 ? (item[2] + item[3] + group - 1) / group : item[3];
-  const int head = blockIdx.y, lane = threadIdx.x;
+  const int head = blockIdx.y, d = threadIdx.x;
   for (int token = 0; token < tokens; ++token) {
     const size_t kept_as = ((size_t)blockIdx.x * tokens_per_tile + token) * heads + head;
     const size_t pair = ((size_t)item[1] + token) * heads + head;
-    const float2 mine = lane < splits ? *(const float2*)(partial_ml + (kept_as * splits + lane) * 2) : make_float2(-INFINITY, 0.f);
-    const float best = wave_max(mine.x);
-    const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);
-    const float total = wave_sum(mine.y * weight);
-    const float inverse = total > 0.f ? 1.f / total : 0.f;
-    const float* acc = partial_acc + kept_as * splits * D;
-    for (int d = lane; d < D; d += WAVE) {
-      float sum = 0.f;
-      for (int split = 0; split < splits; ++split) {
-        const float w = __shfl(weight, split, WAVE);
-        if (w != 0.f) sum += acc[(size_t)split * D + d] * w;
-      }
-      out[pair * D + d] = (bf16_t)(sum * inverse);
-    }
+    const float merged = merged_dimension(partial_ml + kept_as * splits * 2, partial_acc + kept_as * splits * D, splits, d);
+    if (d < D) out[pair * D + d] = (bf16_t)merged;
   }
 }
 
 static int launch_merge(float* partial_acc, float* partial_ml, void* out, int splits, size_t pairs, hipStream_t stream) {
-  hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)pairs), dim3(WAVE), 0, stream, partial_acc, partial_ml,
-                     (bf16_t*)out, splits);
+  hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)pairs), dim3(MERGE_THREADS), 0, stream, partial_acc,
+                     partial_ml, (bf16_t*)out, splits);
   return LAUNCH_STATUS();
 }
 
@@ -1067,7 +1074,7 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   }
   if (status != 0 || splits == 1 || unmerged) return status;
   if (by_item) {
-    hipLaunchKernelGGL(attention_merge_items_kernel, dim3(tiles, heads), dim3(WAVE), 0, stream, partial_acc, partial_ml,
+    hipLaunchKernelGGL(attention_merge_items_kernel, dim3(tiles, heads), dim3(MERGE_THREADS), 0, stream, partial_acc, partial_ml,
                        (bf16_t*)out, work, splits, heads, group, tokens_per_tile);
     return LAUNCH_STATUS();
   }
