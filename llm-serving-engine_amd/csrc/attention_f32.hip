@@ -257,36 +257,46 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
 }
 
 // out[column][:] = sum_s acc_s 2^(m_s - m) / sum_s l_s 2^(m_s - m) over the splits of a column, m the largest m_s.
-// One wave a column, at most 64 splits: lane s asks for split s's maximum and sum (one trip to memory for all of them;
-// a loop over the splits made one after the other), the wave agrees on the largest and on the total, and every lane
-// then adds up its dimensions over the splits, in split order, asking for eight of their partial sums at a time.
+// A thread a dimension, at most 64 splits: in every wave lane s asks for split s's maximum and sum (one trip to memory
+// for all of them; a loop over the splits made one after the other), the wave agrees on the largest and on the total,
+// and every thread then adds up its dimension over the splits, in split order, asking for up to thirty-two of their
+// partial sums at a time.
 #define MERGE_SPLITS_MAX 64
-__global__ __launch_bounds__(64) void attention_f32_merge_kernel(float* __restrict__ out,
-                                                                const float* __restrict__ partial_acc,
-                                                                const float* __restrict__ partial_ml, int splits,
-                                                                int columns_total) {
+constexpr int MERGE_THREADS = (D + 63) / 64 * 64;
+
+template <int AT_ONCE>
+__device__ __forceinline__ float merge_some(const float* acc, size_t split_stride, int first, int splits, float weight) {
+  float part[AT_ONCE];
+#pragma unroll
+  for (int i = 0; i < AT_ONCE; ++i) part[i] = acc[(size_t)min(first + i, splits - 1) * split_stride];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < AT_ONCE; ++i) {
+    const float w = __shfl(weight, min(first + i, MERGE_SPLITS_MAX - 1), 64);
+    if (first + i < splits && w != 0.f) sum += part[i] * w;
+  }
+  return sum;
+}
+
+__global__ __launch_bounds__(MERGE_THREADS) void attention_f32_merge_kernel(float* __restrict__ out,
+                                                                           const float* __restrict__ partial_acc,
+                                                                           const float* __restrict__ partial_ml,
+                                                                           int splits, int columns_total) {
   const size_t column = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, d = threadIdx.x;
   const float2 mine = lane < splits ? *(const float2*)(partial_ml + ((size_t)lane * columns_total + column) * 2)
                                     : make_float2(-INFINITY, 0.f);
   const float best = wave_max(mine.x);
   const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
   const float total = wave_sum(mine.y * weight);                          // (lanes beyond the splits add 0)
   const float inverse = total > 0.f ? 1.f / total : 0.f;
-  for (int d = lane; d < D; d += 64) {
-    float sum = 0.f;
-    for (int first = 0; first < splits; first += 8) {
-      float part[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) part[i] = partial_acc[((size_t)min(first + i, splits - 1) * columns_total + column) * D + d];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float w = __shfl(weight, min(first + i, MERGE_SPLITS_MAX - 1), 64);
-        if (first + i < splits && w != 0.f) sum += part[i] * w;
-      }
-    }
-    out[column * D + d] = sum * inverse;
-  }
+  const float* acc = partial_acc + column * D + min(d, D - 1);
+  const size_t split_stride = (size_t)columns_total * D;
+  float sum = 0.f;
+  int first = 0;
+  for (; splits - first > 8; first += 32) sum += merge_some<32>(acc, split_stride, first, splits, weight);
+  if (first < splits) sum += merge_some<8>(acc, split_stride, first, splits, weight);
+  if (d < D) out[column * D + d] = sum * inverse;
 }
 
 // qkv [tokens, row_width] float32 with the queries in front (heads * D), out [tokens, heads * D]; key pages in
@@ -318,7 +328,7 @@ extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* ou
 #undef LAUNCH_ATTENTION_F32
   int status = LAUNCH_STATUS();
   if (status != 0 || splits == 1) return status;
-  hipLaunchKernelGGL(attention_f32_merge_kernel, dim3(columns_total), dim3(64), 0, stream, out, partial_acc, partial_ml,
+  hipLaunchKernelGGL(attention_f32_merge_kernel, dim3(columns_total), dim3(MERGE_THREADS), 0, stream, out, partial_acc, partial_ml,
                      splits, columns_total);
   return LAUNCH_STATUS();
 }
