@@ -647,30 +647,34 @@ __device__ __forceinline__ float merge_some(const float* acc, int first, int spl
   return sum;
 }
 
-// sum_s acc_s[d] w_s / sum_s l_s w_s of the splits whose maxima and sums lie at `ml` and partial sums at `acc`;
-// every lane of every wave must call it (the weights pass between lanes)
-__device__ __forceinline__ float merged_dimension(const float* ml, const float* acc, int splits, int d) {
+// out[d] = sum_s acc_s[d] w_s / sum_s l_s w_s of the splits whose maxima and sums lie at `ml` and partial sums at
+// `acc`, for the dimensions threadIdx.x, threadIdx.x + blockDim.x, ...; every lane of every wave must call it (the
+// weights pass between lanes)
+__device__ __forceinline__ void merge_splits(const float* ml, const float* acc, int splits, bf16_t* out) {
   const int lane = threadIdx.x & (WAVE - 1);
   const float2 mine = lane < splits ? *(const float2*)(ml + (size_t)lane * 2) : make_float2(-INFINITY, 0.f);
   const float best = wave_max(mine.x);
   const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
   const float total = wave_sum(mine.y * weight);                          // (lanes beyond the splits add 0)
   const float inverse = total > 0.f ? 1.f / total : 0.f;
-  const float* mine_acc = acc + min(d, D - 1);
-  float sum = 0.f;
-  int first = 0;
-  for (; splits - first > 8; first += 32) sum += merge_some<32>(mine_acc, first, splits, weight);
-  if (first < splits) sum += merge_some<8>(mine_acc, first, splits, weight);
-  return sum * inverse;
+  for (int d0 = 0; d0 < D; d0 += blockDim.x) {  // (the same trips for all lanes: those beyond D read D - 1 and store nothing)
+    const int d = d0 + threadIdx.x;
+    const float* mine_acc = acc + min(d, D - 1);
+    float sum = 0.f;
+    int first = 0;
+    for (; splits - first > 8; first += 32) sum += merge_some<32>(mine_acc, first, splits, weight);
+    if (first < splits) sum += merge_some<8>(mine_acc, first, splits, weight);
+    if (d < D) out[d] = (bf16_t)(sum * inverse);
+  }
 }
 
+// (a workgroup of one thread a dimension where the (token, head) pairs are few and the trips count, of one wave where
+// they are many: a prompt portion's 24,576 pairs in four splits 12 us against 15)
 __global__ __launch_bounds__(MERGE_THREADS) void attention_merge_kernel(const float* __restrict__ partial_acc,
                                                                         const float* __restrict__ partial_ml,
                                                                         bf16_t* __restrict__ out, int splits) {
   const size_t pair = blockIdx.x;  // row * heads + head
-  const int d = threadIdx.x;
-  const float merged = merged_dimension(partial_ml + pair * splits * 2, partial_acc + pair * splits * D, splits, d);
-  if (d < D) out[pair * D + d] = (bf16_t)merged;
+  merge_splits(partial_ml + pair * splits * 2, partial_acc + pair * splits * D, splits, out + pair * D);
 }
 
 // The same for partial results that are kept by work item: workgroup (item, head) merges the item's tokens one
@@ -682,18 +686,17 @@ __global__ __launch_bounds__(MERGE_THREADS) void attention_merge_items_kernel(co
                                                                               int heads, int group, int tokens_per_tile) {
   const int* item = work + (size_t)blockIdx.x * 4;
   const int tokens = group <= 16 ? (item[2] + item[3] + group - 1) / group : item[3];
-  const int head = blockIdx.y, d = threadIdx.x;
+  const int head = blockIdx.y;
   for (int token = 0; token < tokens; ++token) {
     const size_t kept_as = ((size_t)blockIdx.x * tokens_per_tile + token) * heads + head;
     const size_t pair = ((size_t)item[1] + token) * heads + head;
-    const float merged = merged_dimension(partial_ml + kept_as * splits * 2, partial_acc + kept_as * splits * D, splits, d);
-    if (d < D) out[pair * D + d] = (bf16_t)merged;
+    merge_splits(partial_ml + kept_as * splits * 2, partial_acc + kept_as * splits * D, splits, out + pair * D);
   }
 }
 
 static int launch_merge(float* partial_acc, float* partial_ml, void* out, int splits, size_t pairs, hipStream_t stream) {
-  hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)pairs), dim3(MERGE_THREADS), 0, stream, partial_acc,
-                     partial_ml, (bf16_t*)out, splits);
+  hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)pairs), dim3(pairs >= 4096 ? WAVE : MERGE_THREADS), 0, stream,
+                     partial_acc, partial_ml, (bf16_t*)out, splits);
   return LAUNCH_STATUS();
 }
 
