@@ -938,6 +938,13 @@ class HipKernels:
                         splits = next(allowed for allowed in (1, 2, 3, 4, 6, 8) if allowed >= wanted)
                     else:
                         unmerged = False
+                if not unmerged and 24 <= blocks <= 48:
+                    # Some tens of workgroups over a short context: since the kernel that merges asks for all splits at
+                    # once, runs of a few steps pay where the chip has room (us a layer at 32 workgroups, unsplit
+                    # against six runs: 640 keys 11.4 / 9.9, 1,024 keys 15.7 / 11.5; a whole step at the 7B sizes
+                    # 3.33 -> 3.28 ms). At 64 workgroups three runs tie (12.5 / 12.3, the 32B step alike); at 16 they
+                    # lose (8.7 / 8.9).
+                    splits = max(splits, min(-(-steps // 4), 192 // blocks))
                 if not unmerged and blocks <= 8 and steps >= 128:
                     # very few requests over a long context: runs of 16 steps, two a wave (one request over 8,192
                     # keys 12.6 -> 11.5 us a layer, four 15.1 -> 13.4)
