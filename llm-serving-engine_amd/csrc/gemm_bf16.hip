@@ -1509,19 +1509,6 @@ static int launch_wide(const void* x, const void* w, const void* bias, int bias_
   return LAUNCH_STATUS();
 }
 
-// As llmserve_gemm_tiled, with K (and K / splits) a multiple of 32.
-extern "C" int llmserve_gemm_wide(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
-                                  int out_is_float, int gated, int M, int N, int K, int splits, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || K % WIDE_K || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
-  if (splits > 1 && (gated || !out_is_float || K % splits || (K / splits) % WIDE_K)) return ERR_BAD_ARGUMENT;
-  if (gated)
-    return out_is_float ? launch_wide<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
-                        : launch_wide<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
-  return out_is_float ? launch_wide<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream)
-                      : launch_wide<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
-}
-
 template <typename TO, bool GATED>
 static int pick_tiled(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
                       int splits, hipStream_t stream) {

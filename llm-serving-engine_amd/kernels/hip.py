@@ -62,7 +62,6 @@ _SIGNATURES = {
     "llmserve_gemm_ring": "pppipiiiiiiip",
     "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
-    "llmserve_gemm_wide": "pppipiiiiiip",
     "llmserve_attention_generic": "pipipppippiiiiifipfp",
     "llmserve_attention_f32": "pippppppippiiiiiifiipfp",
     "llmserve_attention_tiles": "pippppppippiiiiiifiiipippfp",
