@@ -400,10 +400,18 @@ class ModelRunner:
             size *= 2
         return size
 
+    @classmethod
+    def _request_bucket(cls, requests: int) -> int:
+        """The rows of the graph that a step of so many single tokens replays: a power of two up to 128, where the
+        kernels' cost goes by tiles of 16 to 128 rows and padding costs little (65 requests of the 1.5B sizes 2.37 ms a
+        step, 128 requests 2.55), and multiples of 64 beyond, where every product is the library's and goes by its rows
+        (192 requests padded to 256 rows took the 3.80 ms of 256)."""
+        return cls._bucket(requests) if requests <= 128 else -(-requests // 64) * 64
+
     def _pack_decode(self, reservations: list[Reservation], entries: list[StepEntry]):
         """The index arrays of a step of single tokens, padded to its graph's shape; first the graph's key."""
         started = time.perf_counter()
-        requests = self._bucket(len(reservations))
+        requests = self._request_bucket(len(reservations))
         blocks = max(-(-(r.start + 1) // self.cache.page_size) for r in reservations)
         width = min(self._bucket(blocks), self._bucket(self.cache.max_blocks_per_sequence))
         packed = _pack_step(reservations, entries, self.cache, pad_to=requests, width=width)

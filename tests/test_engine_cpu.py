@@ -530,3 +530,14 @@ def test_the_sampler_says_whether_a_row_has_top_p():
         assert kernels.said is expected
         want = [plain.sample(logits[row], c.temperature, c.top_p, plain.uniform_for(c.seed, row)) for row, c in enumerate(configs)]
         assert tokens == want
+
+
+def test_the_rows_of_a_decode_graph_by_the_number_of_requests():
+    """A step of single tokens replays the graph of its padded shape: a power of two up to 128 requests,
+    a multiple of 64 beyond, never fewer rows than requests and never more than twice as many."""
+    rows = [ModelRunner._request_bucket(requests) for requests in range(1, 1025)]
+    assert rows[:5] == [1, 2, 4, 4, 8] and rows[127] == 128 and rows[128] == 192 and rows[192] == 256
+    assert all(later >= earlier for earlier, later in zip(rows, rows[1:]))
+    for requests, padded in enumerate(rows, start=1):
+        assert requests <= padded < 2 * requests or requests == 1
+        assert padded & (padded - 1) == 0 if requests <= 128 else padded % 64 == 0
