@@ -166,12 +166,14 @@ def test_replay_at_benchmark_layer_sizes(wide_models, tmp_path, sizes, dtype, ow
     assert total / count < (walk if dtype == "float32" else BF16_MEAN * spread)
 
 
-@pytest.mark.parametrize("sizes,requests", [("1.5B", 20), ("1.5B", 40), ("7B", 20), ("7B", 40), ("32B", 20), ("32B", 8)])
+@pytest.mark.parametrize("sizes,requests", [("1.5B", 20), ("1.5B", 40), ("7B", 20), ("7B", 40), ("32B", 20), ("32B", 8),
+                                            ("1.5B", 100), ("7B", 70), ("1.5B", 150)])
 def test_captured_steps_of_many_rows_at_benchmark_layer_sizes(wide_models, sizes, requests):
-    """Decode steps of 17 to 64 rows are replayed from a graph in which the products go other ways than
-    in every other step (the BLAS library for the wide ones, the weight-streaming kernel for small
-    weights at up to 32 rows).
-    Twenty and forty requests decode side by side through the step function; every step's logits are
+    """Decode steps of 17 rows and more are replayed from a graph in which the products go other ways than
+    in every other step (up to 64 rows the kernel that streams a weight through a ring in LDS, the BLAS
+    library or the weight-streaming kernel for small weights; 65 to 128 rows the ring kernel with eight tiles
+    of x; beyond that the library, in a graph of a multiple of 64 rows).
+    So many requests decode side by side through the step function; every step's logits are
     compared with the plain forward over each request's whole sequence."""
     from llmserve_amd import CacheConfig, ModelRunner, StepEntry
     from llmserve_amd.kernels import HipKernels
