@@ -131,3 +131,38 @@ def test_routes_at_random_sizes():
             assert in_features % 32 == 0
         else:
             assert way is None
+
+
+def test_attention_work_lists_cover_every_column_once_and_fit_the_padded_shape():
+    """The attention kernels take their work from a list of (request, first token, first head of it, columns)
+    items made on the host; a captured step's list has room for the most items its padded shape can hold.
+    Steps drawn at random: the items cover every (token, head) column of the chosen chunks exactly once, no
+    item is longer than the kernel's tile, and no step of a shape has more items than the shape's room."""
+    from llmserve_amd.engine.batch import SequenceChunk
+
+    draw = random.Random(9)
+    for _ in range(3000):
+        group = draw.choice([1, 2, 5, 6, 7, 8, 16, 17, 28])
+        column_tiles = draw.choice([1, 2])
+        packed = draw.choice([None, True, False])
+        requests = draw.randint(1, 12)
+        counts = [draw.choice([1, 1, 1, 2, 3, 16, 17, draw.randint(1, 700)]) for _ in range(requests)]
+        chunks = [SequenceChunk(f"r{i}", i, draw.randint(0, 5000), count) for i, count in enumerate(counts)]
+        longer_than, up_to = draw.choice([(0, None), (0, 16), (16, None), (1, None), (0, 1)])
+        work, steps = HipKernels._work_items(chunks, group, column_tiles, longer_than, up_to, packed)
+        is_packed = group <= 16 if packed is None else packed
+        per_token = group if is_packed else 1
+        per_item = column_tiles * (16 if is_packed else 1)
+        chosen = [i for i, count in enumerate(counts) if count > longer_than and (up_to is None or count <= up_to)]
+        starts = [sum(counts[:i]) for i in range(requests)]
+        seen = set()
+        for request, token, head, columns in work.tolist():
+            assert request in chosen and 0 < columns <= per_item and 0 <= head < per_token
+            for column in range(columns):
+                at = (token - starts[request]) * per_token + head + column
+                assert 0 <= at < counts[request] * per_token and (request, at) not in seen
+                seen.add((request, at))
+        assert len(seen) == sum(counts[i] * per_token for i in chosen)
+        assert steps >= 0
+        padded_tokens = sum(counts) + draw.randint(0, 64)
+        assert len(work) <= HipKernels._work_capacity((padded_tokens, requests + draw.randint(0, 3)), group, column_tiles, packed)
